@@ -1,0 +1,156 @@
+/*
+ * winoconv.h - C ABI of libwinoconv_hip.so, a Winograd / DWM convolution engine
+ * for AMD gfx950 (MI355X).
+ *
+ * Plain pointers, ints and sizes only: no torch, no HIP types (a stream is passed
+ * as `void*` holding a hipStream_t; NULL is the default stream).  Every function
+ * returns 0 on success or a negative wc_status; wc_last_error() then gives a
+ * thread-local message.  No function allocates device memory, synchronises the
+ * device or keeps state between calls: work is enqueued on the caller's stream
+ * and scratch memory comes from the caller (`workspace`).
+ *
+ * Data layouts (row-major, innermost last).  "Channel-last" means NHWC / NDHWC.
+ *   x   (N, D, H, W, C)        D = 1 for 2-D problems
+ *   w   any strided (K, C, kD, kH, kW) view: element strides are passed in
+ *   y   (N, oD, oH, oW, K)
+ *   U   (T, K,  Cp)            transformed filter, Cp = wc_padded_channels(C)
+ *   V   (T, P,  Cp)            transformed input,  P = N*nD*nH*nW tiles
+ *   M   (T, P,  ldm)           per-element products, ldm = wc_padded_channels8(K)
+ * T is the number of transform-domain elements summed over all pieces of the
+ * DWM plan; element order inside a piece is (d*alpha_h + h)*alpha_w + w.
+ *
+ * Each declaration cites the interface of the reference implementation
+ * (huangdi95/pytorch_winoconv) that it stands in for.
+ */
+#ifndef WINOCONV_H_
+#define WINOCONV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { WC_F32 = 0, WC_F16 = 1 } wc_dtype;
+
+typedef enum {
+  WC_OK = 0,
+  WC_ERR_BAD_ARG = -1,      /* null pointer, non-positive size, inconsistent shapes   */
+  WC_ERR_UNSUPPORTED = -2,  /* kernel size / stride / tile size outside the engine     */
+  WC_ERR_WORKSPACE = -3,    /* workspace missing or too small                          */
+  WC_ERR_HIP = -4           /* a HIP runtime call failed (message carries its text)    */
+} wc_status;
+
+#define WC_MAX_PIECES 64
+
+/* One stride-1 sub-convolution of the DWM plan. */
+typedef struct {
+  int tap0[3];   /* first kernel tap per axis (D, H, W)                      */
+  int r[3];      /* taps per axis, 1..3; taps are tap0 + i*tap_step          */
+  int t_offset;  /* first transform-domain element of this piece             */
+} wc_piece;
+
+typedef struct {
+  int n_pieces;
+  int t_total;                 /* sum over pieces of prod(m + r - 1)                  */
+  int tap_step;                /* = convolution stride                                */
+  int m[3];                    /* output tile extent per axis (1 on a size-1 depth)   */
+  wc_piece piece[WC_MAX_PIECES];
+} wc_plan;
+
+typedef struct {
+  int ndim;        /* 2 or 3                                                   */
+  int N, C, K;
+  int in[3];       /* D, H, W of the input (D = 1 when ndim == 2)               */
+  int kernel[3];   /* kD, kH, kW (kD = 1 when ndim == 2)                        */
+  int pad[3];      /* symmetric zero padding per axis                           */
+  int stride;      /* 1 or 2, same on every axis                                */
+  int m;           /* Winograd output tile: 2, or 4 (2-D 3x3 stride 1 only)     */
+  int dtype;       /* wc_dtype                                                  */
+  int chunk_images;/* images per pass of wc_conv_forward; 0 = choose automatically */
+} wc_conv_desc;
+
+/* ---- library ------------------------------------------------------------------------- */
+const char* wc_version(void);
+/* Replaces the reference's cout + exit(-1) error convention
+ * (src/winograd_conv.cpp:80-84,116-126; src/base_conv_launchers.h:384-387). */
+const char* wc_last_error(void);
+
+/* ---- planning (host only) --------------------------------------------------------------- */
+/* Stride-1 split plan in the reference's own terms; replaces splitControl()
+ * (src/base_conv_launchers.h:58-388) and the kernel_stride prefix sums
+ * (src/base_conv_launchers.cu:307-313).  Arrays must hold WC_MAX_PIECES ints.
+ * Boxes are half-open [start, end).  Works for every extent 1..10, not just the
+ * reference's 36 keys. */
+int wc_plan_dwm(int kD, int kH, int kW, int* num_split,
+                int* D_start, int* D_end, int* H_start, int* H_end,
+                int* W_start, int* W_end, int* kernel_stride, int* t_total);
+/* General plan of a convolution (stride 1 or 2, tile 2 or 4). */
+int wc_plan_conv(const wc_conv_desc* desc, wc_plan* plan);
+/* Output extent and tile grid: replaces the shape arithmetic of DWM<T>
+ * (src/winograd_conv.cpp:71-90) and of dwm2d_/dwm3d_ (dwm.py:56-61,118-121). */
+int wc_conv_out_dims(const wc_conv_desc* desc, int out[3], int grid[3]);
+int wc_padded_channels(int C);   /* channel stride of U and V (multiple of 32) */
+int wc_padded_channels8(int K);  /* row stride of M (multiple of 8)             */
+
+/* ---- tile split / concat (bit-exact copies) ----------------------------------------------- */
+/* Replaces WinoSplit<T> (pybind/extern.hpp:3-4, src/split_and_concat.cpp:14-40) and the
+ * kernels winoSplitKernel2d / winoSplitKernel (src/split_and_concat_kernels.cu:76-101, :8-37).
+ * x channel-last (B, [D,] H, W, C) -> tiles (B*[nD*]nH*nW, C, [block_D,] block_H, block_W),
+ * tile step = m on every axis, zero outside the input.  elem_size is 2 or 4 bytes. */
+int wc_wino_split2d(const void* x, void* tiles, int B, int H, int W, int C,
+                    int block_H, int block_W, int m, int nH, int nW,
+                    int elem_size, void* stream);
+int wc_wino_split3d(const void* x, void* tiles, int B, int D, int H, int W, int C,
+                    int block_D, int block_H, int block_W, int m, int nD, int nH, int nW,
+                    int elem_size, void* stream);
+/* Replaces WinoConcat<T> (pybind/extern.hpp:5-6, src/split_and_concat.cpp:44-76) and the
+ * kernels winoConcatKernel2d / winoConcatKernel (src/split_and_concat_kernels.cu:107-129, :43-70).
+ * tiles (B*[nD*]nH*nW, K, [m,] m, m) -> y channel-last (B, [oD,] oH, oW, K); partial edge
+ * tiles are cropped.  n_X = ceil(o_X / m). */
+int wc_wino_concat2d(const void* tiles, void* y, int B, int oH, int oW, int K, int m,
+                     int elem_size, void* stream);
+int wc_wino_concat3d(const void* tiles, void* y, int B, int oD, int oH, int oW, int K, int m,
+                     int elem_size, void* stream);
+
+/* ---- pipeline stages ---------------------------------------------------------------------- */
+/* U = (G x G x G) g for every piece.  Replaces wNorm2WinoTransform + wNorm2WinoCalculation
+ * (src/split_kernel.cu:14-53, src/calculation_kernels.cu:2-761) and matrix_conv.py:150-153.
+ * w_strides: element strides of w for (K, C, kD, kH, kW). */
+int wc_filter_transform(const wc_conv_desc* desc, const wc_plan* plan,
+                        const void* w, const int64_t w_strides[5], void* U, void* stream);
+/* V = (BT x BT x BT) d for `n_images` images starting at x.  Replaces
+ * inputNorm2WinoTransform + inputNorm2WinoCalculation (src/split_kernel.cu:60-120,
+ * src/calculation_kernels.cu:763-1522) and matrix_conv.py:158-203. */
+int wc_input_transform(const wc_conv_desc* desc, const wc_plan* plan,
+                       const void* x, int n_images, void* V, void* stream);
+/* M[t] (P x K) = V[t] (P x Cp) . U[t]^T for t in [0, T).  Replaces forwardAssign +
+ * cublas{S,H}gemmBatched (src/utils.cu:5-12, src/base_conv_launchers.cu:353-367,
+ * src/base_conv_launchers_half.cu:231-236).  fp16 accumulates in fp32. */
+int wc_batched_gemm(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm,
+                    int dtype, void* stream);
+/* y = sum over pieces of (AT x AT x AT) m, + bias, cropped.  Replaces outputWino2NormTransform +
+ * outputWino2NormCalculation + outputAggregate (src/split_kernel.cu:126-203,
+ * src/calculation_kernels.cu:1524-1770) and matrix_conv.py:207-253.  bias may be NULL
+ * (K values of the tensor dtype otherwise). */
+int wc_output_transform(const wc_conv_desc* desc, const wc_plan* plan,
+                        const void* M, const void* bias, int n_images, void* y, void* stream);
+
+/* ---- whole convolution -------------------------------------------------------------------- */
+/* Replaces DWM<T> (pybind/extern.hpp:7-9, src/winograd_conv.cpp:17-127) and
+ * convLauncherStrideOneLarge<T> (src/base_conv_launchers.cu:282-399).
+ * The workspace holds U, V and M (the reference's tmp_weight_buffer, tmp_input_buffer,
+ * tmp_product_buffer: dwm.py:122-125); images are processed in chunks so that V and M of
+ * one chunk stay cache resident.  `U_cached` (may be NULL) is a filter already transformed
+ * by wc_filter_transform; `w` may then be NULL. */
+int wc_conv_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
+int wc_conv_u_elems(const wc_conv_desc* desc, size_t* elems);
+int wc_conv_forward(const wc_conv_desc* desc, const void* x,
+                    const void* w, const int64_t w_strides[5], const void* U_cached,
+                    const void* bias, void* y, void* workspace, size_t workspace_bytes,
+                    void* stream);
+#ifdef __cplusplus
+}
+#endif
+#endif /* WINOCONV_H_ */

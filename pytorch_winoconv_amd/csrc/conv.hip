@@ -1,0 +1,123 @@
+// Whole convolution: filter transform -> per image chunk (input transform -> batched GEMM ->
+// output transform).  Replaces DWM<T> (src/winograd_conv.cpp:17-127) and
+// convLauncherStrideOneLarge<T> (src/base_conv_launchers.cu:282-399) of the reference, minus
+// its per-call cudaMalloc/cudaMemcpy/cudaFree of the split tables and of tmp_output
+// (base_conv_launchers.cu:323-336, :375-376, :384-391) and its per-call cuBLAS handle
+// (:360-361, :383): the plan travels in kernel arguments, scratch comes from the caller and
+// everything is enqueued on the caller's stream.
+//
+// The batch is processed in chunks of images so that V and M of one chunk (the two large
+// intermediates, written once and read once) can stay resident in the last-level cache
+// between the kernel that writes them and the kernel that reads them.
+#include "wc_common.h"
+
+using namespace wc;
+
+namespace {
+
+struct Layout {
+  wc_plan plan;
+  int out[3], grid[3];
+  int Cp, ldm, chunk;
+  long long tiles_per_image;
+  size_t es;
+  size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
+};
+
+size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+int make_layout(const wc_conv_desc* d, Layout* L) {
+  int rc = wc_plan_conv(d, &L->plan);
+  if (rc) return rc;
+  rc = wc_conv_out_dims(d, L->out, L->grid);
+  if (rc) return rc;
+  L->Cp = wc_padded_channels(d->C);
+  L->ldm = wc_padded_channels8(d->K);
+  L->es = d->dtype == WC_F16 ? 2 : 4;
+  L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
+  const long long T = L->plan.t_total;
+  int chunk = d->chunk_images;
+  if (chunk <= 0) {
+    // V + M of one chunk around 64 MB, but never so small that the GEMM cannot fill the GPU
+    const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es;
+    chunk = (int)(64.0 * 1024 * 1024 / per_image);
+    const long long min_tiles = 8192;   // tile rows per chunk for >= 2 workgroups per CU at T >= 16
+    const int need = (int)((min_tiles + L->tiles_per_image - 1) / L->tiles_per_image);
+    if (chunk < need) chunk = need;
+    if (chunk < 1) chunk = 1;
+  }
+  if (chunk > d->N) chunk = d->N;
+  L->chunk = chunk;
+  const long long Pc = L->tiles_per_image * chunk;
+  if (T * Pc * (long long)(L->Cp > L->ldm ? L->Cp : L->ldm) >= (1ll << 40))
+    return fail(WC_ERR_UNSUPPORTED, "chunk of %d images is too large", chunk);
+  L->u_bytes = round256((size_t)T * d->K * L->Cp * L->es);
+  L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
+  L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
+  return WC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wc_conv_workspace_bytes(const wc_conv_desc* d, size_t* bytes) {
+  WC_CHECK_ARG(bytes != nullptr, "wc_conv_workspace_bytes: null output");
+  Layout L;
+  int rc = make_layout(d, &L);
+  if (rc) return rc;
+  *bytes = L.u_bytes + L.v_bytes + L.m_bytes;
+  return WC_OK;
+}
+
+int wc_conv_u_elems(const wc_conv_desc* d, size_t* elems) {
+  WC_CHECK_ARG(elems != nullptr, "wc_conv_u_elems: null output");
+  Layout L;
+  int rc = make_layout(d, &L);
+  if (rc) return rc;
+  *elems = (size_t)L.plan.t_total * d->K * L.Cp;
+  return WC_OK;
+}
+
+int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
+                    const void* U_cached, const void* bias, void* y, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  Layout L;
+  int rc = make_layout(d, &L);
+  if (rc) return rc;
+  WC_CHECK_ARG(x && y, "wc_conv_forward: null input or output");
+  WC_CHECK_ARG(U_cached || (w && w_strides), "wc_conv_forward: neither a filter nor a transformed filter");
+  if (!workspace) return fail(WC_ERR_WORKSPACE, "wc_conv_forward: null workspace");
+  const size_t need = L.u_bytes + L.v_bytes + L.m_bytes;
+  if (workspace_bytes < need)
+    return fail(WC_ERR_WORKSPACE, "wc_conv_forward: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
+    return fail(WC_ERR_WORKSPACE, "wc_conv_forward: workspace must be 256-byte aligned");
+
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  void* Uws = ws;
+  void* V = ws + L.u_bytes;
+  void* M = ws + L.u_bytes + L.v_bytes;
+  const void* U = U_cached;
+  if (!U) {
+    rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
+    if (rc) return rc;
+    U = Uws;
+  }
+  const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L.es;
+  const size_t y_image = (size_t)L.out[0] * L.out[1] * L.out[2] * d->K * L.es;
+  for (int b0 = 0; b0 < d->N; b0 += L.chunk) {
+    const int n = (d->N - b0 < L.chunk) ? d->N - b0 : L.chunk;
+    const long long P = L.tiles_per_image * n;
+    WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
+    rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);
+    if (rc) return rc;
+    rc = wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+    if (rc) return rc;
+    rc = wc_output_transform(d, &L.plan, M, bias, n, static_cast<unsigned char*>(y) + b0 * y_image, stream);
+    if (rc) return rc;
+  }
+  return WC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,257 @@
+// Batched GEMM of the Winograd domain: M[t] (P x K) = V[t] (P x Cp) . U[t]^T, t in [0, T).
+//
+// Replaces forwardAssign + cublas{S,H}gemmBatched of the reference (src/utils.cu:5-12,
+// src/base_conv_launchers.cu:353-367, src/base_conv_launchers_half.cu:231-236): batches are
+// addressed by stride, so no pointer arrays.  Both operands keep the reduction axis C
+// innermost, which is the layout MFMA wants for both: a lane feeds 8 consecutive halves
+// (one 16-byte LDS read) per operand per v_mfma_f32_32x32x16_f16.
+//
+// Workgroup = 4 wavefronts (2 x 2), each owning WM x WN MFMA blocks of 32 x 32, so the
+// macro tile is (64 WM) tiles x (64 WN) output channels.  Operand tiles go global -> registers ->
+// LDS with two LDS stages (one barrier per reduction step; the global loads of step k+1 are in
+// flight while step k is multiplied).  LDS rows are padded by 16 bytes, which makes the 16-byte
+// fragment reads of 8 consecutive rows hit 32 distinct banks.  The MFMA "A" operand is the
+// filter block and "B" the input block: a lane then holds 4 consecutive output channels of
+// one tile row per accumulator group and stores them as one 8-byte (fp16) / 16-byte (fp32)
+// write.  fp16 accumulates in fp32; fp32 uses v_mfma_f32_32x32x2_f32.
+#include "wc_common.h"
+#include <cstdlib>
+
+namespace wc {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <typename T> struct Mfma;
+template <> struct Mfma<half_t> {
+  using Frag = half8;
+  static constexpr int kpack = 8;    // consecutive reduction elements a lane supplies
+  static constexpr int kstep = 16;   // reduction elements per instruction
+  __device__ static __forceinline__ floatx16 run(Frag a, Frag b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<float> {
+  using Frag = float;
+  static constexpr int kpack = 1;
+  static constexpr int kstep = 2;
+  __device__ static __forceinline__ floatx16 run(Frag a, Frag b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+
+struct GemmArgs {
+  const void* V;
+  const void* U;
+  void* M;
+  int P, K, Cp, ldm;
+  long long sV, sU, sM;     // batch strides in elements
+  int tiles_p, tiles_k, T;
+  int n_blocks, per_xcd;
+};
+
+typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
+
+template <typename T, int WM, int WN, int BK>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g) {
+  using MF = Mfma<T>;
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int EPC = 16 / sizeof(T);              // elements per 16-byte chunk
+  constexpr int CPR = BK / EPC;                    // chunks per tile row
+  constexpr int LDS_STRIDE = BK + EPC;             // padded row, elements
+  constexpr int ROWS = BM + BN;
+  constexpr int RPP = 256 / CPR;                   // rows covered by one pass of the workgroup
+  constexpr int NLOAD = ROWS / RPP;
+  constexpr int STAGE = ROWS * LDS_STRIDE;         // elements per LDS stage
+  static_assert(ROWS % RPP == 0 && BM % RPP == 0, "tile rows must be a multiple of the load pass");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  const int blk = xcd_remap(blockIdx.x, g.per_xcd);
+  if (blk >= g.n_blocks) return;
+  const int kt_ = blk % g.tiles_k;
+  const int pt = (blk / g.tiles_k) % g.tiles_p;
+  const int t = blk / (g.tiles_k * g.tiles_p);
+  const int p0 = pt * BM, k0 = kt_ * BN;
+
+  const T* Vt = static_cast<const T*>(g.V) + (long long)t * g.sV;
+  const T* Ut = static_cast<const T*>(g.U) + (long long)t * g.sU;
+
+  const int tid = threadIdx.x;
+  const int lrow = tid / CPR, lpart = tid % CPR;
+  const T* gptr[NLOAD];
+  int loff[NLOAD];
+#pragma unroll
+  for (int i = 0; i < NLOAD; ++i) {
+    const int row = lrow + i * RPP;                // row of the stacked [X ; W] tile
+    if (row < BM) {
+      const int p = min(p0 + row, g.P - 1);
+      gptr[i] = Vt + (long long)p * g.Cp + lpart * EPC;
+    } else {
+      const int k = min(k0 + row - BM, g.K - 1);
+      gptr[i] = Ut + (long long)k * g.Cp + lpart * EPC;
+    }
+    loff[i] = row * LDS_STRIDE + lpart * EPC;
+  }
+
+  Chunk16 regs[NLOAD];
+  auto gload = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) regs[i] = *reinterpret_cast<const Chunk16*>(gptr[i] + kt * BK);
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) *reinterpret_cast<Chunk16*>(lds + buf * STAGE + loff[i]) = regs[i];
+  };
+
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave >> 1, wk = wave & 1;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  // fragment read offsets inside a stage (elements)
+  const int xoff = (wp * WM * 32 + l32) * LDS_STRIDE + lhi * MF::kpack;
+  const int woff = (BM + wk * WN * 32 + l32) * LDS_STRIDE + lhi * MF::kpack;
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nk = g.Cp / BK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) gload(kt + 1);
+    const T* st = lds + cur * STAGE;
+#pragma unroll
+    for (int kk = 0; kk < BK / MF::kstep; ++kk) {
+      typename MF::Frag xf[WM], wf[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        xf[i] = *reinterpret_cast<const typename MF::Frag*>(st + xoff + i * 32 * LDS_STRIDE + kk * MF::kstep);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        wf[j] = *reinterpret_cast<const typename MF::Frag*>(st + woff + j * 32 * LDS_STRIDE + kk * MF::kstep);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[j], xf[i], acc[i][j]);
+    }
+    if (kt + 1 < nk) lstore(cur ^ 1);
+    __syncthreads();
+  }
+
+  // accumulator (i, j), register 4g + e: output channel 32j + 8g + 4*lhi + e of tile row 32i + l32
+  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int p = p0 + wp * WM * 32 + i * 32 + l32;
+    if (p >= g.P) continue;
+    T* row = Mt + (long long)p * g.ldm;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int kc = k0 + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi;
+        if (kc < g.ldm) {
+          Pack<T, 4> o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
+          *reinterpret_cast<Pack<T, 4>*>(row + kc) = o;
+        }
+      }
+    }
+  }
+}
+
+using GemmKernel = void (*)(GemmArgs);
+
+struct GemmConfig {
+  GemmKernel fn;
+  int bm, bn, bk;
+  size_t lds;
+};
+
+template <typename T, int WM, int WN, int BK>
+static GemmConfig make_config() {
+  constexpr int EPC = 16 / sizeof(T);
+  return GemmConfig{&gemm_kernel<T, WM, WN, BK>, 64 * WM, 64 * WN, BK,
+                    (size_t)2 * (64 * WM + 64 * WN) * (BK + EPC) * sizeof(T)};
+}
+
+// Tile shapes, largest first.  All keep LDS at or below 64 KB.
+template <typename T> struct Configs;
+template <> struct Configs<half_t> {
+  static constexpr int n = 5;
+  static GemmConfig get(int i) {
+    switch (i) {
+      case 0: return make_config<half_t, 4, 2, 32>();   // 256 x 128
+      case 1: return make_config<half_t, 2, 2, 32>();   // 128 x 128
+      case 2: return make_config<half_t, 4, 1, 32>();   // 256 x 64
+      case 3: return make_config<half_t, 2, 1, 32>();   // 128 x 64
+      default: return make_config<half_t, 1, 1, 32>();  // 64 x 64
+    }
+  }
+};
+template <> struct Configs<float> {
+  static constexpr int n = 5;
+  static GemmConfig get(int i) {
+    switch (i) {
+      case 0: return make_config<float, 4, 2, 16>();
+      case 1: return make_config<float, 2, 2, 16>();
+      case 2: return make_config<float, 4, 1, 16>();
+      case 3: return make_config<float, 2, 1, 16>();
+      default: return make_config<float, 1, 1, 16>();
+    }
+  }
+};
+
+// Picks the largest tile that still gives the 256 CUs about two workgroups each and does not
+// waste more than half a tile on the channel axis.
+template <typename T>
+static GemmConfig choose(int T_, int P, int K) {
+  const char* force = std::getenv("WINOCONV_GEMM_CONFIG");
+  if (force) {
+    const int i = std::atoi(force);
+    if (i >= 0 && i < Configs<T>::n) return Configs<T>::get(i);
+  }
+  GemmConfig best = Configs<T>::get(Configs<T>::n - 1);
+  for (int i = 0; i < Configs<T>::n; ++i) {
+    GemmConfig c = Configs<T>::get(i);
+    if (c.bn > 64 && c.bn / 2 >= K) continue;                 // half of the tile would be padding
+    const long long blocks = (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_;
+    if (blocks >= 512 || i == Configs<T>::n - 1) { best = c; break; }
+  }
+  return best;
+}
+
+}  // namespace wc
+
+using namespace wc;
+
+extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, int P, int Cp, int K,
+                               int ldm, int dtype, void* stream) {
+  WC_CHECK_ARG(V && U && M, "wc_batched_gemm: null pointer");
+  WC_CHECK_ARG(T_ > 0 && P > 0 && K > 0, "wc_batched_gemm: T %d, P %d, K %d", T_, P, K);
+  WC_CHECK_ARG(Cp > 0 && Cp % 32 == 0, "wc_batched_gemm: reduction extent %d is not a multiple of 32", Cp);
+  WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "wc_batched_gemm: row stride %d (needs >= K, multiple of 8)", ldm);
+  WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32, "wc_batched_gemm: dtype %d", dtype);
+  GemmConfig c = dtype == WC_F16 ? choose<half_t>(T_, P, K) : choose<float>(T_, P, K);
+  GemmArgs g;
+  g.V = V; g.U = U; g.M = M;
+  g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;
+  g.sV = (long long)P * Cp; g.sU = (long long)K * Cp; g.sM = (long long)P * ldm;
+  g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
+  const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
+  WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");
+  g.n_blocks = (int)blocks;
+  g.per_xcd = ceil_div((int)blocks, kXcds);
+  hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(256), c.lds, as_stream(stream), g);
+  WC_CHECK_LAUNCH("gemm_kernel");
+  return WC_OK;
+}

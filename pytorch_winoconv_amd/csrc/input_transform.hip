@@ -1,0 +1,52 @@
+// Host entry of the input transform: picks the kernel of each piece and launches it.
+#include "input_transform_impl.h"
+
+using namespace wc;
+
+extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x,
+                                  int n_images, void* V, void* stream) {
+  WC_CHECK_ARG(d && plan && x && V, "wc_input_transform: null pointer");
+  WC_CHECK_ARG(n_images > 0, "wc_input_transform: n_images %d", n_images);
+  int out[3], grid[3];
+  int rc = wc_conv_out_dims(d, out, grid);
+  if (rc) return rc;
+  WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_input_transform: bad plan");
+  const int Cp = wc_padded_channels(d->C);
+  const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
+  const bool flat = plan->m[0] == 1;
+  const int vmax = flat ? 4 : 2;
+  const int vec = (d->C % vmax == 0) ? vmax : 1;
+  for (int s = 0; s < plan->n_pieces; ++s) {
+    const wc_piece& pc = plan->piece[s];
+    int k[3];
+    for (int a = 0; a < 3; ++a) {
+      k[a] = kind_of(plan->m[a], pc.r[a]);
+      if (k[a] < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[a], pc.r[a]);
+    }
+    InKernel fn = nullptr;
+    switch (k[0]) {
+      case KIND_11: fn = pick_in_2d(d->dtype, k[1], k[2], vec); break;
+      case KIND_21: fn = pick_in_3d_21(d->dtype, k[1], k[2], vec); break;
+      case KIND_22: fn = pick_in_3d_22(d->dtype, k[1], k[2], vec); break;
+      case KIND_23: fn = pick_in_3d_23(d->dtype, k[1], k[2], vec); break;
+      default: break;
+    }
+    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for kinds (%d,%d,%d) not built", k[0], k[1], k[2]);
+    InArgs a;
+    a.x = x; a.V = V;
+    a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = Cp;
+    a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
+    a.base0 = pc.tap0[0] - d->pad[0]; a.base1 = pc.tap0[1] - d->pad[1]; a.base2 = pc.tap0[2] - d->pad[2];
+    a.step = plan->tap_step;
+    a.t_stride = P * Cp;
+    a.t_offset = pc.t_offset;
+    a.n_cvec = Cp / vec;
+    a.total = P * a.n_cvec;
+    const long long blocks = ceil_div_ll(a.total, 256);
+    a.per_xcd = (int)ceil_div_ll(blocks, kXcds);
+    WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
+    hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, as_stream(stream), a);
+    WC_CHECK_LAUNCH("input_transform_kernel");
+  }
+  return WC_OK;
+}

@@ -1,0 +1,99 @@
+// Input transform kernel (included by the per-shape translation units).
+// Input transform V = (BT_d x BT_h x BT_w) d, channel-last input, one launch per piece.
+//
+// Replaces inputNorm2WinoTransform + inputNorm2WinoCalculation of the reference
+// (src/split_kernel.cu:60-120, src/calculation_kernels.cu:763-1522).  Window of tile t,
+// element i on one axis: step*(m*t + i) + tap0 - pad, zero outside (split_kernel.cu:78-100).
+//
+// HBM-bound: each thread owns one tile x VEC consecutive channels (lanes run along C, so a
+// wavefront reads and writes contiguous runs), transforms in fp32 registers with compile-time
+// tile sizes (no run-time indexed private arrays) and stores each transform-domain element once.
+// Workgroup ids are remapped so that one XCD walks a contiguous range of tiles: the halo rows
+// and columns shared by neighbouring tiles are then served by that XCD's L2.
+#pragma once
+#include "wc_transform.h"
+
+namespace wc {
+
+struct InArgs {
+  const void* x;
+  void* V;
+  int D, H, W, C, Cp;
+  int nD, nH, nW;
+  int base0, base1, base2;   // tap0 - pad per axis
+  int step;                  // convolution stride
+  long long t_stride;        // P * Cp
+  int t_offset;
+  int n_cvec;                // Cp / VEC
+  long long total;           // P * n_cvec
+  int per_xcd;
+};
+
+template <typename T, int K0, int K1, int K2, int VEC>
+__global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
+  constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
+  constexpr int m0 = Mats<K0>::m, m1 = Mats<K1>::m, m2 = Mats<K2>::m;
+  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int cv = (int)(idx % a.n_cvec);
+  const long long p = idx / a.n_cvec;
+  const int tw = (int)(p % a.nW); long long q = p / a.nW;
+  const int th = (int)(q % a.nH); q /= a.nH;
+  const int td = (int)(q % a.nD);
+  const long long b = q / a.nD;
+  const int c = cv * VEC;
+  const bool c_ok = c < a.C;
+  const T* x = static_cast<const T*>(a.x);
+
+  float d[A0 * A1 * A2][VEC];
+  static_for<0, A0>([&](auto i0_) {
+    constexpr int i0 = decltype(i0_)::value;
+    const int z = a.step * (m0 * td + i0) + a.base0;
+    const bool z_ok = c_ok && (unsigned)z < (unsigned)a.D;
+    static_for<0, A1>([&](auto i1_) {
+      constexpr int i1 = decltype(i1_)::value;
+      const int yy = a.step * (m1 * th + i1) + a.base1;
+      const bool y_ok = z_ok && (unsigned)yy < (unsigned)a.H;
+      const long long row = ((b * a.D + z) * a.H + yy) * a.W;
+      static_for<0, A2>([&](auto i2_) {
+        constexpr int i2 = decltype(i2_)::value;
+        constexpr int e = (i0 * A1 + i1) * A2 + i2;
+        const int xx = a.step * (m2 * tw + i2) + a.base2;
+        if (y_ok && (unsigned)xx < (unsigned)a.W) {
+          load_pack<T, VEC>(x + (row + xx) * a.C + c, d[e]);
+        } else {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) d[e][v] = 0.f;
+        }
+      });
+    });
+  });
+
+  // W, then H, then D (reference order: matrix_conv3d.py:162-163)
+  float t2[A0 * A1 * A2][VEC];
+  apply_axis<MatSel<K2, false>, 2, A0, A1, A2, VEC>(d, t2);
+  apply_axis<MatSel<K1, false>, 1, A0, A1, A2, VEC>(t2, d);
+  if constexpr (A0 > 1) {
+    apply_axis<MatSel<K0, false>, 0, A0, A1, A2, VEC>(d, t2);
+  }
+  T* V = static_cast<T*>(a.V) + (long long)a.t_offset * a.t_stride + p * a.Cp + c;
+  static_for<0, A0 * A1 * A2>([&](auto e_) {
+    constexpr int e = decltype(e_)::value;
+    if constexpr (A0 > 1) store_pack<T, VEC>(V + e * a.t_stride, t2[e]);
+    else store_pack<T, VEC>(V + e * a.t_stride, d[e]);
+  });
+}
+
+using InKernel = void (*)(InArgs);
+
+template <typename T, int VEC, int K0, int K1, int K2>
+constexpr InKernel in_kernel() { return &input_transform_kernel<T, K0, K1, K2, VEC>; }
+
+// Kernel look-up, one translation unit per depth kind so that they compile in parallel.
+InKernel pick_in_2d(int dtype, int k1, int k2, int vec);          // depth kind KIND_11, vec 4 or 1
+InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
+InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
+InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);
+
+}  // namespace wc

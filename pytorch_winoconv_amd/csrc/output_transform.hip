@@ -1,0 +1,248 @@
+// Output transform y = sum over pieces of (AT_d x AT_h x AT_w) m, + bias, cropped at the edges.
+//
+// Replaces outputWino2NormTransform + outputWino2NormCalculation + outputAggregate of the
+// reference (src/split_kernel.cu:126-203, src/calculation_kernels.cu:1524-1770).  The reference
+// stores one partial output per piece (tmp_output, base_conv_launchers.cu:375-377) and sums
+// them in a second pass; here every piece is accumulated in fp32 registers and y is written
+// once.  Edge rule as in the reference (split_kernel.cu:162-176): an output position is
+// written iff it lies inside (oD, oH, oW).
+//
+// HBM-bound: a thread owns one tile x VEC consecutive output channels (lanes along K).
+// Two kernels: a separable compile-time one for single-piece plans (F(2,3)^2, F(4,3)^2,
+// F(2,3)^3) and a streaming one for any multi-piece F(2,r) plan, where each loaded element
+// is scattered into the 2^d accumulators with coefficients from a constant table.
+#include "wc_transform.h"
+
+namespace wc {
+
+struct OutArgs {
+  const void* M;
+  const void* bias;
+  void* y;
+  int oD, oH, oW, K, ldm;
+  int nD, nH, nW;
+  long long t_stride;   // P * ldm
+  int t_offset;
+  int n_kvec;           // K / VEC
+  long long total;      // P * n_kvec
+  int per_xcd;
+};
+
+struct Where { int tw, th, td; long long b; };
+
+__device__ __forceinline__ Where decode_tile(long long p, int nD, int nH, int nW) {
+  Where w;
+  w.tw = (int)(p % nW); long long q = p / nW;
+  w.th = (int)(q % nH); q /= nH;
+  w.td = (int)(q % nD);
+  w.b = q / nD;
+  return w;
+}
+
+template <typename T, int M0, int M1, int M2, int VEC>
+__device__ __forceinline__ void write_tile(const OutArgs& a, const Where& w, int k,
+                                           float (&o)[M0 * M1 * M2][VEC]) {
+  T* y = static_cast<T*>(a.y);
+  float bias[VEC];
+  if (a.bias) load_pack<T, VEC>(static_cast<const T*>(a.bias) + k, bias);
+  static_for<0, M0>([&](auto a0_) {
+    constexpr int a0 = decltype(a0_)::value;
+    const int od = M0 * w.td + a0;
+    static_for<0, M1>([&](auto a1_) {
+      constexpr int a1 = decltype(a1_)::value;
+      const int oh = M1 * w.th + a1;
+      static_for<0, M2>([&](auto a2_) {
+        constexpr int a2 = decltype(a2_)::value;
+        constexpr int e = (a0 * M1 + a1) * M2 + a2;
+        const int ow = M2 * w.tw + a2;
+        if (od < a.oD && oh < a.oH && ow < a.oW) {
+          if (a.bias) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) o[e][v] += bias[v];
+          }
+          store_pack<T, VEC>(y + (((w.b * a.oD + od) * a.oH + oh) * a.oW + ow) * a.K + k, o[e]);
+        }
+      });
+    });
+  });
+}
+
+// ---- single piece, separable ------------------------------------------------------------------
+template <typename T, int K0, int K1, int K2, int VEC>
+__global__ __launch_bounds__(256) void output_transform_kernel(OutArgs a) {
+  constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
+  constexpr int M0 = Mats<K0>::m, M1 = Mats<K1>::m, M2 = Mats<K2>::m;
+  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int k = (int)(idx % a.n_kvec) * VEC;
+  const long long p = idx / a.n_kvec;
+  const Where w = decode_tile(p, a.nD, a.nH, a.nW);
+  const T* M = static_cast<const T*>(a.M) + (long long)a.t_offset * a.t_stride + p * a.ldm + k;
+
+  float m[A0 * A1 * A2][VEC];
+  static_for<0, A0 * A1 * A2>([&](auto e_) {
+    constexpr int e = decltype(e_)::value;
+    load_pack<T, VEC>(M + e * a.t_stride, m[e]);
+  });
+  float s2[A0 * A1 * M2][VEC];
+  apply_axis<MatSel<K2, true>, 2, A0, A1, A2, VEC>(m, s2);
+  float s1[A0 * M1 * M2][VEC];
+  apply_axis<MatSel<K1, true>, 1, A0, A1, M2, VEC>(s2, s1);
+  if constexpr (A0 > 1) {
+    float s0[M0 * M1 * M2][VEC];
+    apply_axis<MatSel<K0, true>, 0, A0, M1, M2, VEC>(s1, s0);
+    write_tile<T, M0, M1, M2, VEC>(a, w, k, s0);
+  } else {
+    write_tile<T, M0, M1, M2, VEC>(a, w, k, s1);
+  }
+}
+
+// ---- any number of F(2, r) pieces, streaming -----------------------------------------------------
+// AT of F(2, r) by [r][output a][element i] (r = 0 is the one-element depth axis)
+__constant__ const float kAT2[4][2][4] = {
+    {{1, 0, 0, 0}, {0, 0, 0, 0}},
+    {{1, 0, 0, 0}, {0, 1, 0, 0}},
+    {{1, 1, 0, 0}, {0, 1, 1, 0}},
+    {{1, 1, 1, 0}, {0, 1, -1, -1}},
+};
+
+struct OutMultiArgs {
+  OutArgs o;
+  int n_pieces;
+  int info[WC_MAX_PIECES];   // t_offset | r0 << 16 | r1 << 20 | r2 << 24 (r0 = 0: flat depth)
+};
+
+template <typename T, bool FLAT, int VEC>
+__global__ __launch_bounds__(256) void output_multi_kernel(OutMultiArgs g) {
+  constexpr int M0 = FLAT ? 1 : 2;
+  const OutArgs& a = g.o;
+  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int k = (int)(idx % a.n_kvec) * VEC;
+  const long long p = idx / a.n_kvec;
+  const Where w = decode_tile(p, a.nD, a.nH, a.nW);
+  const T* M = static_cast<const T*>(a.M) + p * a.ldm + k;
+
+  float acc[M0 * 4][VEC];
+#pragma unroll
+  for (int e = 0; e < M0 * 4; ++e)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[e][v] = 0.f;
+
+  for (int s = 0; s < g.n_pieces; ++s) {
+    const int info = g.info[s];
+    const int r0 = (info >> 16) & 15, r1 = (info >> 20) & 15, r2 = (info >> 24) & 15;
+    const int n0 = FLAT ? 1 : r0 + 1, n1 = r1 + 1, n2 = r2 + 1;
+    const T* Ms = M + (long long)(info & 0xffff) * a.t_stride;
+    for (int i0 = 0; i0 < n0; ++i0)
+      for (int i1 = 0; i1 < n1; ++i1)
+        for (int i2 = 0; i2 < n2; ++i2) {
+          float v[VEC];
+          load_pack<T, VEC>(Ms + (long long)((i0 * n1 + i1) * n2 + i2) * a.t_stride, v);
+          static_for<0, M0>([&](auto a0_) {
+            constexpr int a0 = decltype(a0_)::value;
+            const float c0 = kAT2[r0][a0][i0];
+            static_for<0, 2>([&](auto a1_) {
+              constexpr int a1 = decltype(a1_)::value;
+              const float c01 = c0 * kAT2[r1][a1][i1];
+              static_for<0, 2>([&](auto a2_) {
+                constexpr int a2 = decltype(a2_)::value;
+                const float c = c01 * kAT2[r2][a2][i2];
+#pragma unroll
+                for (int q = 0; q < VEC; ++q)
+                  acc[(a0 * 2 + a1) * 2 + a2][q] = __builtin_fmaf(c, v[q], acc[(a0 * 2 + a1) * 2 + a2][q]);
+              });
+            });
+          });
+        }
+  }
+  write_tile<T, M0, 2, 2, VEC>(a, w, k, acc);
+}
+
+using OutKernel = void (*)(OutArgs);
+using OutMultiKernel = void (*)(OutMultiArgs);
+
+template <typename T>
+static OutKernel pick_single(int k0, int k1, int k2, int vec) {
+  if (k0 == KIND_11 && k1 == KIND_23 && k2 == KIND_23)
+    return vec == 4 ? &output_transform_kernel<T, KIND_11, KIND_23, KIND_23, 4>
+                    : &output_transform_kernel<T, KIND_11, KIND_23, KIND_23, 1>;
+  if (k0 == KIND_11 && k1 == KIND_43 && k2 == KIND_43)
+    return vec == 4 ? &output_transform_kernel<T, KIND_11, KIND_43, KIND_43, 4>
+                    : &output_transform_kernel<T, KIND_11, KIND_43, KIND_43, 1>;
+  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23)
+    return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 2>
+                    : &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 1>;
+  return nullptr;
+}
+
+template <typename T>
+static OutMultiKernel pick_multi(bool flat, int vec) {
+  if (flat) return vec == 4 ? &output_multi_kernel<T, true, 4> : &output_multi_kernel<T, true, 1>;
+  return vec == 4 ? &output_multi_kernel<T, false, 4> : &output_multi_kernel<T, false, 1>;
+}
+
+}  // namespace wc
+
+using namespace wc;
+
+extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, const void* M,
+                                   const void* bias, int n_images, void* y, void* stream) {
+  WC_CHECK_ARG(d && plan && M && y, "wc_output_transform: null pointer");
+  WC_CHECK_ARG(n_images > 0, "wc_output_transform: n_images %d", n_images);
+  int out[3], grid[3];
+  int rc = wc_conv_out_dims(d, out, grid);
+  if (rc) return rc;
+  WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_output_transform: bad plan");
+  const int ldm = wc_padded_channels8(d->K);
+  const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
+  const int vec = (d->K % 4 == 0) ? 4 : 1;
+  OutArgs a;
+  a.M = M; a.bias = bias; a.y = y;
+  a.oD = out[0]; a.oH = out[1]; a.oW = out[2]; a.K = d->K; a.ldm = ldm;
+  a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
+  a.t_stride = P * ldm;
+  a.t_offset = 0;
+  hipStream_t s = as_stream(stream);
+
+  int k[3] = {0, 0, 0};
+  OutKernel single = nullptr;
+  if (plan->n_pieces == 1) {
+    for (int q = 0; q < 3; ++q) k[q] = kind_of(plan->m[q], plan->piece[0].r[q]);
+    single = d->dtype == WC_F16 ? pick_single<half_t>(k[0], k[1], k[2], vec)
+                                : pick_single<float>(k[0], k[1], k[2], vec);
+  }
+  if (single) {
+    const int v = (k[0] == KIND_23 && vec == 4) ? 2 : vec;   // 3-D tiles use 2 channels per thread
+    a.n_kvec = d->K / v;
+    a.total = P * a.n_kvec;
+    a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);
+    a.t_offset = plan->piece[0].t_offset;
+    hipLaunchKernelGGL(single, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, a);
+    WC_CHECK_LAUNCH("output_transform_kernel");
+    return WC_OK;
+  }
+  if (plan->m[1] != 2 || plan->m[2] != 2 || (plan->m[0] != 1 && plan->m[0] != 2))
+    return fail(WC_ERR_UNSUPPORTED, "multi-piece output transform needs output tile 2");
+  if (plan->t_total > 0xffff)
+    return fail(WC_ERR_UNSUPPORTED, "plan with %d transform elements is too large", plan->t_total);
+  OutMultiArgs g;
+  const bool flat = plan->m[0] == 1;
+  a.n_kvec = d->K / vec;
+  a.total = P * a.n_kvec;
+  a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);
+  g.o = a;
+  g.n_pieces = plan->n_pieces;
+  for (int i = 0; i < plan->n_pieces; ++i) {
+    const wc_piece& pc = plan->piece[i];
+    for (int q = 0; q < 3; ++q)
+      if (pc.r[q] < 1 || pc.r[q] > 3) return fail(WC_ERR_UNSUPPORTED, "piece with %d taps", pc.r[q]);
+    g.info[i] = pc.t_offset | ((flat ? 0 : pc.r[0]) << 16) | (pc.r[1] << 20) | (pc.r[2] << 24);
+  }
+  OutMultiKernel fn = d->dtype == WC_F16 ? pick_multi<half_t>(flat, vec) : pick_multi<float>(flat, vec);
+  hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, g);
+  WC_CHECK_LAUNCH("output_multi_kernel");
+  return WC_OK;
+}

@@ -1,0 +1,180 @@
+// Host-side planning and error reporting (no device code).
+//
+// The split rule replaces the reference's 36-key look-up table
+// (reference: src/base_conv_launchers.h:58-388): per axis an extent k is cut into chunks of
+// 3 with the remainder last, except 4 -> 2 + 2; boxes are the Cartesian product of the
+// per-axis chunks, depth outermost and width fastest; the transform-domain offset of a box
+// is the running sum of prod(size + m - 1) (reference: src/base_conv_launchers.cu:307-313).
+// Stride 2 - which the reference rejects (src/winograd_conv.cpp:122-126) - is handled by
+// separating the taps of each axis by parity first:
+//   y[o] = sum_k x[2o + k - pad] w[k] = sum_q sum_j x[2(o + j) + q - pad] w[2j + q].
+#include "wc_common.h"
+#include "wc_tables.h"
+#include <cstring>
+#include <string>
+
+namespace wc {
+
+static thread_local std::string g_err;
+
+void set_error(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+}
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+struct AxisPiece { int tap0, r; };
+
+// chunks of one axis at stride 1: fills (start, size), returns the count
+static int axis_chunks(int k, int* start, int* size) {
+  int n = 0, s = 0;
+  if (k == 4) {
+    start[0] = 0; size[0] = 2; start[1] = 2; size[1] = 2;
+    return 2;
+  }
+  while (k - s >= 3) { start[n] = s; size[n] = 3; s += 3; ++n; }
+  if (k - s > 0) { start[n] = s; size[n] = k - s; ++n; }
+  return n;
+}
+
+static int axis_pieces(int k, int stride, AxisPiece* out) {
+  int n = 0;
+  int start[8], size[8];
+  for (int q = 0; q < stride; ++q) {
+    int taps = (k - q + stride - 1) / stride;
+    if (taps <= 0) continue;
+    int c = axis_chunks(taps, start, size);
+    for (int i = 0; i < c; ++i) { out[n].tap0 = q + stride * start[i]; out[n].r = size[i]; ++n; }
+  }
+  return n;
+}
+
+}  // namespace wc
+
+using namespace wc;
+
+extern "C" {
+
+const char* wc_version(void) { return "winoconv-hip 0.1 (gfx950)"; }
+const char* wc_last_error(void) { return g_err.c_str(); }
+
+int wc_padded_channels(int C) { return (C + 31) / 32 * 32; }
+int wc_padded_channels8(int K) { return (K + 7) / 8 * 8; }
+
+int wc_plan_dwm(int kD, int kH, int kW, int* num_split, int* D_start, int* D_end, int* H_start,
+                int* H_end, int* W_start, int* W_end, int* kernel_stride, int* t_total) {
+  WC_CHECK_ARG(num_split && D_start && D_end && H_start && H_end && W_start && W_end &&
+                   kernel_stride && t_total, "wc_plan_dwm: null output pointer");
+  if (kD < 1 || kH < 1 || kW < 1 || kD > 10 || kH > 10 || kW > 10)
+    return fail(WC_ERR_UNSUPPORTED, "wc_plan_dwm: kernel %dx%dx%d outside 1..10", kD, kH, kW);
+  int ds[8], dz[8], hs[8], hz[8], ws[8], wz[8];
+  int nd = axis_chunks(kD, ds, dz), nh = axis_chunks(kH, hs, hz), nw = axis_chunks(kW, ws, wz);
+  if (nd * nh * nw > WC_MAX_PIECES)
+    return fail(WC_ERR_UNSUPPORTED, "wc_plan_dwm: %d pieces exceed %d", nd * nh * nw, WC_MAX_PIECES);
+  int n = 0, t = 0;
+  for (int a = 0; a < nd; ++a)
+    for (int b = 0; b < nh; ++b)
+      for (int c = 0; c < nw; ++c) {
+        D_start[n] = ds[a]; D_end[n] = ds[a] + dz[a];
+        H_start[n] = hs[b]; H_end[n] = hs[b] + hz[b];
+        W_start[n] = ws[c]; W_end[n] = ws[c] + wz[c];
+        kernel_stride[n] = t;
+        t += (dz[a] + 1) * (hz[b] + 1) * (wz[c] + 1);
+        ++n;
+      }
+  *num_split = n;
+  *t_total = t;
+  return WC_OK;
+}
+
+static int check_desc(const wc_conv_desc* d) {
+  WC_CHECK_ARG(d != nullptr, "null descriptor");
+  WC_CHECK_ARG(d->ndim == 2 || d->ndim == 3, "ndim must be 2 or 3, got %d", d->ndim);
+  WC_CHECK_ARG(d->N > 0 && d->C > 0 && d->K > 0, "N, C, K must be positive (%d, %d, %d)", d->N, d->C, d->K);
+  WC_CHECK_ARG(d->dtype == WC_F32 || d->dtype == WC_F16, "unknown dtype %d", d->dtype);
+  for (int a = 0; a < 3; ++a) {
+    WC_CHECK_ARG(d->in[a] > 0 && d->kernel[a] > 0 && d->pad[a] >= 0,
+                 "axis %d: input %d, kernel %d, pad %d", a, d->in[a], d->kernel[a], d->pad[a]);
+    if (d->kernel[a] > 10)
+      return fail(WC_ERR_UNSUPPORTED, "kernel extent %d > 10 on axis %d", d->kernel[a], a);
+    if (d->in[a] + 2 * d->pad[a] < d->kernel[a])
+      return fail(WC_ERR_BAD_ARG, "axis %d: padded input %d smaller than kernel %d", a,
+                  d->in[a] + 2 * d->pad[a], d->kernel[a]);
+  }
+  if (d->ndim == 2)
+    WC_CHECK_ARG(d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0,
+                 "2-D problem needs depth extent 1, kernel 1, pad 0");
+  if (d->stride != 1 && d->stride != 2)
+    return fail(WC_ERR_UNSUPPORTED, "stride %d not implemented (1 or 2)", d->stride);
+  if (d->m != 2 && d->m != 4)
+    return fail(WC_ERR_UNSUPPORTED, "output tile %d not implemented (2 or 4)", d->m);
+  if (d->m == 4 && !(d->ndim == 2 && d->stride == 1 && d->kernel[1] == 3 && d->kernel[2] == 3))
+    return fail(WC_ERR_UNSUPPORTED, "output tile 4 is implemented for 2-D 3x3 stride-1 only");
+  WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
+  return WC_OK;
+}
+
+int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
+  int rc = check_desc(d);
+  if (rc) return rc;
+  WC_CHECK_ARG(plan != nullptr, "wc_plan_conv: null plan");
+  AxisPiece ax[3][8];
+  int n[3];
+  for (int a = 0; a < 3; ++a) n[a] = axis_pieces(d->kernel[a], d->stride, ax[a]);
+  if (n[0] * n[1] * n[2] > WC_MAX_PIECES)
+    return fail(WC_ERR_UNSUPPORTED, "%d pieces exceed %d", n[0] * n[1] * n[2], WC_MAX_PIECES);
+  std::memset(plan, 0, sizeof(*plan));
+  plan->tap_step = d->stride;
+  const bool flat_depth = (d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0);
+  plan->m[0] = flat_depth ? 1 : d->m;
+  plan->m[1] = d->m;
+  plan->m[2] = d->m;
+  int np = 0, t = 0;
+  for (int a = 0; a < n[0]; ++a)
+    for (int b = 0; b < n[1]; ++b)
+      for (int c = 0; c < n[2]; ++c) {
+        wc_piece& p = plan->piece[np++];
+        p.tap0[0] = ax[0][a].tap0; p.r[0] = ax[0][a].r;
+        p.tap0[1] = ax[1][b].tap0; p.r[1] = ax[1][b].r;
+        p.tap0[2] = ax[2][c].tap0; p.r[2] = ax[2][c].r;
+        p.t_offset = t;
+        int e = 1;
+        for (int q = 0; q < 3; ++q) {
+          if (kind_of(plan->m[q], p.r[q]) < 0)
+            return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) on axis %d not implemented", plan->m[q], p.r[q], q);
+          e *= plan->m[q] + p.r[q] - 1;
+        }
+        t += e;
+      }
+  plan->n_pieces = np;
+  plan->t_total = t;
+  return WC_OK;
+}
+
+int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
+  int rc = check_desc(d);
+  if (rc) return rc;
+  WC_CHECK_ARG(out && grid, "wc_conv_out_dims: null output");
+  const bool flat_depth = (d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0);
+  for (int a = 0; a < 3; ++a) {
+    out[a] = (d->in[a] + 2 * d->pad[a] - d->kernel[a]) / d->stride + 1;
+    int m = (a == 0 && flat_depth) ? 1 : d->m;
+    grid[a] = (out[a] + m - 1) / m;
+  }
+  return WC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+// Shared host/device helpers for the gfx950 Winograd engine.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <cstdarg>
+#include <type_traits>
+#include "../../include/winoconv.h"
+
+namespace wc {
+
+// ---- error reporting (thread-local message behind wc_last_error) -------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+
+#define WC_CHECK_ARG(cond, ...) \
+  do { if (!(cond)) return ::wc::fail(WC_ERR_BAD_ARG, __VA_ARGS__); } while (0)
+#define WC_CHECK_HIP(expr)                                                               \
+  do { hipError_t e_ = (expr);                                                           \
+       if (e_ != hipSuccess)                                                             \
+         return ::wc::fail(WC_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));   \
+  } while (0)
+#define WC_CHECK_LAUNCH(name)                                                            \
+  do { hipError_t e_ = hipGetLastError();                                                \
+       if (e_ != hipSuccess)                                                             \
+         return ::wc::fail(WC_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline long long ceil_div_ll(long long a, long long b) { return (a + b - 1) / b; }
+
+// ---- compile-time loops ---------------------------------------------------------------------
+template <int I> using ic = std::integral_constant<int, I>;
+
+template <int Begin, int End, typename F>
+__host__ __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (Begin < End) {
+    f(ic<Begin>{});
+    static_for<Begin + 1, End>(static_cast<F&&>(f));
+  }
+}
+
+// ---- packed element vectors -------------------------------------------------------------------
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+
+using half_t = _Float16;
+
+// Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
+constexpr int kXcds = 8;
+
+// Maps the hardware workgroup id to a logical one so that each XCD owns one contiguous
+// range of logical ids (neighbouring tiles then share that XCD's L2).  `per_xcd` is
+// ceil(n_logical / 8); the launch uses 8 * per_xcd workgroups, ids >= n_logical idle.
+__device__ __forceinline__ int xcd_remap(int hw_id, int per_xcd) {
+  return (hw_id % kXcds) * per_xcd + hw_id / kXcds;
+}
+
+}  // namespace wc

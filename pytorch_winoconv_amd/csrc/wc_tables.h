@@ -1,0 +1,120 @@
+// Winograd transform matrices as compile-time tables.
+//
+// Kinds (one per axis of a piece):
+//   KIND_11  F(1,1)  alpha 1   size-1 axis (the depth of a 2-D problem)
+//   KIND_21  F(2,1)  alpha 2   (reference literal: matrix_conv.py:15-20)
+//   KIND_22  F(2,2)  alpha 3   (reference literal: matrix_convnd.py:20-27)
+//   KIND_23  F(2,3)  alpha 4   (reference literal: matrix_conv.py:21-30)
+//   KIND_43  F(4,3)  alpha 6   Cook-Toom over the points 0, 1, -1, 2, -2 - the point set the
+//                              reference uses for F(2,5) (matrix_conv.py:33); BT equals the
+//                              reference's commented B25 (transform.py:35-40).
+// AT is m x alpha, G is alpha x r, BT is alpha x alpha, all stored in 6-wide rows.
+#pragma once
+#include "wc_common.h"
+
+namespace wc {
+
+enum Kind { KIND_11 = 0, KIND_21 = 1, KIND_22 = 2, KIND_23 = 3, KIND_43 = 4, KIND_COUNT = 5 };
+
+__host__ __device__ constexpr int kind_m(int k) { return k == KIND_11 ? 1 : (k == KIND_43 ? 4 : 2); }
+__host__ __device__ constexpr int kind_r(int k) {
+  return k == KIND_11 ? 1 : k == KIND_21 ? 1 : k == KIND_22 ? 2 : 3;
+}
+__host__ __device__ constexpr int kind_alpha(int k) { return kind_m(k) + kind_r(k) - 1; }
+
+// kind for (m, r); -1 if the pair is not supported
+inline int kind_of(int m, int r) {
+  if (m == 1 && r == 1) return KIND_11;
+  if (m == 2 && r >= 1 && r <= 3) return KIND_21 + (r - 1);
+  if (m == 4 && r == 3) return KIND_43;
+  return -1;
+}
+
+template <int KIND> struct Mats;
+
+template <> struct Mats<KIND_11> {
+  static constexpr int m = 1, r = 1, alpha = 1;
+  __host__ __device__ static constexpr float at(int i, int j) { return 1.f; }
+  __host__ __device__ static constexpr float g(int i, int j) { return 1.f; }
+  __host__ __device__ static constexpr float bt(int i, int j) { return 1.f; }
+};
+template <> struct Mats<KIND_21> {
+  static constexpr int m = 2, r = 1, alpha = 2;
+  __host__ __device__ static constexpr float at(int i, int j) { return i == j ? 1.f : 0.f; }
+  __host__ __device__ static constexpr float g(int i, int j) { return 1.f; }
+  __host__ __device__ static constexpr float bt(int i, int j) { return i == j ? 1.f : 0.f; }
+};
+template <> struct Mats<KIND_22> {
+  static constexpr int m = 2, r = 2, alpha = 3;
+  __host__ __device__ static constexpr float at(int i, int j) {
+    constexpr float t[2][3] = {{1, 1, 0}, {0, 1, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float g(int i, int j) {
+    constexpr float t[3][2] = {{1, 0}, {1, 1}, {0, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float bt(int i, int j) {
+    constexpr float t[3][3] = {{1, -1, 0}, {0, 1, 0}, {0, -1, 1}};
+    return t[i][j];
+  }
+};
+template <> struct Mats<KIND_23> {
+  static constexpr int m = 2, r = 3, alpha = 4;
+  __host__ __device__ static constexpr float at(int i, int j) {
+    constexpr float t[2][4] = {{1, 1, 1, 0}, {0, 1, -1, -1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float g(int i, int j) {
+    constexpr float t[4][3] = {{1, 0, 0}, {.5f, .5f, .5f}, {.5f, -.5f, .5f}, {0, 0, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float bt(int i, int j) {
+    constexpr float t[4][4] = {{1, 0, -1, 0}, {0, 1, 1, 0}, {0, -1, 1, 0}, {0, 1, 0, -1}};
+    return t[i][j];
+  }
+};
+template <> struct Mats<KIND_43> {
+  static constexpr int m = 4, r = 3, alpha = 6;
+  __host__ __device__ static constexpr float at(int i, int j) {
+    constexpr float t[4][6] = {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, 0},
+                               {0, 1, 1, 4, 4, 0}, {0, 1, -1, 8, -8, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float g(int i, int j) {
+    constexpr float t[6][3] = {{1.f / 4, 0, 0},
+                               {-1.f / 6, -1.f / 6, -1.f / 6},
+                               {-1.f / 6, 1.f / 6, -1.f / 6},
+                               {1.f / 24, 1.f / 12, 1.f / 6},
+                               {1.f / 24, -1.f / 12, 1.f / 6},
+                               {0, 0, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float bt(int i, int j) {
+    constexpr float t[6][6] = {{4, 0, -5, 0, 1, 0},  {0, -4, -4, 1, 1, 0}, {0, 4, -4, -1, 1, 0},
+                               {0, -2, -1, 2, 1, 0}, {0, 2, -1, -2, 1, 0}, {0, 4, 0, -5, 0, 1}};
+    return t[i][j];
+  }
+};
+
+// Run-time views of the same tables (host planning, the generic filter / multi-piece kernels).
+__host__ __device__ inline float table_g(int kind, int i, int j) {
+  switch (kind) {
+    case KIND_11: return Mats<KIND_11>::g(i, j);
+    case KIND_21: return Mats<KIND_21>::g(i, j);
+    case KIND_22: return Mats<KIND_22>::g(i, j);
+    case KIND_23: return Mats<KIND_23>::g(i, j);
+    default: return Mats<KIND_43>::g(i, j);
+  }
+}
+__host__ __device__ inline float table_at(int kind, int i, int j) {
+  switch (kind) {
+    case KIND_11: return Mats<KIND_11>::at(i, j);
+    case KIND_21: return Mats<KIND_21>::at(i, j);
+    case KIND_22: return Mats<KIND_22>::at(i, j);
+    case KIND_23: return Mats<KIND_23>::at(i, j);
+    default: return Mats<KIND_43>::at(i, j);
+  }
+}
+
+}  // namespace wc

@@ -1,0 +1,189 @@
+"""Host-side orchestration over the C ABI: descriptors, plans, workspaces, streams.
+
+torch is used for device memory (its caching allocator) and for the current HIP
+stream only; all arithmetic is done by the HIP kernels behind libwinoconv_hip.so.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import ConvDesc, Plan, check
+
+_DTYPES = {torch.float32: _lib.WC_F32, torch.float16: _lib.WC_F16}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("winoconv runs on the GPU only: got a %s tensor" % t.device)
+        if t.dtype not in _DTYPES:
+            raise TypeError("winoconv supports float32 and float16, got %s" % t.dtype)
+
+
+def _triple(v, nd, fill):
+    if isinstance(v, int):
+        v = (v,) * nd
+    v = tuple(int(a) for a in v)
+    if len(v) != nd:
+        raise ValueError("expected %d values, got %r" % (nd, v))
+    return ((fill,) if nd == 2 else ()) + v
+
+
+def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0):
+    """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter."""
+    nd = len(x_shape) - 2
+    if nd not in (2, 3) or len(w_shape) != nd + 2:
+        raise ValueError("expected 4-D or 5-D input and matching filter, got %r and %r"
+                         % (tuple(x_shape), tuple(w_shape)))
+    if x_shape[1] != w_shape[1]:
+        raise ValueError("input has %d channels, filter expects %d (groups are not supported)"
+                         % (x_shape[1], w_shape[1]))
+    if isinstance(stride, (tuple, list)):
+        if len(set(int(s) for s in stride)) != 1:
+            raise NotImplementedError("stride must be the same on every axis, got %r" % (stride,))
+        stride = int(stride[0])
+    d = ConvDesc()
+    d.ndim = nd
+    d.N, d.C, d.K = int(x_shape[0]), int(x_shape[1]), int(w_shape[0])
+    d.in_[:] = ((1,) if nd == 2 else ()) + tuple(int(v) for v in x_shape[2:])
+    d.kernel[:] = ((1,) if nd == 2 else ()) + tuple(int(v) for v in w_shape[2:])
+    d.pad[:] = _triple(padding, nd, 0)
+    d.stride = int(stride)
+    d.m = int(m)
+    d.dtype = _DTYPES[dtype]
+    d.chunk_images = int(chunk_images)
+    return d
+
+
+def plan_conv(desc):
+    plan = Plan()
+    check(_lib.load().wc_plan_conv(ctypes.byref(desc), ctypes.byref(plan)))
+    return plan
+
+
+def out_dims(desc):
+    out = (ctypes.c_int * 3)()
+    grid = (ctypes.c_int * 3)()
+    check(_lib.load().wc_conv_out_dims(ctypes.byref(desc), out, grid))
+    return list(out), list(grid)
+
+
+def plan_dwm(kD, kH, kW):
+    """The reference's splitControl() table for one kernel size, as a dict of lists."""
+    arrs = [(ctypes.c_int * _lib.WC_MAX_PIECES)() for _ in range(7)]
+    n, t = ctypes.c_int(), ctypes.c_int()
+    check(_lib.load().wc_plan_dwm(kD, kH, kW, ctypes.byref(n), *arrs, ctypes.byref(t)))
+    names = ("D_start", "D_end", "H_start", "H_end", "W_start", "W_end", "kernel_stride")
+    out = {k: list(a[:n.value]) for k, a in zip(names, arrs)}
+    out["T_total"] = t.value
+    return out
+
+
+def channel_last(x):
+    """(N, C, *sp) tensor -> contiguous (N, *sp, C) view; zero-copy for channels_last memory."""
+    nd = x.dim() - 2
+    perm = (0,) + tuple(range(2, 2 + nd)) + (1,)
+    v = x.permute(perm)
+    return v if v.is_contiguous() else v.contiguous()
+
+
+def channel_first_view(y_cl):
+    """(N, *sp, K) contiguous tensor -> (N, K, *sp) view (channels_last memory format)."""
+    nd = y_cl.dim() - 2
+    return y_cl.permute((0, nd + 1) + tuple(range(1, nd + 1)))
+
+
+def _w_strides(w):
+    """Element strides of a (K, C, [kD,] kH, kW) filter view as (K, C, kD, kH, kW)."""
+    s = list(w.stride())
+    if w.dim() == 4:
+        s = s[:2] + [0] + s[2:]
+    return (ctypes.c_int64 * 5)(*s)
+
+
+# ---------------------------------------------------------------- stages (used by the tests)
+def filter_transform(desc, plan, w):
+    _require_gpu(w)
+    Cp = _lib.load().wc_padded_channels(desc.C)
+    U = torch.empty(plan.t_total, desc.K, Cp, dtype=w.dtype, device=w.device)
+    check(_lib.load().wc_filter_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(w),
+                                          _w_strides(w), _ptr(U), _stream(w)))
+    return U
+
+
+def input_transform(desc, plan, x_cl):
+    _require_gpu(x_cl)
+    lib = _lib.load()
+    _, grid = out_dims(desc)
+    n = x_cl.shape[0]
+    P = n * grid[0] * grid[1] * grid[2]
+    V = torch.empty(plan.t_total, P, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
+    check(lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(x_cl), n, _ptr(V), _stream(x_cl)))
+    return V
+
+
+def batched_gemm(V, U):
+    _require_gpu(V, U)
+    lib = _lib.load()
+    T, P, Cp = V.shape
+    K = U.shape[1]
+    if U.shape[0] != T or U.shape[2] != Cp or not V.is_contiguous() or not U.is_contiguous():
+        raise ValueError("V (T,P,Cp) and U (T,K,Cp) must be contiguous and agree on T and Cp")
+    ldm = lib.wc_padded_channels8(K)
+    M = torch.empty(T, P, ldm, dtype=V.dtype, device=V.device)
+    check(lib.wc_batched_gemm(_ptr(V), _ptr(U), _ptr(M), T, P, Cp, K, ldm, _DTYPES[V.dtype], _stream(V)))
+    return M
+
+
+def output_transform(desc, plan, M, bias, n_images):
+    _require_gpu(M, bias)
+    lib = _lib.load()
+    out, _ = out_dims(desc)
+    y = torch.empty(n_images, out[0], out[1], out[2], desc.K, dtype=M.dtype, device=M.device)
+    check(lib.wc_output_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(M), _ptr(bias),
+                                  n_images, _ptr(y), _stream(M)))
+    return y
+
+
+# ---------------------------------------------------------------- whole convolution
+def transform_filter(w, x_shape, stride=1, padding=0, m=2):
+    """Transformed filter U for later calls of conv_forward(..., U=U)."""
+    _require_gpu(w)
+    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m)
+    return filter_transform(desc, plan_conv(desc), w)
+
+
+def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0):
+    """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
+    is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
+    without a copy, any other layout is permuted once."""
+    _require_gpu(x, w, bias, U)
+    if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("input, filter and bias must share one dtype")
+    lib = _lib.load()
+    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images)
+    out, _ = out_dims(desc)
+    x_cl = channel_last(x)
+    nbytes = ctypes.c_size_t()
+    check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+    osp = out[1:] if desc.ndim == 2 else out
+    y = torch.empty([desc.N] + osp + [desc.K], dtype=x.dtype, device=x.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    if U is not None and not U.is_contiguous():
+        raise ValueError("U must be contiguous")
+    check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_cl), _ptr(w), _w_strides(w), _ptr(U),
+                              _ptr(bias), _ptr(y), _ptr(ws), nbytes.value, _stream(x)))
+    return channel_first_view(y)

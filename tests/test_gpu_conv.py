@@ -1,0 +1,148 @@
+"""End-to-end parity of wc_conv_forward (through the C ABI) against fp64 torch convolution and
+against the CPU oracle run in the same arithmetic discipline.
+
+Tolerances (max |y - y64| / max |y64|, fp64 conv fed the same already-rounded inputs):
+  fp32 F(2x2,3x3) and every fp32 F(2,r) plan: 1e-3 (measured ~1e-6),
+  fp16 (any plan, F(4x4,3x3) included):       2e-2.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import winograd as ow
+from pytorch_winoconv_amd import engine
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-3, torch.float16: 2e-2}
+DISC = {torch.float32: "fp32", torch.float16: "fp16"}
+
+
+def _data(xs, ws, dtype, seed=0, uniform=False):
+    g = torch.Generator().manual_seed(seed)
+    if uniform:
+        x, w = torch.rand(*xs, generator=g), torch.rand(*ws, generator=g)
+    else:
+        fan_in = 1
+        for v in ws[1:]:
+            fan_in *= v
+        x = torch.randn(*xs, generator=g)
+        w = torch.randn(*ws, generator=g) * (2.0 / fan_in) ** 0.5
+    b = torch.randn(ws[0], generator=g)
+    return x.to(dtype), w.to(dtype), b.to(dtype)
+
+
+def _conv64(x, w, b, stride, pad):
+    f = F.conv2d if x.dim() == 4 else F.conv3d
+    return f(x.double(), w.double(), None if b is None else b.double(), stride=stride, padding=pad)
+
+
+def _nerr(y, ref):
+    return float((y.double().cpu() - ref).abs().max() / ref.abs().max())
+
+
+CASES = [
+    # reduced-size versions of the benchmark configurations and of the reference's own demos
+    ((1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2),        # configs[0] at full size
+    ((2, 64, 56, 56), (64, 64, 3, 3), 1, 1, 4),
+    ((2, 3, 32, 32), (64, 3, 3, 3), 1, 1, 2),           # VGG first layer shape (C = 3)
+    ((2, 3, 32, 32), (64, 3, 3, 3), 1, 1, 4),
+    ((3, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4),      # ResNet-style
+    ((4, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4),
+    ((4, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4),
+    ((2, 32, 23, 21), (48, 32, 3, 3), 1, 1, 4),         # odd extents: partial edge tiles
+    ((2, 32, 23, 21), (48, 32, 3, 3), 1, 0, 2),
+    ((2, 32, 28, 28), (32, 32, 5, 5), 1, 2, 2),         # DWM
+    ((2, 32, 28, 28), (32, 32, 7, 7), 1, 3, 2),
+    ((2, 32, 28, 28), (32, 32, 3, 3), 2, 1, 2),
+    ((2, 32, 28, 28), (32, 32, 7, 7), 2, 3, 2),
+    ((1, 224, 10, 10), (32, 224, 7, 7), 1, 0, 2),       # example.py:100-101
+    ((1, 32, 10, 10, 10), (32, 32, 3, 3, 3), 1, 0, 2),  # example.py:112-113
+    ((2, 32, 8, 14, 14), (32, 32, 3, 3, 3), 1, 1, 2),   # C3D-style
+    ((1, 16, 6, 9, 9), (16, 16, 5, 5, 5), 1, 2, 2),
+    ((1, 8, 12, 12), (8, 8, 9, 9), 1, 4, 2),
+    ((1, 8, 14, 14), (8, 8, 4, 3), 1, 0, 2),
+    ((1, 8, 9, 9, 9), (8, 8, 1, 3, 3), 1, 0, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_conv_vs_fp64(dev, dtype, case):
+    xs, ws, stride, pad, m = case
+    x, w, b = _data(xs, ws, dtype)
+    ref = _conv64(x, w, b, stride, pad)
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), stride, pad, m)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert y.dtype == dtype
+    assert _nerr(y, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", [c for c in CASES if c[0][0] * c[0][1] <= 256])
+def test_conv_vs_oracle_same_discipline(dev, dtype, case):
+    """HIP result against the CPU restatement with the same storage/rounding points: only the
+    summation order differs.  fp32: <= 1e-5.  fp16: a different order flips single fp16
+    roundings of M by one ulp (4.9e-4 relative), which A^T x A^T of F(4,3) amplifies by up to
+    64: <= 1e-2 of the output range."""
+    xs, ws, stride, pad, m = case
+    x, w, _ = _data(xs, ws, dtype, seed=5)
+    want = ow.dwm_conv(x, w, None, stride, pad, m, DISC[dtype])
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, stride, pad, m)
+    assert _nerr(y, want.double()) <= (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", [
+    ((2, 16, 11, 12), (8, 16, 3, 3), 1, 1, 2, 4),
+    ((2, 16, 12, 12), (8, 16, 5, 5), 1, 2, 2, 4),
+    ((1, 16, 13, 12), (8, 16, 7, 7), 2, 3, 2, 4),
+    ((1, 8, 6, 8, 8), (8, 8, 3, 3, 3), 1, 1, 2, 8),
+])
+def test_integer_exactness(dev, dtype, case):
+    """With integer inputs and integer weights that are multiples of the common denominator of
+    G x G (x G) (4 in 2-D, 8 in 3-D for F(2,r), whose G holds only 0, 1 and 1/2) every
+    intermediate is exactly representable, so Winograd must equal direct convolution bit for bit.
+    F(4,3) is left out: its G holds 1/6, 1/12 and 1/24, which binary floating point cannot
+    represent, so no choice of inputs makes the filter transform exact."""
+    xs, ws, stride, pad, m, wmul = case
+    g = torch.Generator().manual_seed(7)
+    x = torch.randint(-2, 3, xs, generator=g).to(dtype)
+    w = (torch.randint(-2, 3, ws, generator=g) * wmul).to(dtype)
+    ref = _conv64(x, w, None, stride, pad)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, stride, pad, m)
+    assert torch.equal(y.double().cpu(), ref)
+
+
+def test_reference_statistic(dev):
+    """The reference's own accuracy statistic mean(|(y - y64) / y64|) on U(0,1) data at its own
+    shapes (example.py:99-119); recorded for continuity, bounded loosely."""
+    for xs, ws in [((1, 224, 10, 10), (32, 224, 7, 7)), ((1, 32, 10, 10, 10), (32, 32, 3, 3, 3))]:
+        x, w, _ = _data(xs, ws, torch.float32, uniform=True)
+        ref = _conv64(x, w, None, 1, 0)
+        y = engine.conv_forward(x.to(dev), w.to(dev), None, 1, 0, 2)
+        assert float(((y.double().cpu() - ref) / ref).abs().mean()) < 1e-5
+        yh = engine.conv_forward(x.half().to(dev), w.half().to(dev), None, 1, 0, 2)
+        refh = _conv64(x.half(), w.half(), None, 1, 0)
+        assert float(((yh.double().cpu() - refh) / refh).abs().mean()) < 5e-3
+
+
+@pytest.mark.parametrize("chunk", [1, 2, 5])
+def test_chunking_is_invisible(dev, chunk):
+    xs, ws = (5, 32, 20, 20), (32, 32, 3, 3)
+    x, w, b = _data(xs, ws, torch.float16)
+    y0 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, 1, 4, chunk_images=0)
+    y1 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, 1, 4, chunk_images=chunk)
+    assert torch.equal(y0, y1)
+
+
+def test_channels_last_input_and_cached_filter(dev):
+    xs, ws = (2, 32, 20, 20), (32, 32, 3, 3)
+    x, w, b = _data(xs, ws, torch.float16)
+    xd = x.to(dev)
+    y0 = engine.conv_forward(xd, w.to(dev), b.to(dev), 1, 1, 4)
+    xcl = xd.contiguous(memory_format=torch.channels_last)
+    U = engine.transform_filter(w.to(dev), xs, 1, 1, 4)
+    y1 = engine.conv_forward(xcl, w.to(dev), b.to(dev), 1, 1, 4, U=U)
+    assert torch.equal(y0, y1)
+    assert y1.is_contiguous(memory_format=torch.channels_last)

@@ -1,0 +1,185 @@
+"""Parity of every HIP stage (called through the C ABI) against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import tiles as otiles
+from oracle import winograd as ow
+from pytorch_winoconv_amd import engine, Split_and_Concat
+
+pytestmark = pytest.mark.gpu
+
+DISC = {torch.float32: "fp32", torch.float16: "fp16"}
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+# ------------------------------------------------------------------ split / concat: bit-exact
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("shape,wshape,m", [
+    ((2, 5, 9, 11), (3, 5, 3, 3), 2),
+    ((1, 70, 8, 8), (3, 70, 3, 3), 2),
+    ((2, 64, 14, 14), (3, 64, 3, 3), 4),
+    ((1, 3, 12, 7), (3, 3, 5, 5), 2),
+    ((2, 6, 6, 7, 9), (3, 6, 3, 3, 3), 2),
+    ((1, 130, 5, 6, 6), (3, 130, 2, 3, 2), 2),
+])
+def test_wino_split_bit_exact(dev, dtype, shape, wshape, m):
+    torch.manual_seed(1)
+    x = torch.randn(*shape).to(dtype)
+    want = torch.from_numpy(otiles.wino_split(x.numpy(), wshape, m))
+    got = Split_and_Concat.wino_split(x.to(dev), wshape, m)
+    assert got.shape == want.shape
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("osize,K,B,m", [
+    ((7, 9), 5, 2, 2), ((8, 8), 70, 1, 2), ((13, 10), 64, 2, 4), ((5, 7, 6), 6, 2, 2), ((4, 4, 5), 130, 1, 2),
+])
+def test_wino_concat_bit_exact(dev, dtype, osize, K, B, m):
+    torch.manual_seed(2)
+    n = [(o + m - 1) // m for o in osize]
+    P = B
+    for v in n:
+        P *= v
+    t = torch.randn(P, K, *([m] * len(osize))).to(dtype)
+    want = torch.from_numpy(otiles.wino_concat(t.numpy(), osize, m))
+    got = Split_and_Concat.wino_concat(t.to(dev), osize, m)
+    assert got.shape == want.shape
+    assert torch.equal(got.cpu(), want)
+
+
+# ------------------------------------------------------------------ transforms and GEMM
+CASES = [
+    # x shape, w shape, stride, pad, m
+    ((2, 8, 9, 11), (12, 8, 3, 3), 1, 1, 2),
+    ((2, 8, 9, 11), (12, 8, 3, 3), 1, 1, 4),
+    ((1, 3, 10, 10), (5, 3, 3, 3), 1, 0, 2),
+    ((2, 16, 12, 13), (8, 16, 5, 5), 1, 2, 2),
+    ((1, 8, 12, 12), (8, 8, 7, 7), 1, 3, 2),
+    ((2, 8, 12, 13), (8, 8, 3, 3), 2, 1, 2),
+    ((1, 8, 15, 14), (4, 8, 7, 7), 2, 3, 2),
+    ((2, 8, 6, 9, 11), (8, 8, 3, 3, 3), 1, 1, 2),
+    ((1, 4, 7, 9, 8), (4, 4, 5, 5, 5), 1, 2, 2),
+    ((1, 6, 6, 8, 8), (5, 6, 2, 3, 1), 1, 0, 2),
+]
+
+
+def _setup(case, dtype, dev, seed=0, integer=False):
+    xs, ws, stride, pad, m = case
+    g = torch.Generator().manual_seed(seed)
+    if integer:
+        x = torch.randint(-3, 4, xs, generator=g).float()
+        w = torch.randint(-2, 3, ws, generator=g).float()
+    else:
+        x = torch.randn(*xs, generator=g)
+        fan_in = 1
+        for v in ws[1:]:
+            fan_in *= v
+        w = torch.randn(*ws, generator=g) * (2.0 / fan_in) ** 0.5
+    x, w = x.to(dtype), w.to(dtype)
+    stages = {}
+    ow.dwm_conv(x, w, None, stride, pad, m, DISC[dtype], stages)
+    desc = engine.make_desc(xs, ws, dtype, stride, pad, m)
+    plan = engine.plan_conv(desc)
+    return x, w, stages, desc, plan
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_plan_matches_oracle(dev, dtype, case):
+    _, _, stages, desc, plan = _setup(case, dtype, dev)
+    op = stages["plan"]
+    assert plan.t_total == op["T_total"] and plan.n_pieces == len(op["pieces"])
+    for i, pc in enumerate(op["pieces"]):
+        assert [a[0] for a in pc["axes"]] == list(plan.piece[i].tap0)
+        assert [a[2] for a in pc["axes"]] == list(plan.piece[i].r)
+        assert pc["t_offset"] == plan.piece[i].t_offset
+    out, grid = engine.out_dims(desc)
+    assert out == op["odims"] and grid == op["grid"]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_filter_transform(dev, dtype, case):
+    x, w, stages, desc, plan = _setup(case, dtype, dev)
+    U = engine.filter_transform(desc, plan, w.to(dev))
+    C = desc.C
+    assert torch.count_nonzero(U[:, :, C:]) == 0          # channel padding is zero
+    tol = 2e-6 if dtype == torch.float32 else 1.5e-3      # fp16: one rounding of a value <= a few ulp
+    assert _rel(U[:, :, :C], stages["U"]) <= tol
+    # the reference's (kD, kH, kW, C, K) filter layout (dwm.py:85,133) through strides
+    w5 = w.to(dev) if w.dim() == 5 else w.to(dev).unsqueeze(2)
+    w_ref_layout = w5.permute(2, 3, 4, 1, 0).contiguous().permute(4, 3, 0, 1, 2)
+    if w.dim() == 4:
+        w_ref_layout = w_ref_layout[:, :, 0]
+    U2 = engine.filter_transform(desc, plan, w_ref_layout)
+    assert torch.equal(U, U2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_input_transform(dev, dtype, case):
+    x, w, stages, desc, plan = _setup(case, dtype, dev)
+    V = engine.input_transform(desc, plan, engine.channel_last(x.to(dev)))
+    C = desc.C
+    assert torch.count_nonzero(V[:, :, C:]) == 0
+    tol = 2e-6 if dtype == torch.float32 else 1.5e-3
+    assert _rel(V[:, :, :C], stages["V"]) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_input_transform_integer_exact(dev, dtype, case):
+    """BT of F(2,r) and F(4,3) is integer: small integer inputs give bit-identical V."""
+    x, w, stages, desc, plan = _setup(case, dtype, dev, integer=True)
+    V = engine.input_transform(desc, plan, engine.channel_last(x.to(dev)))
+    assert torch.equal(V[:, :, :desc.C].cpu(), stages["V"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("T,P,C,K", [
+    (4, 100, 32, 64), (16, 784, 64, 64), (3, 300, 96, 40), (2, 257, 160, 130), (36, 512, 256, 256),
+    (1, 31, 32, 3), (5, 1000, 64, 512),
+])
+def test_batched_gemm(dev, dtype, T, P, C, K):
+    g = torch.Generator().manual_seed(3)
+    V = (torch.randn(T, P, C, generator=g)).to(dtype)
+    U = (torch.randn(T, K, C, generator=g) / C ** 0.5).to(dtype)
+    want = torch.bmm(V.double(), U.double().transpose(1, 2))
+    M = engine.batched_gemm(V.to(dev), U.to(dev))
+    assert M.shape[2] % 8 == 0
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert _rel(M[:, :, :K], want) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_batched_gemm_integer_exact(dev, dtype):
+    g = torch.Generator().manual_seed(4)
+    V = torch.randint(-4, 5, (6, 333, 64), generator=g).to(dtype)
+    U = torch.randint(-3, 4, (6, 72, 64), generator=g).to(dtype)
+    want = torch.bmm(V.double(), U.double().transpose(1, 2))
+    M = engine.batched_gemm(V.to(dev), U.to(dev))
+    assert torch.equal(M[:, :, :72].double().cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_output_transform(dev, dtype, case, with_bias):
+    x, w, stages, desc, plan = _setup(case, dtype, dev)
+    Mo = stages["M"]
+    K = desc.K
+    ldm = engine._lib.load().wc_padded_channels8(K)
+    M = torch.full((Mo.shape[0], Mo.shape[1], ldm), float("nan"), dtype=dtype)
+    M[:, :, :K] = Mo
+    bias = torch.randn(K).to(dtype) if with_bias else None
+    op = stages["plan"]
+    want = ow.output_transform(Mo, op["pieces"], desc.N, op["grid"], op["odims"], bias, DISC[dtype])
+    got = engine.output_transform(desc, plan, M.to(dev), None if bias is None else bias.to(dev), desc.N)
+    assert got.shape == want.shape
+    tol = 2e-6 if dtype == torch.float32 else 1.5e-3
+    assert _rel(got, want) <= tol
