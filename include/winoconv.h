@@ -141,8 +141,8 @@ int wc_output_transform(const wc_conv_desc* desc, const wc_plan* plan,
 /* Replaces DWM<T> (pybind/extern.hpp:7-9, src/winograd_conv.cpp:17-127) and
  * convLauncherStrideOneLarge<T> (src/base_conv_launchers.cu:282-399).
  * The workspace holds U, V and M (the reference's tmp_weight_buffer, tmp_input_buffer,
- * tmp_product_buffer: dwm.py:122-125); images are processed in chunks so that V and M of
- * one chunk stay cache resident.  `U_cached` (may be NULL) is a filter already transformed
+ * tmp_product_buffer: dwm.py:122-125); images are processed in chunks that bound the size
+ * of V and M.  `U_cached` (may be NULL) is a filter already transformed
  * by wc_filter_transform; `w` may then be NULL. */
 int wc_conv_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
 int wc_conv_u_elems(const wc_conv_desc* desc, size_t* elems);

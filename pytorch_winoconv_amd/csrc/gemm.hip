@@ -48,12 +48,13 @@ struct GemmArgs {
   long long sV, sU, sM;     // batch strides in elements
   int tiles_p, tiles_k, T;
   int n_blocks, per_xcd;
+  int dbg;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
 
 template <typename T, int WM, int WN, int BK>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
   using MF = Mfma<T>;
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int EPC = 16 / sizeof(T);              // elements per 16-byte chunk
@@ -126,45 +127,62 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g) {
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
-    if (kt + 1 < nk) gload(kt + 1);
+    if (kt + 1 < nk && !(g.dbg & 2)) gload(kt + 1);
     const T* st = lds + cur * STAGE;
-#pragma unroll
-    for (int kk = 0; kk < BK / MF::kstep; ++kk) {
-      typename MF::Frag xf[WM], wf[WN];
+    // fragments of step kk+1 are read from LDS while the MFMAs of step kk run
+    constexpr int KK = BK / MF::kstep;
+    typename MF::Frag xf[2][WM], wf[2][WN];
+    auto fload = [&](int kk, int b) {
 #pragma unroll
       for (int i = 0; i < WM; ++i)
-        xf[i] = *reinterpret_cast<const typename MF::Frag*>(st + xoff + i * 32 * LDS_STRIDE + kk * MF::kstep);
+        xf[b][i] = *reinterpret_cast<const typename MF::Frag*>(st + xoff + i * 32 * LDS_STRIDE + kk * MF::kstep);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
-        wf[j] = *reinterpret_cast<const typename MF::Frag*>(st + woff + j * 32 * LDS_STRIDE + kk * MF::kstep);
+        wf[b][j] = *reinterpret_cast<const typename MF::Frag*>(st + woff + j * 32 * LDS_STRIDE + kk * MF::kstep);
+    };
+    fload(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) fload(kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);   // keep the LDS reads above ahead of the MFMAs below
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[j], xf[i], acc[i][j]);
+        for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[kk & 1][j], xf[kk & 1][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (kt + 1 < nk) lstore(cur ^ 1);
     __syncthreads();
   }
 
-  // accumulator (i, j), register 4g + e: output channel 32j + 8g + 4*lhi + e of tile row 32i + l32
-  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
+  // Epilogue through LDS so that global stores are whole rows.  Accumulator (i, j), register
+  // 4q + e holds output channel 32j + 8q + 4*lhi + e of tile row 32i + l32.
+  constexpr int CS = BN + EPC;                     // padded row of the staged output tile
+  T* cs = lds;   // operand stages are free after the last barrier; the launch sizes LDS for both uses
 #pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    const int p = p0 + wp * WM * 32 + i * 32 + l32;
-    if (p >= g.P) continue;
-    T* row = Mt + (long long)p * g.ldm;
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int kc = k0 + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi;
-        if (kc < g.ldm) {
-          Pack<T, 4> o;
+        Pack<T, 4> o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
-          *reinterpret_cast<Pack<T, 4>*>(row + kc) = o;
-        }
+        for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
+        *reinterpret_cast<Pack<T, 4>*>(cs + (wp * WM * 32 + i * 32 + l32) * CS + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi) = o;
       }
+  __syncthreads();
+  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
+  constexpr int CPRO = BN / EPC;                   // 16-byte chunks per output row
+  constexpr int RPPO = 256 / CPRO;                 // rows per pass
+  static_assert(256 % CPRO == 0 && BM % RPPO == 0, "output tile shape");
+  const int orow = tid / CPRO, ocol = (tid % CPRO) * EPC;
+  if (!(g.dbg & 1) && k0 + ocol < g.ldm) {
+#pragma unroll
+    for (int r = 0; r < BM / RPPO; ++r) {
+      const int row = orow + r * RPPO;
+      if (p0 + row < g.P)
+        *reinterpret_cast<Chunk16*>(Mt + (long long)(p0 + row) * g.ldm + k0 + ocol) =
+            *reinterpret_cast<const Chunk16*>(cs + row * CS + ocol);
     }
   }
 }
@@ -180,21 +198,28 @@ struct GemmConfig {
 template <typename T, int WM, int WN, int BK>
 static GemmConfig make_config() {
   constexpr int EPC = 16 / sizeof(T);
+  constexpr size_t stages = (size_t)2 * (64 * WM + 64 * WN) * (BK + EPC) * sizeof(T);
+  constexpr size_t out_tile = (size_t)64 * WM * (64 * WN + EPC) * sizeof(T);
   return GemmConfig{&gemm_kernel<T, WM, WN, BK>, 64 * WM, 64 * WN, BK,
-                    (size_t)2 * (64 * WM + 64 * WN) * (BK + EPC) * sizeof(T)};
+                    stages > out_tile ? stages : out_tile};
 }
 
 // Tile shapes, largest first.  All keep LDS at or below 64 KB.
 template <typename T> struct Configs;
 template <> struct Configs<half_t> {
-  static constexpr int n = 5;
+  static constexpr int n = 10;
   static GemmConfig get(int i) {
     switch (i) {
       case 0: return make_config<half_t, 4, 2, 32>();   // 256 x 128
       case 1: return make_config<half_t, 2, 2, 32>();   // 128 x 128
       case 2: return make_config<half_t, 4, 1, 32>();   // 256 x 64
       case 3: return make_config<half_t, 2, 1, 32>();   // 128 x 64
-      default: return make_config<half_t, 1, 1, 32>();  // 64 x 64
+      case 4: return make_config<half_t, 1, 1, 32>();   // 64 x 64
+      case 5: return make_config<half_t, 2, 2, 64>();
+      case 6: return make_config<half_t, 4, 2, 64>();
+      case 7: return make_config<half_t, 4, 4, 32>();
+      case 8: return make_config<half_t, 4, 4, 64>();
+      default: return make_config<half_t, 2, 4, 64>();
     }
   }
 };
@@ -220,12 +245,13 @@ static GemmConfig choose(int T_, int P, int K) {
     const int i = std::atoi(force);
     if (i >= 0 && i < Configs<T>::n) return Configs<T>::get(i);
   }
-  GemmConfig best = Configs<T>::get(Configs<T>::n - 1);
-  for (int i = 0; i < Configs<T>::n; ++i) {
+  constexpr int n_auto = 5;
+  GemmConfig best = Configs<T>::get(n_auto - 1);
+  for (int i = 0; i < n_auto; ++i) {
     GemmConfig c = Configs<T>::get(i);
     if (c.bn > 64 && c.bn / 2 >= K) continue;                 // half of the tile would be padding
     const long long blocks = (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_;
-    if (blocks >= 512 || i == Configs<T>::n - 1) { best = c; break; }
+    if (blocks >= 512 || i == n_auto - 1) { best = c; break; }
   }
   return best;
 }
@@ -249,8 +275,13 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");
+  WC_CHECK_ARG(Cp % c.bk == 0, "wc_batched_gemm: tile depth %d does not divide %d", c.bk, Cp);
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
+  { const char* e = std::getenv("WINOCONV_DBG"); g.dbg = e ? std::atoi(e) : 0; }
+  if (c.lds > 64 * 1024)
+    WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(256), c.lds, as_stream(stream), g);
   WC_CHECK_LAUNCH("gemm_kernel");
   return WC_OK;

@@ -14,8 +14,16 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   const int Cp = wc_padded_channels(d->C);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
   const bool flat = plan->m[0] == 1;
-  const int vmax = flat ? 4 : 2;
-  const int vec = (d->C % vmax == 0) ? vmax : 1;
+  // Channels per thread.  Measured on MI355X at N=64, C=256, 56x56 fp16: F(4,3) tiles (36 live
+  // elements per channel) run best with 2 channels per thread (more wavefronts in flight),
+  // F(2,r) tiles with 16-byte accesses; 3-D tiles (up to 64 elements) use 2.
+  int want;
+  if (!flat) want = 2;
+  else if (plan->m[1] == 4) want = 2;
+  else want = d->dtype == WC_F16 ? 8 : 4;
+  int vec = 1;
+  for (int v = want; v > 1; v /= 2)
+    if (d->C % v == 0) { vec = v; break; }
   for (int s = 0; s < plan->n_pieces; ++s) {
     const wc_piece& pc = plan->piece[s];
     int k[3];

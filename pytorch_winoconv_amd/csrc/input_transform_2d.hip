@@ -15,7 +15,12 @@ static InKernel pick2d(int k1, int k2) {
 }
 
 InKernel pick_in_2d(int dtype, int k1, int k2, int vec) {
-  if (dtype == WC_F16) return vec == 4 ? pick2d<half_t, 4>(k1, k2) : pick2d<half_t, 1>(k1, k2);
+  if (dtype == WC_F16) {
+    if (vec == 8) return pick2d<half_t, 8>(k1, k2);
+    if (vec == 2) return pick2d<half_t, 2>(k1, k2);
+    return vec == 4 ? pick2d<half_t, 4>(k1, k2) : pick2d<half_t, 1>(k1, k2);
+  }
+  if (vec == 2) return pick2d<float, 2>(k1, k2);
   return vec == 4 ? pick2d<float, 4>(k1, k2) : pick2d<float, 1>(k1, k2);
 }
 

@@ -46,26 +46,31 @@ __global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
   const bool c_ok = c < a.C;
   const T* x = static_cast<const T*>(a.x);
 
+  // Every load is issued unconditionally from a clamped address and zeroed afterwards if the
+  // window element lies outside the image: the loads of a tile are then all in flight together
+  // instead of one per divergent branch.
   float d[A0 * A1 * A2][VEC];
+  const int cc = c_ok ? c : 0;
   static_for<0, A0>([&](auto i0_) {
     constexpr int i0 = decltype(i0_)::value;
     const int z = a.step * (m0 * td + i0) + a.base0;
     const bool z_ok = c_ok && (unsigned)z < (unsigned)a.D;
+    const int zc = min(max(z, 0), a.D - 1);
     static_for<0, A1>([&](auto i1_) {
       constexpr int i1 = decltype(i1_)::value;
       const int yy = a.step * (m1 * th + i1) + a.base1;
       const bool y_ok = z_ok && (unsigned)yy < (unsigned)a.H;
-      const long long row = ((b * a.D + z) * a.H + yy) * a.W;
+      const int yc = min(max(yy, 0), a.H - 1);
+      const long long row = ((b * a.D + zc) * a.H + yc) * a.W;
       static_for<0, A2>([&](auto i2_) {
         constexpr int i2 = decltype(i2_)::value;
         constexpr int e = (i0 * A1 + i1) * A2 + i2;
         const int xx = a.step * (m2 * tw + i2) + a.base2;
-        if (y_ok && (unsigned)xx < (unsigned)a.W) {
-          load_pack<T, VEC>(x + (row + xx) * a.C + c, d[e]);
-        } else {
+        const bool ok = y_ok && (unsigned)xx < (unsigned)a.W;
+        const int xc = min(max(xx, 0), a.W - 1);
+        load_pack<T, VEC>(x + (row + xc) * a.C + cc, d[e]);
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) d[e][v] = 0.f;
-        }
+        for (int v = 0; v < VEC; ++v) d[e][v] = ok ? d[e][v] : 0.f;
       });
     });
   });
