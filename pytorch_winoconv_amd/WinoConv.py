@@ -1,0 +1,93 @@
+"""The `Wino` function object of the reference (reference: WinoConv.py:8-229, whose code is
+stale: it names `tf`, an undefined `A` and `fp16`) and the modules that give the patched
+nn.Conv2d / nn.Conv3d of the reference (conv.py:324-339, 465-480) a working form.
+
+Routing rule of the modules: groups == 1 and dilation == 1 are required for the Winograd
+path; 3x3(x3) stride-1 kernels use plain Winograd (output tile 4 in 2-D, 2 in 3-D), larger
+kernels and stride 2 use the DWM decomposition; anything else falls back to
+torch.nn.functional.conv2d/conv3d like the reference does (conv.py:326-332).  The transformed
+filter is cached and recomputed only when the weight changes.
+"""
+import torch
+from torch import nn
+import torch.nn.functional as F
+
+from . import engine, matrix_conv, matrix_conv3d
+
+
+class Wino:
+    """conv32 / conv16 as methods (reference: WinoConv.py:43-109)."""
+
+    def __init__(self):
+        self.input = None
+        self.kernel = None
+        self.m = 0
+        self.r = 0
+
+    matrix_alloc = staticmethod(matrix_conv.matrix_alloc)
+
+    def _mod(self, input):
+        return matrix_conv if input.dim() == 4 else matrix_conv3d
+
+    def conv16(self, input, kernel, bias=None, stride=1, padding=0, groups=1, output_block=2):
+        return self._mod(input).conv16(input, kernel, bias, stride, padding, groups, output_block)
+
+    def conv32(self, input, kernel, bias=None, stride=1, padding=0, groups=1, output_block=2):
+        return self._mod(input).conv32(input, kernel, bias, stride, padding, groups, output_block)
+
+    def conv(self, input, kernel, output_block, stride, fp16=False):
+        return self._mod(input).conv(input, kernel, output_block, stride, fp16)
+
+
+class _WinoConvNd(nn.Module):
+    nd = 2
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, output_block=None, device=None, dtype=None):
+        super().__init__()
+        tup = lambda v: (v,) * self.nd if isinstance(v, int) else tuple(v)
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = tup(kernel_size), tup(stride)
+        self.padding, self.dilation, self.groups = tup(padding), tup(dilation), groups
+        self.output_block = output_block
+        self.weight = nn.Parameter(torch.empty((out_channels, in_channels // groups) + self.kernel_size,
+                                               device=device, dtype=dtype))
+        self.bias = nn.Parameter(torch.empty(out_channels, device=device, dtype=dtype)) if bias else None
+        nn.init.kaiming_normal_(self.weight)
+        if self.bias is not None:
+            nn.init.zeros_(self.bias)
+        self._cache = None
+
+    def _winograd_ok(self, x):
+        return (self.groups == 1 and set(self.dilation) == {1} and len(set(self.stride)) == 1
+                and self.stride[0] in (1, 2) and max(self.kernel_size) <= 10 and x.is_cuda
+                and x.dtype in (torch.float16, torch.float32))
+
+    def _tile(self):
+        plain = set(self.kernel_size) == {3} and self.stride[0] == 1
+        if self.output_block is not None:
+            return int(self.output_block)
+        return 4 if (plain and self.nd == 2) else 2
+
+    def forward(self, x):
+        conv = F.conv2d if self.nd == 2 else F.conv3d
+        if not self._winograd_ok(x):
+            return conv(x, self.weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
+        w = self.weight.to(x.dtype)
+        m = self._tile()
+        key = (self.weight._version, self.weight.data_ptr(), tuple(x.shape[2:]), x.dtype, m)
+        if self._cache is None or self._cache[0] != key:
+            U = engine.transform_filter(w.detach(), x.shape, self.stride[0], self.padding, m)
+            self._cache = (key, U)
+        b = None if self.bias is None else self.bias.to(x.dtype)
+        return engine.conv_forward(x, w.detach(), b, self.stride[0], self.padding, m, U=self._cache[1])
+
+
+class WinoConv2d(_WinoConvNd):
+    """nn.Conv2d whose forward runs the Winograd / DWM engine (reference: conv.py:324-339)."""
+    nd = 2
+
+
+class WinoConv3d(_WinoConvNd):
+    """nn.Conv3d whose forward runs the Winograd / DWM engine (reference: conv.py:465-480)."""
+    nd = 3

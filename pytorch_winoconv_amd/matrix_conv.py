@@ -1,0 +1,94 @@
+"""conv32 / conv16 / conv / base_conv32 with the reference's signatures
+(reference: matrix_conv.py:70-254).
+
+The reference expresses the transforms and the product as torch matmuls on tiles produced by
+wino_split; here the same functions run the HIP engine.  Differences: kernels larger than 3
+are decomposed into <= 3x3 pieces (DWM) instead of one large F(2,r) tile built from
+fractional interpolation points (matrix_conv.py:31-40) - the decomposition is the numerically
+better of the two; stride 2 is computed by the engine instead of falling back to
+F.conv2d (matrix_conv.py:71-75,93-95); output_block may be 2, or 4 for 3x3 kernels.
+"""
+import numpy as np
+import torch
+
+from . import engine
+from .Split_and_Concat import wino_split, wino_concat  # noqa: F401  (re-exported like the reference)
+
+# transform tables under the reference's names: A = AT (m x alpha), G (alpha x r), B = BT
+A, G, B = {}, {}, {}
+A[(2, 1)] = np.array([[1., 0.], [0., 1.]])
+G[(2, 1)] = np.array([[1.], [1.]])
+B[(2, 1)] = np.array([[1., 0.], [0., 1.]])
+A[(2, 2)] = np.array([[1., 1., 0.], [0., 1., 1.]])
+G[(2, 2)] = np.array([[1., 0.], [1., 1.], [0., 1.]])
+B[(2, 2)] = np.array([[1., -1., 0.], [0., 1., 0.], [0., -1., 1.]])
+A[(2, 3)] = np.array([[1., 1., 1., 0.], [0., 1., -1., -1.]])
+G[(2, 3)] = np.array([[1., 0., 0.], [.5, .5, .5], [.5, -.5, .5], [0., 0., 1.]])
+B[(2, 3)] = np.array([[1., 0., -1., 0.], [0., 1., 1., 0.], [0., -1., 1., 0.], [0., 1., 0., -1.]])
+A[(4, 3)] = np.array([[1., 1., 1., 1., 1., 0.], [0., 1., -1., 2., -2., 0.],
+                      [0., 1., 1., 4., 4., 0.], [0., 1., -1., 8., -8., 1.]])
+G[(4, 3)] = np.array([[1 / 4., 0., 0.], [-1 / 6., -1 / 6., -1 / 6.], [-1 / 6., 1 / 6., -1 / 6.],
+                      [1 / 24., 1 / 12., 1 / 6.], [1 / 24., -1 / 12., 1 / 6.], [0., 0., 1.]])
+B[(4, 3)] = np.array([[4., 0., -5., 0., 1., 0.], [0., -4., -4., 1., 1., 0.], [0., 4., -4., -1., 1., 0.],
+                      [0., -2., -1., 2., 1., 0.], [0., 2., -1., -2., 1., 0.], [0., 4., 0., -5., 0., 1.]])
+
+
+def matrix_alloc(m, r):
+    """Transform matrices for every axis (reference: matrix_conv.py:42-68); raises instead of
+    sys.exit when a size is not available."""
+    A_, B_, G_ = [], [], []
+    for mi, ri in zip(m, r):
+        if (mi, ri) not in A:
+            raise NotImplementedError("Size Error: F(%d, %d) not implemented yet." % (ri, mi))
+        A_.append(torch.from_numpy(A[(mi, ri)]))
+        B_.append(torch.from_numpy(B[(mi, ri)]))
+        G_.append(torch.from_numpy(G[(mi, ri)]))
+    return A_, B_, G_
+
+
+def _same_stride(stride):
+    s = (stride,) if isinstance(stride, int) else tuple(int(v) for v in stride)
+    if len(set(s)) != 1:
+        raise NotImplementedError("stride must be equal on all axes, got %r" % (stride,))
+    return s[0]
+
+
+def _run(input, kernel, bias, stride, padding, groups, output_block, dtype):
+    if groups != 1:
+        raise NotImplementedError("groups != 1 is not supported")
+    x = input.to(dtype)
+    w = kernel.to(dtype)
+    b = None if bias is None else bias.to(dtype)
+    big = any(int(k) > 3 for k in kernel.shape[2:])
+    s = _same_stride(stride)
+    m = 2 if (big or s != 1) else int(output_block)
+    return engine.conv_forward(x, w, b, s, padding, m)
+
+
+def conv16(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2):
+    """Half-precision Winograd convolution returning float32 (reference: matrix_conv.py:70-90)."""
+    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float16).float()
+
+
+def conv32(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2):
+    """Single-precision Winograd convolution (reference: matrix_conv.py:92-110)."""
+    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float32)
+
+
+def conv(input, kernel, output_block, stride, fp16=False):
+    """VALID stride-1 convolution (reference: matrix_conv.py:112-135)."""
+    dtype = torch.float16 if fp16 else torch.float32
+    out = _run(input, kernel, None, 1, 0, 1, output_block, dtype)
+    return out.float() if fp16 else out
+
+
+def base_conv32(input, kernel, fp16, m, r):
+    """Tile-domain Winograd: tiles (P, C, a_h, a_w) and kernel (K, C, r_h, r_w) -> (P, K, m_h, m_w)
+    (reference: matrix_conv.py:137-254).  Each tile is a complete little VALID convolution
+    problem with exactly one Winograd tile, so it runs through the same engine."""
+    if len(set(m)) != 1:
+        raise NotImplementedError("base_conv32: output tile must be square")
+    if list(input.shape[2:]) != [mi + ri - 1 for mi, ri in zip(m, r)]:
+        raise ValueError("base_conv32: tiles of shape %r do not match F(%r, %r)" % (tuple(input.shape[2:]), m, r))
+    dtype = torch.float16 if fp16 else input.dtype
+    return engine.conv_forward(input.to(dtype), kernel.to(dtype), None, 1, 0, int(m[0])).contiguous()

@@ -1,0 +1,154 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares,
+plans exactly like the reference's table and the oracle, and reports errors by status code
+(no GPU call is made here: every call below returns before its first launch)."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+import pytorch_winoconv_amd as pkg
+from pytorch_winoconv_amd import _lib, engine
+from oracle import split_plan as osp
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LUT = json.load(open(os.path.join(ROOT, "tests", "golden", "split_lut.json")))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "winoconv.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(wc_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert b"gfx950" in _lib.load().wc_version()
+
+
+@pytest.mark.parametrize("key", sorted(LUT))
+def test_wc_plan_dwm_matches_reference_table(key):
+    kd, kh, kw = (int(v) for v in key.split("x"))
+    p = engine.plan_dwm(kd, kh, kw)
+    g = LUT[key]
+    for a, b in [("D_s", "D_start"), ("D_e", "D_end"), ("H_s", "H_start"), ("H_e", "H_end"),
+                 ("W_s", "W_start"), ("W_e", "W_end")]:
+        assert g[a] == p[b], (key, a)
+    o = osp.split_plan(kd, kh, kw)
+    assert p["kernel_stride"] == o["kernel_stride"] and p["T_total"] == o["T_total"]
+
+
+@pytest.mark.parametrize("xs,ws,stride,m", [
+    ((1, 4, 20, 20), (4, 4, 3, 3), 1, 2), ((1, 4, 20, 20), (4, 4, 3, 3), 1, 4),
+    ((1, 4, 20, 20), (4, 4, 7, 7), 1, 2), ((1, 4, 20, 20), (4, 4, 7, 7), 2, 2),
+    ((1, 4, 20, 20), (4, 4, 3, 3), 2, 2), ((1, 4, 20, 20), (4, 4, 10, 9), 2, 2),
+    ((1, 4, 9, 20, 20), (4, 4, 3, 3, 3), 1, 2), ((1, 4, 9, 20, 20), (4, 4, 5, 7, 4), 1, 2),
+])
+def test_wc_plan_conv_matches_oracle(xs, ws, stride, m):
+    desc = engine.make_desc(xs, ws, torch.float16, stride, 1, m)
+    plan = engine.plan_conv(desc)
+    two_d = len(xs) == 4
+    ks = ([1] if two_d else []) + list(ws[2:])
+    pieces, T = osp.conv_pieces(ks, stride, m, degenerate_depth=two_d)
+    assert plan.t_total == T and plan.n_pieces == len(pieces) and plan.tap_step == stride
+    assert list(plan.m) == pieces[0]["ms"]
+    for i, pc in enumerate(pieces):
+        assert list(plan.piece[i].tap0) == [a[0] for a in pc["axes"]]
+        assert list(plan.piece[i].r) == [a[2] for a in pc["axes"]]
+        assert plan.piece[i].t_offset == pc["t_offset"]
+
+
+def test_out_dims_follow_the_reference_arithmetic():
+    """oX = X + 2 pad - kX + 1, nX = (oX + 1) / 2 (src/base_conv_launchers.cu:290-295)."""
+    desc = engine.make_desc((2, 8, 10, 13), (4, 8, 7, 7), torch.float32, 1, 0, 2)
+    out, grid = engine.out_dims(desc)
+    assert out == [1, 4, 7] and grid == [1, 2, 4]
+    desc = engine.make_desc((2, 8, 56, 56), (4, 8, 3, 3), torch.float16, 1, 1, 4)
+    assert engine.out_dims(desc) == ([1, 56, 56], [1, 14, 14])
+    desc = engine.make_desc((2, 8, 112, 112), (4, 8, 7, 7), torch.float16, 2, 3, 2)
+    assert engine.out_dims(desc) == ([1, 56, 56], [1, 28, 28])
+
+
+def test_errors_are_status_codes_with_messages_not_exits():
+    lib = _lib.load()
+    # unsupported: stride 3, tile 4 with a 5x5 kernel, kernel extent 11
+    for kw in (dict(stride=3), dict(m=4, w=(4, 4, 5, 5)), dict(w=(4, 4, 11, 3))):
+        desc = engine.make_desc((1, 4, 20, 20), kw.get("w", (4, 4, 3, 3)), torch.float32,
+                                kw.get("stride", 1), 0, kw.get("m", 2))
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(desc)
+        assert len(lib.wc_last_error()) > 0
+    # bad argument: kernel larger than the padded input
+    desc = engine.make_desc((1, 4, 2, 2), (4, 4, 3, 3), torch.float32, 1, 0, 2)
+    with pytest.raises(ValueError):
+        engine.out_dims(desc)
+    # null pointers are rejected before any launch
+    desc = engine.make_desc((1, 4, 8, 8), (4, 4, 3, 3), torch.float32, 1, 0, 2)
+    plan = engine.plan_conv(desc)
+    null = ctypes.c_void_p(0)
+    assert lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), null, 1, null, null) == _lib.WC_ERR_BAD_ARG
+    assert lib.wc_batched_gemm(null, null, null, 1, 1, 32, 1, 8, 0, null) == _lib.WC_ERR_BAD_ARG
+    assert lib.wc_wino_split2d(null, null, 1, 4, 4, 4, 4, 4, 2, 1, 1, 4, null) == _lib.WC_ERR_BAD_ARG
+    # workspace: missing / too small
+    nbytes = ctypes.c_size_t()
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0 and nbytes.value > 0
+    fake = ctypes.c_void_p(256)   # never dereferenced: the size check fails first
+    strides = (ctypes.c_int64 * 5)(36, 9, 0, 3, 1)
+    rc = lib.wc_conv_forward(ctypes.byref(desc), fake, fake, strides, null, null, fake, null, 0, null)
+    assert rc == _lib.WC_ERR_WORKSPACE
+    rc = lib.wc_conv_forward(ctypes.byref(desc), fake, fake, strides, null, null, fake, fake, 16, null)
+    assert rc == _lib.WC_ERR_WORKSPACE and b"needed" in lib.wc_last_error()
+
+
+def test_workspace_size_is_u_plus_v_plus_m():
+    lib = _lib.load()
+    desc = engine.make_desc((64, 256, 56, 56), (256, 256, 3, 3), torch.float16, 1, 1, 4)
+    nbytes, ue = ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0
+    assert lib.wc_conv_u_elems(ctypes.byref(desc), ctypes.byref(ue)) == 0
+    T, P = 36, 64 * 14 * 14
+    assert ue.value == T * 256 * 256
+    assert nbytes.value == 2 * (T * 256 * 256 + 2 * T * P * 256)
+    desc.chunk_images = 8
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0
+    assert nbytes.value == 2 * (T * 256 * 256 + 2 * T * (P // 8) * 256)
+
+
+def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
+    x = torch.randn(1, 4, 8, 8)
+    w = torch.randn(4, 4, 3, 3)
+    with pytest.raises(ValueError, match="GPU only"):
+        engine.conv_forward(x, w)
+    with pytest.raises(ValueError, match="GPU only"):
+        pkg.wino_split(x, w.shape, 2)
+    with pytest.raises(ValueError):
+        engine.make_desc((1, 4, 8, 8), (4, 5, 3, 3), torch.float32)        # channel mismatch
+    with pytest.raises(NotImplementedError):
+        engine.make_desc((1, 4, 8, 8), (4, 4, 3, 3), torch.float32, stride=(1, 2))
+    with pytest.raises(NotImplementedError):
+        pkg.dwm.dwm2d(x, w, groups=2)
+
+
+def test_reference_names_are_importable():
+    for name in ("AddGPU", "Foo", "WinoSplit", "WinoConcat", "DWM", "add_gpu", "wino_split", "wino_concat",
+                 "winograd_conv", "split_and_concat", "Wino", "Dwm", "WinoConv2d", "WinoConv3d"):
+        assert hasattr(pkg, name), name
+    for mod, names in (("dwm", ("dwm2d", "dwm3d", "dwm2d_", "dwm3d_")),
+                       ("matrix_conv", ("conv16", "conv32", "conv", "base_conv32", "matrix_alloc", "A", "G", "B")),
+                       ("matrix_conv3d", ("conv16", "conv32", "conv", "base_conv32"))):
+        for n in names:
+            assert hasattr(getattr(pkg, mod), n), (mod, n)
+    f = pkg.Foo(); f.setKey(3)
+    assert f.getKey() == 3 and "3" in repr(f)
+
+
+def test_module_tables_equal_oracle_tables():
+    import numpy as np
+    from oracle import cook_toom
+    for key in ((2, 1), (2, 2), (2, 3), (4, 3)):
+        AT, G, BT = cook_toom.matrices(*key)
+        assert np.allclose(pkg.matrix_conv.A[key], AT, atol=1e-16, rtol=0)
+        assert np.allclose(pkg.matrix_conv.G[key], G, atol=1e-16, rtol=0)
+        assert np.allclose(pkg.matrix_conv.B[key], BT, atol=1e-16, rtol=0)

@@ -1,0 +1,159 @@
+"""The reference-shaped Python API (dwm, matrix_conv, matrix_conv3d, backend, modules) on the GPU,
+checked against fp64 torch convolution and the oracle.  Tolerances as in test_gpu_conv.py."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import pytorch_winoconv_amd as pkg
+from oracle import winograd as ow
+
+pytestmark = pytest.mark.gpu
+
+
+def _nerr(y, ref):
+    return float((y.double().cpu() - ref).abs().max() / ref.abs().max())
+
+
+def _mk(xs, ws, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    fan = 1
+    for v in ws[1:]:
+        fan *= v
+    return (torch.randn(*xs, generator=g), torch.randn(*ws, generator=g) * (2.0 / fan) ** .5,
+            torch.randn(ws[0], generator=g))
+
+
+def test_dwm2d_matches_the_reference_demo(dev):
+    """example.py:99-109: x (1,224,10,10) U(0,1), w (32,224,7,7); mean relative error vs fp64."""
+    g = torch.Generator().manual_seed(0)
+    x, w = torch.rand(1, 224, 10, 10, generator=g), torch.rand(32, 224, 7, 7, generator=g)
+    ref = F.conv2d(x.double(), w.double())
+    y = pkg.dwm.dwm2d(x.to(dev), w.to(dev), None, (1, 1))
+    assert y.shape == ref.shape
+    assert float(((y.double().cpu() - ref) / ref).abs().mean()) < 1e-6
+    y16 = pkg.matrix_conv.conv16(x.to(dev), w.to(dev), None, (1, 1))
+    assert y16.dtype == torch.float32                                     # matrix_conv.py:89
+    ref16 = F.conv2d(x.half().double(), w.half().double())
+    assert float(((y16.double().cpu() - ref16) / ref16).abs().mean()) < 5e-3
+
+
+def test_dwm3d_and_module(dev):
+    x, w, b = _mk((1, 32, 10, 10, 10), (32, 32, 3, 3, 3))                 # example.py:111-113
+    ref = F.conv3d(x.double(), w.double(), b.double())
+    y = pkg.dwm.dwm3d(x.to(dev), w.to(dev), b.to(dev), (1, 1, 1))
+    assert _nerr(y, ref) < 1e-3
+    y2 = pkg.Dwm().forward(x.to(dev), w.to(dev))                          # network.py:33-35
+    assert _nerr(y2, F.conv3d(x.double(), w.double())) < 1e-3
+    assert _nerr(pkg.dwm.dwm3d_(x.to(dev), w.to(dev)), F.conv3d(x.double(), w.double())) < 1e-3
+
+
+@pytest.mark.parametrize("pad", [(1, 2), 2, 0])
+def test_dwm2d_padding_bias_stride(dev, pad):
+    x, w, b = _mk((2, 16, 21, 20), (24, 16, 5, 5))
+    for stride in (1, 2):
+        ref = F.conv2d(x.double(), w.double(), b.double(), stride=stride, padding=pad)
+        y = pkg.dwm.dwm2d(x.to(dev), w.to(dev), b.to(dev), (stride, stride), pad)
+        assert y.shape == ref.shape and _nerr(y, ref) < 1e-3
+    yh = pkg.dwm.dwm2d(x.half().to(dev), w.half().to(dev), b.half().to(dev), (1, 1), pad)
+    refh = F.conv2d(x.half().double(), w.half().double(), b.half().double(), padding=pad)
+    assert yh.dtype == torch.float16 and _nerr(yh, refh) < 2e-2
+
+
+def test_matrix_conv_functions(dev):
+    x, w, b = _mk((2, 16, 18, 17), (8, 16, 3, 3))
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=1)
+    for ob in (2, 4):
+        assert _nerr(pkg.matrix_conv.conv32(x.to(dev), w.to(dev), b.to(dev), (1, 1), (1, 1), 1, ob), ref) < 1e-3
+        y16 = pkg.matrix_conv.conv16(x.to(dev), w.to(dev), b.to(dev), (1, 1), (1, 1), 1, ob)
+        refh = F.conv2d(x.half().double(), w.half().double(), b.half().double(), padding=1)
+        assert y16.dtype == torch.float32 and _nerr(y16, refh) < 2e-2
+    assert _nerr(pkg.matrix_conv.conv(x.to(dev), w.to(dev), 2, 1), F.conv2d(x.double(), w.double())) < 1e-3
+    assert _nerr(pkg.Wino().conv32(x.to(dev), w.to(dev), b.to(dev), 1, (1, 1)), ref) < 1e-3
+    x3, w3, b3 = _mk((1, 8, 7, 10, 9), (8, 8, 3, 3, 3))
+    ref3 = F.conv3d(x3.double(), w3.double(), b3.double(), padding=1)
+    assert _nerr(pkg.matrix_conv3d.conv32(x3.to(dev), w3.to(dev), b3.to(dev), (1, 1, 1), (1, 1, 1)), ref3) < 1e-3
+
+
+def test_split_base_conv_concat_pipeline_like_the_reference(dev):
+    """matrix_conv.conv's own sequence (matrix_conv.py:126-134): wino_split -> base_conv32 ->
+    wino_concat, against the oracle's restatement of that path and fp64 convolution."""
+    x, w, _ = _mk((2, 8, 11, 12), (6, 8, 3, 3))
+    tiles = pkg.wino_split(x.to(dev), w.shape, 2)
+    out = pkg.matrix_conv.base_conv32(tiles, w.to(dev), False, [2, 2], [3, 3])
+    y = pkg.wino_concat(out, [9, 10], 2)
+    ref = F.conv2d(x.double(), w.double())
+    assert y.shape == ref.shape and _nerr(y, ref) < 1e-3
+    assert _nerr(y, ow.matrix_conv(x, w, 2, "fp32").double()) < 1e-5
+    x3, w3, _ = _mk((1, 4, 6, 7, 8), (5, 4, 3, 3, 3))
+    t3 = pkg.wino_split(x3.to(dev), w3.shape, 2)
+    o3 = pkg.matrix_conv3d.base_conv32(t3, w3.to(dev), False, [2, 2, 2], [3, 3, 3])
+    y3 = pkg.wino_concat(o3, [4, 5, 6], 2)
+    assert _nerr(y3, F.conv3d(x3.double(), w3.double())) < 1e-3
+
+
+def test_backend_entry_points_with_reference_layouts(dev):
+    """DWM / WinoSplit / WinoConcat called exactly as dwm2d_ and wino_split call them
+    (dwm.py:122-136, Split_and_Concat.py:42-48,77-80)."""
+    x, w, _ = _mk((2, 8, 12, 13), (6, 8, 5, 5))
+    xd, wd = x.to(dev), w.to(dev)
+    xin = xd.unsqueeze(2).permute(0, 2, 3, 4, 1).contiguous()             # NDHWC
+    win = wd.unsqueeze(2).permute(2, 3, 4, 1, 0).contiguous()             # (kD,kH,kW,C,K)
+    out = torch.zeros(2, 1, 8, 9, 6, device=dev)
+    scratch = torch.zeros(4, device=dev)
+    pkg.DWM(xin, win, out, 1, scratch, scratch, scratch, scratch.long())
+    ref = F.conv2d(x.double(), w.double())
+    assert _nerr(out[:, 0].permute(0, 3, 1, 2), ref) < 1e-3
+    out2 = torch.zeros(2, 1, 4, 5, 6, device=dev)
+    pkg.DWM(xin, win, out2, 2, scratch, scratch, scratch, scratch.long())
+    assert _nerr(out2[:, 0].permute(0, 3, 1, 2), F.conv2d(x.double(), w.double(), stride=2)) < 1e-3
+    # plain 3x3 through DWM: a key the reference's table lacks (base_conv_launchers.h:59-121)
+    w3 = torch.randn(6, 8, 3, 3)
+    out3 = torch.zeros(2, 1, 10, 11, 6, device=dev)
+    pkg.DWM(xin, w3.to(dev).unsqueeze(2).permute(2, 3, 4, 1, 0).contiguous(), out3, 1)
+    assert _nerr(out3[:, 0].permute(0, 3, 1, 2), F.conv2d(x.double(), w3.double())) < 1e-3
+    # tile copies
+    a = xd.permute(0, 2, 3, 1).contiguous()
+    tiles = torch.zeros(2 * 5 * 6, 8, 4, 4, device=dev)
+    pkg.WinoSplit(a, tiles, 0, 4, 4, 2, 0, 5, 6, True)
+    assert torch.equal(tiles, pkg.wino_split(xd, (6, 8, 3, 3), 2))
+    back = torch.zeros(2, 10, 11, 8, device=dev)
+    t2 = torch.randn(2 * 5 * 6, 8, 2, 2, device=dev)
+    pkg.split_and_concat("concat", t2, back, 2, True)
+    assert torch.equal(back.permute(0, 3, 1, 2), pkg.wino_concat(t2, [10, 11], 2))
+    with pytest.raises(ValueError):
+        pkg.WinoSplit(a, torch.zeros(3, device=dev), 0, 4, 4, 2, 0, 5, 6, True)
+    c = pkg.add_gpu(xd, xd)
+    assert torch.equal(c, xd + xd)
+
+
+@pytest.mark.parametrize("k,stride,pad", [(3, 1, 1), (5, 1, 2), (7, 2, 3), (3, 2, 1)])
+def test_winoconv2d_module_routes_and_caches(dev, k, stride, pad):
+    torch.manual_seed(0)
+    mod = pkg.WinoConv2d(16, 24, k, stride, pad, dtype=torch.float16, device=dev)
+    x = torch.randn(2, 16, 20, 20, device=dev).half()
+    ref = F.conv2d(x.double().cpu(), mod.weight.detach().double().cpu(), mod.bias.detach().double().cpu(),
+                   stride=stride, padding=pad)
+    y = mod(x)
+    assert y.shape == ref.shape and _nerr(y, ref) < 2e-2
+    U0 = mod._cache[1]
+    mod(x)
+    assert mod._cache[1] is U0                       # cached filter transform reused
+    with torch.no_grad():
+        mod.weight.mul_(2.0)
+    y2 = mod(x)
+    assert mod._cache[1] is not U0                   # weight changed: recomputed
+    ref2 = F.conv2d(x.double().cpu(), mod.weight.detach().double().cpu(), mod.bias.detach().double().cpu(),
+                    stride=stride, padding=pad)
+    assert _nerr(y2, ref2) < 2e-2
+    # dilation falls back to torch like the reference's cuDNN branch (conv.py:326-332)
+    mod_d = pkg.WinoConv2d(16, 24, 3, 1, 2, dilation=2, dtype=torch.float16, device=dev)
+    yd = mod_d(x)
+    assert yd.shape == (2, 24, 20, 20)
+
+
+def test_winoconv3d_module(dev):
+    torch.manual_seed(0)
+    mod = pkg.WinoConv3d(8, 8, 3, 1, 1, device=dev)
+    x = torch.randn(1, 8, 6, 10, 10, device=dev)
+    ref = F.conv3d(x.double().cpu(), mod.weight.detach().double().cpu(), mod.bias.detach().double().cpu(), padding=1)
+    assert _nerr(mod(x), ref) < 1e-3

@@ -1,0 +1,105 @@
+"""Pins oracle.cook_toom: the transform matrices every other oracle function builds on.
+
+Independent facts used (none is a retyped copy of the generator's formula):
+  * the literal F(2,1), F(2,2), F(2,3) tables of the reference (matrix_conv.py:15-30,
+    matrix_convnd.py:20-27) - typed in here from the textbook definition of each and checked
+    through the FIR identity rather than compared entry by entry with the oracle's copy;
+  * the exact-rational FIR identity  AT . ((G g) o (BT d)) == valid correlation of d with g
+    (what wincnn.filterVerify checks symbolically, wincnn.py:73-87), on basis vectors;
+  * the published Lavin & Gray F(4x4,3x3) matrices, equal to the reference's commented B25 / G25
+    literals (transform.py:29-40);
+  * spot formulas of the reference's unrolled kernels (transform_kernels.cu:1191,1587-1588,
+    transform_kernels_3d.cu:4998).
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from oracle import cook_toom as ct
+
+
+def _fir_identity_exact(AT, G, BT, m, r):
+    alpha = m + r - 1
+    for di in range(alpha):
+        for gi in range(r):
+            d = [Fraction(int(i == di)) for i in range(alpha)]
+            g = [Fraction(int(i == gi)) for i in range(r)]
+            U = [sum(Fraction(G[i][j]) * g[j] for j in range(r)) for i in range(alpha)]
+            V = [sum(Fraction(BT[i][j]) * d[j] for j in range(alpha)) for i in range(alpha)]
+            Y = [sum(Fraction(AT[o][i]) * U[i] * V[i] for i in range(alpha)) for o in range(m)]
+            want = [sum(d[o + j] * g[j] for j in range(r)) for o in range(m)]
+            assert Y == want, (m, r, di, gi)
+
+
+@pytest.mark.parametrize("m,r,points", [
+    (2, 2, (0, 1)), (2, 3, (0, 1, -1)), (4, 3, (0, 1, -1, 2, -2)), (2, 5, (0, 1, -1, 2, -2)),
+    (6, 3, (0, 1, -1, 2, -2, Fraction(1, 2), Fraction(-1, 2))), (2, 4, (0, 1, -1, 2)),
+])
+def test_generator_satisfies_fir_identity_exactly(m, r, points):
+    AT, G, BT = ct.cook_toom_exact(points, m, r)
+    _fir_identity_exact(AT, G, BT, m, r)
+
+
+@pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 3)])
+def test_tables_in_use_satisfy_fir_identity_exactly(m, r):
+    AT, G, BT = ct.matrices(m, r)
+    as_frac = lambda M: [[Fraction(v).limit_denominator(1000) for v in row] for row in M]
+    _fir_identity_exact(as_frac(AT), as_frac(G), as_frac(BT), m, r)
+
+
+def test_f43_is_the_published_lavin_gray_matrix_set():
+    AT, G, BT = ct.matrices(4, 3)
+    # Lavin & Gray, "Fast Algorithms for Convolutional Neural Networks", F(4x4,3x3)
+    BT_pub = [[4, 0, -5, 0, 1, 0], [0, -4, -4, 1, 1, 0], [0, 4, -4, -1, 1, 0],
+              [0, -2, -1, 2, 1, 0], [0, 2, -1, -2, 1, 0], [0, 4, 0, -5, 0, 1]]
+    G_pub = [[1 / 4, 0, 0], [-1 / 6, -1 / 6, -1 / 6], [-1 / 6, 1 / 6, -1 / 6],
+             [1 / 24, 1 / 12, 1 / 6], [1 / 24, -1 / 12, 1 / 6], [0, 0, 1]]
+    AT_pub = [[1, 1, 1, 1, 1, 0], [0, 1, -1, 2, -2, 0], [0, 1, 1, 4, 4, 0], [0, 1, -1, 8, -8, 1]]
+    assert np.array_equal(BT, np.array(BT_pub, dtype=np.float64))
+    assert np.allclose(G, np.array(G_pub), rtol=0, atol=1e-16)
+    assert np.array_equal(AT, np.array(AT_pub, dtype=np.float64))
+
+
+def test_f25_generator_reproduces_the_reference_literals():
+    """F(2,5) over the points (0,1,-1,2,-2) is what the reference generates at import
+    (matrix_conv.py:33); its commented literals A25/G25/B25 (transform.py:27-40) give the
+    expected output of the generator, sign and scaling split included."""
+    AT, G, BT = ct.cook_toom((0, 1, -1, 2, -2), 2, 5)
+    A25 = [[1, 1, 1, 1, 1, 0], [0, 1, -1, 2, -2, 1]]
+    G25 = [[1 / 4, 0, 0, 0, 0], [-1 / 6] * 5, [-1 / 6, 1 / 6, -1 / 6, 1 / 6, -1 / 6],
+           [1 / 24, 1 / 12, 1 / 6, 1 / 3, 2 / 3], [1 / 24, -1 / 12, 1 / 6, -1 / 3, 2 / 3], [0, 0, 0, 0, 1]]
+    B25 = [[4, 0, -5, 0, 1, 0], [0, -4, -4, 1, 1, 0], [0, 4, -4, -1, 1, 0],
+           [0, -2, -1, 2, 1, 0], [0, 2, -1, -2, 1, 0], [0, 4, 0, -5, 0, 1]]
+    assert np.array_equal(AT, np.array(A25, dtype=np.float64))
+    assert np.allclose(G, np.array(G25), rtol=0, atol=1e-16)
+    assert np.array_equal(BT, np.array(B25, dtype=np.float64))
+
+
+def test_kernel_spot_formulas():
+    """Kronecker products of the tables reproduce single lines of the reference's unrolled code."""
+    AT, G, BT = ct.matrices(2, 3)
+    # 2-D input element 0 = d0 - d2 - d8 + d10          (transform_kernels.cu:1191)
+    row = np.kron(BT[0], BT[0])
+    want = np.zeros(16); want[[0, 10]] = 1; want[[2, 8]] = -1
+    assert np.array_equal(row, want)
+    # 3-D input element 0 = d0 + d10 - d2 - d32 + d34 + d40 - d42 - d8   (transform_kernels_3d.cu:4998)
+    row = np.kron(BT[0], np.kron(BT[0], BT[0]))
+    want = np.zeros(64); want[[0, 10, 34, 40]] = 1; want[[2, 32, 42, 8]] = -1
+    assert np.array_equal(row, want)
+    # 2-D output y00 = m0+m1+m2+m4+m5+m6+m8+m9+m10      (transform_kernels.cu:1587-1588)
+    row = np.kron(AT[0], AT[0])
+    want = np.zeros(16); want[[0, 1, 2, 4, 5, 6, 8, 9, 10]] = 1
+    assert np.array_equal(row, want)
+    # filter, r = 3 along W: [g0, (g0+g1+g2)/2, (g0-g1+g2)/2, g2]   (calculation_kernels.cu:26-29)
+    assert np.array_equal(G, np.array([[1, 0, 0], [.5, .5, .5], [.5, -.5, .5], [0, 0, 1]]))
+    # r = 2: input [d0-d1, d1, d2-d1], output [m0+m1, m1+m2]        (calculation_kernels.cu:773-775, 1536-1537)
+    AT2, G2, BT2 = ct.matrices(2, 2)
+    assert np.array_equal(BT2, np.array([[1, -1, 0], [0, 1, 0], [0, -1, 1]]))
+    assert np.array_equal(AT2, np.array([[1, 1, 0], [0, 1, 1]]))
+    assert np.array_equal(G2, np.array([[1, 0], [1, 1], [0, 1]]))
+
+
+def test_unsupported_pair_is_rejected():
+    with pytest.raises(ValueError):
+        ct.matrices(3, 3)
