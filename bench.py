@@ -32,9 +32,10 @@ sys.path.insert(0, ROOT)
 
 N, C, K, H, W, R, PAD, M_TILE = 64, 256, 256, 56, 56, 3, 1, 4
 MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
-# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/gemm_f16_n64_c256_56x56.md for the runs and the copy-kernel scale factors).
-GEMM_HBM_TRAFFIC_BYTES = None
+# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116734 KiB, x2.00 by the copy
+# probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
+# profiles/conv3x3_f16_n64_c256_56x56_all_kernels.md.
+GEMM_HBM_TRAFFIC_BYTES = int((116734 * 2.0 + 225792 * 1.0) * 1024)
 
 
 def synthetic(n):
@@ -75,6 +76,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three 128 MiB device-to-device copies before the timed region "
+                         "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this engine is a single-GPU operator with no collectives; it is "
@@ -117,6 +121,11 @@ def main():
         _lib.check(lib.wc_output_transform(d_, p_, pM, None, N, py, st))
         if ev: ev[4].record()
 
+    if args.copy_probe:
+        src = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
