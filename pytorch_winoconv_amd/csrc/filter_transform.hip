@@ -7,11 +7,81 @@
 // reduction axis C innermost and zero-padded to Cp so that the batched GEMM reads both of
 // its operands along contiguous rows (the reference keeps (T, C, K): split_kernel.cu:51).
 // Arithmetic in fp32, one rounding to the storage type.  Tiny (K*C*T outputs); run once per
-// weight update by callers that cache U.
-#include "wc_common.h"
-#include "wc_tables.h"
+// weight update by callers that cache U.  Single-piece plans of the common shapes take a
+// compile-time kernel (taps loaded once per (k, c)); anything else the generic one.
+#include "wc_transform.h"
 
 namespace wc {
+
+// G of one kind as an apply_axis matrix (alpha x r)
+template <int KIND>
+struct MatG {
+  static constexpr int rows = Mats<KIND>::alpha;
+  static constexpr int cols = Mats<KIND>::r;
+  __host__ __device__ static constexpr float get(int i, int j) { return Mats<KIND>::g(i, j); }
+  __host__ __device__ static constexpr int first_nz(int i) {
+    for (int j = 0; j < cols; ++j)
+      if (get(i, j) != 0.f) return j;
+    return cols;
+  }
+};
+
+struct FilterFastArgs {
+  const void* w;
+  void* U;
+  long long s[5];
+  int C, Cp, K;
+  int tap0[3];
+  int step;
+  int t_offset;
+};
+
+// Single piece with compile-time kinds: one thread per (k, c) loads its taps once, transforms
+// in registers and writes the alpha^d elements with lanes along c (coalesced rows of U).
+template <typename T, int K0, int K1, int K2>
+__global__ __launch_bounds__(256) void filter_transform_fast_kernel(const FilterFastArgs a) {
+  constexpr int R0 = Mats<K0>::r, R1 = Mats<K1>::r, R2 = Mats<K2>::r;
+  constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.K * a.Cp) return;
+  const int c = idx % a.Cp, k = idx / a.Cp;
+  T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + idx;
+  const long long plane = (long long)a.K * a.Cp;
+  float g[R0 * R1 * R2][1];
+  const bool ok = c < a.C;
+  const T* w = static_cast<const T*>(a.w) + k * a.s[0] + (ok ? c : 0) * a.s[1];
+  static_for<0, R0>([&](auto j0_) {
+    static_for<0, R1>([&](auto j1_) {
+      static_for<0, R2>([&](auto j2_) {
+        constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
+        const float v = static_cast<float>(w[(a.tap0[0] + j0 * a.step) * a.s[2] +
+                                            (a.tap0[1] + j1 * a.step) * a.s[3] +
+                                            (a.tap0[2] + j2 * a.step) * a.s[4]]);
+        g[(j0 * R1 + j1) * R2 + j2][0] = ok ? v : 0.f;
+      });
+    });
+  });
+  float u2[R0 * R1 * A2][1];
+  apply_axis<MatG<K2>, 2, R0, R1, R2, 1>(g, u2);
+  float u1[R0 * A1 * A2][1];
+  apply_axis<MatG<K1>, 1, R0, R1, A2, 1>(u2, u1);
+  float u0[A0 * A1 * A2][1];
+  apply_axis<MatG<K0>, 0, R0, A1, A2, 1>(u1, u0);
+  static_for<0, A0 * A1 * A2>([&](auto e_) {
+    constexpr int e = decltype(e_)::value;
+    U[e * plane] = static_cast<T>(u0[e][0]);
+  });
+}
+
+using FilterFastKernel = void (*)(FilterFastArgs);
+
+template <typename T>
+static FilterFastKernel pick_fast(int k0, int k1, int k2) {
+  if (k0 == KIND_11 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_11, KIND_43, KIND_43>;
+  if (k0 == KIND_11 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_11, KIND_23, KIND_23>;
+  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_23, KIND_23, KIND_23>;
+  return nullptr;
+}
 
 struct FilterArgs {
   const void* w;
@@ -75,6 +145,25 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   int rc = wc_conv_out_dims(d, out, grid);   // validates the descriptor
   if (rc) return rc;
   WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_filter_transform: bad plan");
+  if (plan->n_pieces == 1) {
+    const wc_piece& pc = plan->piece[0];
+    const int k0 = kind_of(plan->m[0], pc.r[0]), k1 = kind_of(plan->m[1], pc.r[1]), k2 = kind_of(plan->m[2], pc.r[2]);
+    FilterFastKernel fn = d->dtype == WC_F16 ? pick_fast<half_t>(k0, k1, k2) : pick_fast<float>(k0, k1, k2);
+    if (fn) {
+      FilterFastArgs f;
+      f.w = w; f.U = U;
+      for (int i = 0; i < 5; ++i) f.s[i] = w_strides[i];
+      f.C = d->C; f.Cp = wc_padded_channels(d->C); f.K = d->K;
+      for (int i = 0; i < 3; ++i) f.tap0[i] = pc.tap0[i];
+      f.step = plan->tap_step;
+      f.t_offset = pc.t_offset;
+      const long long n = (long long)d->K * f.Cp;
+      WC_CHECK_ARG(n < (1ll << 31), "wc_filter_transform: problem too large");
+      hipLaunchKernelGGL(fn, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, as_stream(stream), f);
+      WC_CHECK_LAUNCH("filter_transform_fast_kernel");
+      return WC_OK;
+    }
+  }
   FilterArgs a;
   a.w = w; a.U = U;
   for (int i = 0; i < 5; ++i) a.s[i] = w_strides[i];
