@@ -70,12 +70,77 @@ def cpu_baseline(sample_images=32, repeats=3):
     }
 
 
+SUITE = [
+    # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size)
+    ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
+    ("c2 vgg16 fp32 N8 F(2,3) x13", "vgg", None, 1, 1, 2, "f32"),
+    ("c2 vgg16 fp32 N8 F(4,3) x13", "vgg", None, 1, 1, 4, "f32"),
+    ("c3 fp16 N64 C64 56x56 F(4,3)", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 4, "f16"),
+    ("c3 fp16 N64 C128 28x28 F(4,3)", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, "f16"),
+    ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, "f16"),
+    ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
+    ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
+    ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
+]
+VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),
+         (256, 256, 56), (256, 512, 28), (512, 512, 28), (512, 512, 28), (512, 512, 14), (512, 512, 14),
+         (512, 512, 14)]
+
+
+def run_suite(steps=10):
+    """ms per layer (whole forward through the one-call entry point, filter transform included)
+    and direct-convolution-equivalent TFLOP/s for every other benchmark configuration."""
+    import torch
+    from pytorch_winoconv_amd import engine
+    dev = torch.device("cuda:0")
+    out = []
+
+    def one(xs, ws, stride, pad, m, dt):
+        dtype = torch.float16 if dt == "f16" else torch.float32
+        g = torch.Generator().manual_seed(0)
+        fan = 1
+        for v in ws[1:]:
+            fan *= v
+        x = torch.randn(*xs, generator=g).to(dtype).to(dev)
+        x = x.contiguous(memory_format=torch.channels_last if len(xs) == 4 else torch.channels_last_3d)
+        w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype).to(dev)
+        for _ in range(2):
+            y = engine.conv_forward(x, w, None, stride, pad, m)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            engine.conv_forward(x, w, None, stride, pad, m)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        flops = 2.0 * xs[0] * ws[0] * ws[1]
+        for v in list(y.shape[2:]) + list(ws[2:]):
+            flops *= v
+        return ms, flops
+
+    for name, xs, ws, stride, pad, m, dt in SUITE:
+        if xs == "vgg":
+            ms = fl = 0.0
+            for c, k, hw in VGG16:
+                a, b = one((8, c, hw, hw), (k, c, 3, 3), stride, pad, m, dt)
+                ms, fl = ms + a, fl + b
+        else:
+            ms, fl = one(xs, ws, stride, pad, m, dt)
+        out.append({"config": name, "ms": round(ms, 4), "effective_tflops": round(fl / ms / 1e9, 1)})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--suite", action="store_true",
+                    help="also time every other benchmark configuration (adds a 'suite' list)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -181,6 +246,8 @@ def main():
         "ms_per_layer_one_call": ms_one_call,
         "one_call_matches_stages": same,
     }
+    if args.suite:
+        result["suite"] = run_suite()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
