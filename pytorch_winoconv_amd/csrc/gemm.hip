@@ -48,7 +48,6 @@ struct GemmArgs {
   long long sV, sU, sM;     // batch strides in elements
   int tiles_p, tiles_k, T;
   int n_blocks, per_xcd;
-  int dbg;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -127,7 +126,7 @@ __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
-    if (kt + 1 < nk && !(g.dbg & 2)) gload(kt + 1);
+    if (kt + 1 < nk) gload(kt + 1);
     const T* st = lds + cur * STAGE;
     // fragments of step kk+1 are read from LDS while the MFMAs of step kk run
     constexpr int KK = BK / MF::kstep;
@@ -176,7 +175,7 @@ __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
   constexpr int RPPO = 256 / CPRO;                 // rows per pass
   static_assert(256 % CPRO == 0 && BM % RPPO == 0, "output tile shape");
   const int orow = tid / CPRO, ocol = (tid % CPRO) * EPC;
-  if (!(g.dbg & 1) && k0 + ocol < g.ldm) {
+  if (k0 + ocol < g.ldm) {
 #pragma unroll
     for (int r = 0; r < BM / RPPO; ++r) {
       const int row = orow + r * RPPO;
@@ -278,7 +277,6 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(Cp % c.bk == 0, "wc_batched_gemm: tile depth %d does not divide %d", c.bk, Cp);
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
-  { const char* e = std::getenv("WINOCONV_DBG"); g.dbg = e ? std::atoi(e) : 0; }
   if (c.lds > 64 * 1024)
     WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
