@@ -79,10 +79,13 @@ SUITE = [
     ("c3 fp16 N64 C128 28x28 F(4,3)", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16"),
     ("c4 fp16 N32 C128 112x112 3x3 s2 DWM", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
     ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
 ]

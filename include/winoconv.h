@@ -66,7 +66,7 @@ typedef struct {
   int kernel[3];   /* kD, kH, kW (kD = 1 when ndim == 2)                        */
   int pad[3];      /* symmetric zero padding per axis                           */
   int stride;      /* 1 or 2, same on every axis                                */
-  int m;           /* Winograd output tile: 2, or 4 (2-D 3x3 stride 1 only)     */
+  int m;           /* Winograd output tile: 2, or 4 (2-D problems only)         */
   int dtype;       /* wc_dtype                                                  */
   int chunk_images;/* images per pass of wc_conv_forward; 0 = choose automatically */
 } wc_conv_desc;
@@ -86,7 +86,8 @@ const char* wc_last_error(void);
 int wc_plan_dwm(int kD, int kH, int kW, int* num_split,
                 int* D_start, int* D_end, int* H_start, int* H_end,
                 int* W_start, int* W_end, int* kernel_stride, int* t_total);
-/* General plan of a convolution (stride 1 or 2, tile 2 or 4). */
+/* General plan of a convolution (stride 1 or 2; tile 2 with F(2,r) pieces, or tile 4 with
+ * F(4,r) pieces in 2-D). */
 int wc_plan_conv(const wc_conv_desc* desc, wc_plan* plan);
 /* Output extent and tile grid: replaces the shape arithmetic of DWM<T>
  * (src/winograd_conv.cpp:71-90) and of dwm2d_/dwm3d_ (dwm.py:56-61,118-121). */

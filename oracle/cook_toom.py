@@ -101,14 +101,21 @@ _LIT = {
 }
 
 POINTS_F43 = (0, 1, -1, 2, -2)   # same point set the reference uses for F(2,5) (matrix_conv.py:33)
+POINTS_F42 = (0, 1, -1, 2)       # the reference's point set for F(2,4) (matrix_conv.py:32)
+_LIT[(4, 1)] = (                 # one tap: identity, like the reference's F(2,1) literal
+    [[1., 0., 0., 0.], [0., 1., 0., 0.], [0., 0., 1., 0.], [0., 0., 0., 1.]],
+    [[1.], [1.], [1.], [1.]],
+    [[1., 0., 0., 0.], [0., 1., 0., 0.], [0., 0., 1., 0.], [0., 0., 0., 1.]])
 
 
 def matrices(m, r):
-    """(AT, G, BT) float64 for F(m, r).  F(2,1..3) literal, F(4,3) Cook-Toom."""
+    """(AT, G, BT) float64 for F(m, r).  F(2,1..3) and F(4,1) literal, F(4,2), F(4,3) Cook-Toom."""
     if (m, r) in _LIT:
         AT, G, BT = _LIT[(m, r)]
         return (np.array(AT, dtype=np.float64), np.array(G, dtype=np.float64),
                 np.array(BT, dtype=np.float64))
     if (m, r) == (4, 3):
         return cook_toom(POINTS_F43, 4, 3)
+    if (m, r) == (4, 2):
+        return cook_toom(POINTS_F42, 4, 2)
     raise ValueError("F(%d,%d) not on the hot path" % (m, r))

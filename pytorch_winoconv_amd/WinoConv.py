@@ -3,8 +3,8 @@ stale: it names `tf`, an undefined `A` and `fp16`) and the modules that give the
 nn.Conv2d / nn.Conv3d of the reference (conv.py:324-339, 465-480) a working form.
 
 Routing rule of the modules: groups == 1 and dilation == 1 are required for the Winograd
-path; 3x3(x3) stride-1 kernels use plain Winograd (output tile 4 in 2-D, 2 in 3-D), larger
-kernels and stride 2 use the DWM decomposition; anything else falls back to
+path; 3x3(x3) stride-1 kernels use plain Winograd, larger kernels and stride 2 the DWM
+decomposition (output tile 4 in 2-D, 2 in 3-D); anything else falls back to
 torch.nn.functional.conv2d/conv3d like the reference does (conv.py:326-332).  The transformed
 filter is cached and recomputed only when the weight changes.
 """
@@ -64,10 +64,9 @@ class _WinoConvNd(nn.Module):
                 and x.dtype in (torch.float16, torch.float32))
 
     def _tile(self):
-        plain = set(self.kernel_size) == {3} and self.stride[0] == 1
         if self.output_block is not None:
             return int(self.output_block)
-        return 4 if (plain and self.nd == 2) else 2
+        return 4 if self.nd == 2 else 2
 
     def forward(self, x):
         conv = F.conv2d if self.nd == 2 else F.conv3d

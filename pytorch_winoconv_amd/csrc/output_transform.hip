@@ -9,8 +9,9 @@
 //
 // HBM-bound: a thread owns one tile x VEC consecutive output channels (lanes along K).
 // Two kernels: a separable compile-time one for single-piece plans (F(2,3)^2, F(4,3)^2,
-// F(2,3)^3) and a streaming one for any multi-piece F(2,r) plan, where each loaded element
-// is scattered into the 2^d accumulators with coefficients from a constant table.
+// F(2,3)^3) and a streaming one for any other plan (F(2,r) pieces, or F(4,r) pieces in 2-D),
+// where each loaded tile row is transformed along the width and then scattered into the m^d
+// accumulators with coefficients from a constant table.
 #include "wc_transform.h"
 
 namespace wc {
@@ -107,15 +108,25 @@ __constant__ const float kAT2[4][2][4] = {
     {{1, 1, 1, 0}, {0, 1, -1, -1}},
 };
 
+// A^T of F(4, r) by [r][output a][element i]
+__constant__ const float kAT4[4][4][6] = {
+    {{0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0}},
+    {{1, 0, 0, 0, 0, 0}, {0, 1, 0, 0, 0, 0}, {0, 0, 1, 0, 0, 0}, {0, 0, 0, 1, 0, 0}},
+    {{1, 1, 1, 1, 0, 0}, {0, 1, -1, 2, 0, 0}, {0, 1, 1, 4, 0, 0}, {0, 1, -1, 8, 1, 0}},
+    {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, 0}, {0, 1, 1, 4, 4, 0}, {0, 1, -1, 8, -8, 1}},
+};
+
 struct OutMultiArgs {
   OutArgs o;
   int n_pieces;
   int info[WC_MAX_PIECES];   // t_offset | r0 << 16 | r1 << 20 | r2 << 24 (r0 = 0: flat depth)
 };
 
-template <typename T, bool FLAT, int VEC>
+// MO: output tile extent on the image axes (2, or 4 for 2-D problems); FLAT: one-element depth axis
+template <typename T, bool FLAT, int MO, int VEC>
 __global__ __launch_bounds__(256) void output_multi_kernel(OutMultiArgs g) {
   constexpr int M0 = FLAT ? 1 : 2;
+  static_assert(MO == 2 || (MO == 4 && FLAT), "tile 4 is 2-D only");
   const OutArgs& a = g.o;
   const int blk = xcd_remap(blockIdx.x, a.per_xcd);
   const long long idx = (long long)blk * 256 + threadIdx.x;
@@ -125,40 +136,71 @@ __global__ __launch_bounds__(256) void output_multi_kernel(OutMultiArgs g) {
   const Where w = decode_tile(p, a.nD, a.nH, a.nW);
   const T* M = static_cast<const T*>(a.M) + p * a.ldm + k;
 
-  float acc[M0 * 4][VEC];
+  float acc[M0 * MO * MO][VEC];
 #pragma unroll
-  for (int e = 0; e < M0 * 4; ++e)
+  for (int e = 0; e < M0 * MO * MO; ++e)
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[e][v] = 0.f;
 
   for (int s = 0; s < g.n_pieces; ++s) {
     const int info = g.info[s];
     const int r0 = (info >> 16) & 15, r1 = (info >> 20) & 15, r2 = (info >> 24) & 15;
-    const int n0 = FLAT ? 1 : r0 + 1, n1 = r1 + 1, n2 = r2 + 1;
+    const int n0 = FLAT ? 1 : r0 + 1, n1 = r1 + MO - 1, n2 = r2 + MO - 1;
     const T* Ms = M + (long long)(info & 0xffff) * a.t_stride;
-    for (int i0 = 0; i0 < n0; ++i0)
-      for (int i1 = 0; i1 < n1; ++i1)
-        for (int i2 = 0; i2 < n2; ++i2) {
-          float v[VEC];
-          load_pack<T, VEC>(Ms + (long long)((i0 * n1 + i1) * n2 + i2) * a.t_stride, v);
-          static_for<0, M0>([&](auto a0_) {
-            constexpr int a0 = decltype(a0_)::value;
-            const float c0 = kAT2[r0][a0][i0];
-            static_for<0, 2>([&](auto a1_) {
-              constexpr int a1 = decltype(a1_)::value;
-              const float c01 = c0 * kAT2[r1][a1][i1];
-              static_for<0, 2>([&](auto a2_) {
-                constexpr int a2 = decltype(a2_)::value;
-                const float c = c01 * kAT2[r2][a2][i2];
+    // coefficients of this piece, fetched once (wave-uniform, they live in scalar registers)
+    constexpr int NW = MO + 2;
+    float cH[MO][NW], cW[MO][NW];
 #pragma unroll
-                for (int q = 0; q < VEC; ++q)
-                  acc[(a0 * 2 + a1) * 2 + a2][q] = __builtin_fmaf(c, v[q], acc[(a0 * 2 + a1) * 2 + a2][q]);
-              });
-            });
-          });
+    for (int o = 0; o < MO; ++o)
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        cH[o][i] = MO == 2 ? kAT2[r1][o & 1][i & 3] : kAT4[r1][o][i];
+        cW[o][i] = MO == 2 ? kAT2[r2][o & 1][i & 3] : kAT4[r2][o][i];
+      }
+    // one tile row (up to MO + 2 elements) at a time: all its loads are issued before the first
+    // FMA so that a thread keeps several requests in flight; width pass on the row, then the MO
+    // results are scattered along height / depth
+    for (int i0 = 0; i0 < n0; ++i0) {
+#pragma unroll
+      for (int i1 = 0; i1 < NW; ++i1) {
+        if (i1 < n1) {
+          const T* Mr = Ms + (long long)((i0 * n1 + i1) * n2) * a.t_stride;
+          float v[NW][VEC];
+#pragma unroll
+          for (int i2 = 0; i2 < NW; ++i2)
+            if (i2 < n2) load_pack<T, VEC>(Mr + (long long)i2 * a.t_stride, v[i2]);
+          float rowres[MO][VEC];
+#pragma unroll
+          for (int a2 = 0; a2 < MO; ++a2)
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) rowres[a2][q] = 0.f;
+#pragma unroll
+          for (int i2 = 0; i2 < NW; ++i2) {
+            if (i2 < n2) {
+#pragma unroll
+              for (int a2 = 0; a2 < MO; ++a2)
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) rowres[a2][q] = __builtin_fmaf(cW[a2][i2], v[i2][q], rowres[a2][q]);
+            }
+          }
+#pragma unroll
+          for (int a0 = 0; a0 < M0; ++a0)
+#pragma unroll
+            for (int a1 = 0; a1 < MO; ++a1) {
+              const float c01 = kAT2[r0][a0][i0] * cH[a1][i1];
+              if (c01 != 0.f) {
+#pragma unroll
+                for (int a2 = 0; a2 < MO; ++a2)
+#pragma unroll
+                  for (int q = 0; q < VEC; ++q)
+                    acc[(a0 * MO + a1) * MO + a2][q] = __builtin_fmaf(c01, rowres[a2][q], acc[(a0 * MO + a1) * MO + a2][q]);
+              }
+            }
         }
+      }
+    }
   }
-  write_tile<T, M0, 2, 2, VEC>(a, w, k, acc);
+  write_tile<T, M0, MO, MO, VEC>(a, w, k, acc);
 }
 
 using OutKernel = void (*)(OutArgs);
@@ -179,9 +221,10 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
 }
 
 template <typename T>
-static OutMultiKernel pick_multi(bool flat, int vec) {
-  if (flat) return vec == 4 ? &output_multi_kernel<T, true, 4> : &output_multi_kernel<T, true, 1>;
-  return vec == 4 ? &output_multi_kernel<T, false, 4> : &output_multi_kernel<T, false, 1>;
+static OutMultiKernel pick_multi(bool flat, int m, int vec) {
+  if (flat && m == 4) return vec == 4 ? &output_multi_kernel<T, true, 4, 4> : &output_multi_kernel<T, true, 4, 1>;
+  if (flat) return vec == 4 ? &output_multi_kernel<T, true, 2, 4> : &output_multi_kernel<T, true, 2, 1>;
+  return vec == 4 ? &output_multi_kernel<T, false, 2, 4> : &output_multi_kernel<T, false, 2, 1>;
 }
 
 }  // namespace wc
@@ -226,8 +269,10 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
     WC_CHECK_LAUNCH("output_transform_kernel");
     return WC_OK;
   }
-  if (plan->m[1] != 2 || plan->m[2] != 2 || (plan->m[0] != 1 && plan->m[0] != 2))
-    return fail(WC_ERR_UNSUPPORTED, "multi-piece output transform needs output tile 2");
+  const bool tile4 = plan->m[0] == 1 && plan->m[1] == 4 && plan->m[2] == 4;
+  const bool tile2 = plan->m[1] == 2 && plan->m[2] == 2 && (plan->m[0] == 1 || plan->m[0] == 2);
+  if (!tile2 && !tile4)
+    return fail(WC_ERR_UNSUPPORTED, "multi-piece output transform needs output tile 2, or 4 in 2-D");
   if (plan->t_total > 0xffff)
     return fail(WC_ERR_UNSUPPORTED, "plan with %d transform elements is too large", plan->t_total);
   OutMultiArgs g;
@@ -243,7 +288,7 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
       if (pc.r[q] < 1 || pc.r[q] > 3) return fail(WC_ERR_UNSUPPORTED, "piece with %d taps", pc.r[q]);
     g.info[i] = pc.t_offset | ((flat ? 0 : pc.r[0]) << 16) | (pc.r[1] << 20) | (pc.r[2] << 24);
   }
-  OutMultiKernel fn = d->dtype == WC_F16 ? pick_multi<half_t>(flat, vec) : pick_multi<float>(flat, vec);
+  OutMultiKernel fn = d->dtype == WC_F16 ? pick_multi<half_t>(flat, plan->m[1], vec) : pick_multi<float>(flat, plan->m[1], vec);
   hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, g);
   WC_CHECK_LAUNCH("output_multi_kernel");
   return WC_OK;

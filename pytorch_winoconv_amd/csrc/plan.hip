@@ -121,8 +121,8 @@ static int check_desc(const wc_conv_desc* d) {
     return fail(WC_ERR_UNSUPPORTED, "stride %d not implemented (1 or 2)", d->stride);
   if (d->m != 2 && d->m != 4)
     return fail(WC_ERR_UNSUPPORTED, "output tile %d not implemented (2 or 4)", d->m);
-  if (d->m == 4 && !(d->ndim == 2 && d->stride == 1 && d->kernel[1] == 3 && d->kernel[2] == 3))
-    return fail(WC_ERR_UNSUPPORTED, "output tile 4 is implemented for 2-D 3x3 stride-1 only");
+  if (d->m == 4 && d->ndim != 2)
+    return fail(WC_ERR_UNSUPPORTED, "output tile 4 is implemented for 2-D problems only");
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   return WC_OK;
 }

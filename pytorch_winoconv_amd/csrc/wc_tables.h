@@ -8,17 +8,21 @@
 //   KIND_43  F(4,3)  alpha 6   Cook-Toom over the points 0, 1, -1, 2, -2 - the point set the
 //                              reference uses for F(2,5) (matrix_conv.py:33); BT equals the
 //                              reference's commented B25 (transform.py:35-40).
+//   KIND_41  F(4,1)  alpha 4   identity, like the reference's F(2,1) literal (matrix_conv.py:15-20)
+//   KIND_42  F(4,2)  alpha 5   Cook-Toom over the points 0, 1, -1, 2 (the reference's point set
+//                              for F(2,4), matrix_conv.py:32), same construction as wincnn.py:49-70
+// KIND_41 / KIND_42 serve the pieces of a decomposed (DWM) kernel when the output tile is 4.
 // AT is m x alpha, G is alpha x r, BT is alpha x alpha, all stored in 6-wide rows.
 #pragma once
 #include "wc_common.h"
 
 namespace wc {
 
-enum Kind { KIND_11 = 0, KIND_21 = 1, KIND_22 = 2, KIND_23 = 3, KIND_43 = 4, KIND_COUNT = 5 };
+enum Kind { KIND_11 = 0, KIND_21 = 1, KIND_22 = 2, KIND_23 = 3, KIND_43 = 4, KIND_41 = 5, KIND_42 = 6, KIND_COUNT = 7 };
 
-__host__ __device__ constexpr int kind_m(int k) { return k == KIND_11 ? 1 : (k == KIND_43 ? 4 : 2); }
+__host__ __device__ constexpr int kind_m(int k) { return k == KIND_11 ? 1 : (k >= KIND_43 ? 4 : 2); }
 __host__ __device__ constexpr int kind_r(int k) {
-  return k == KIND_11 ? 1 : k == KIND_21 ? 1 : k == KIND_22 ? 2 : 3;
+  return (k == KIND_11 || k == KIND_21 || k == KIND_41) ? 1 : (k == KIND_22 || k == KIND_42) ? 2 : 3;
 }
 __host__ __device__ constexpr int kind_alpha(int k) { return kind_m(k) + kind_r(k) - 1; }
 
@@ -27,6 +31,8 @@ inline int kind_of(int m, int r) {
   if (m == 1 && r == 1) return KIND_11;
   if (m == 2 && r >= 1 && r <= 3) return KIND_21 + (r - 1);
   if (m == 4 && r == 3) return KIND_43;
+  if (m == 4 && r == 1) return KIND_41;
+  if (m == 4 && r == 2) return KIND_42;
   return -1;
 }
 
@@ -97,6 +103,28 @@ template <> struct Mats<KIND_43> {
   }
 };
 
+template <> struct Mats<KIND_41> {
+  static constexpr int m = 4, r = 1, alpha = 4;
+  __host__ __device__ static constexpr float at(int i, int j) { return i == j ? 1.f : 0.f; }
+  __host__ __device__ static constexpr float g(int i, int j) { return 1.f; }
+  __host__ __device__ static constexpr float bt(int i, int j) { return i == j ? 1.f : 0.f; }
+};
+template <> struct Mats<KIND_42> {
+  static constexpr int m = 4, r = 2, alpha = 5;
+  __host__ __device__ static constexpr float at(int i, int j) {
+    constexpr float t[4][5] = {{1, 1, 1, 1, 0}, {0, 1, -1, 2, 0}, {0, 1, 1, 4, 0}, {0, 1, -1, 8, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float g(int i, int j) {
+    constexpr float t[5][2] = {{1.f / 2, 0}, {-1.f / 2, -1.f / 2}, {-1.f / 6, 1.f / 6}, {1.f / 6, 1.f / 3}, {0, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float bt(int i, int j) {
+    constexpr float t[5][5] = {{2, -1, -2, 1, 0}, {0, -2, -1, 1, 0}, {0, 2, -3, 1, 0}, {0, -1, 0, 1, 0}, {0, 2, -1, -2, 1}};
+    return t[i][j];
+  }
+};
+
 // Run-time views of the same tables (host planning, the generic filter / multi-piece kernels).
 __host__ __device__ inline float table_g(int kind, int i, int j) {
   switch (kind) {
@@ -104,6 +132,8 @@ __host__ __device__ inline float table_g(int kind, int i, int j) {
     case KIND_21: return Mats<KIND_21>::g(i, j);
     case KIND_22: return Mats<KIND_22>::g(i, j);
     case KIND_23: return Mats<KIND_23>::g(i, j);
+    case KIND_41: return Mats<KIND_41>::g(i, j);
+    case KIND_42: return Mats<KIND_42>::g(i, j);
     default: return Mats<KIND_43>::g(i, j);
   }
 }
@@ -113,6 +143,8 @@ __host__ __device__ inline float table_at(int kind, int i, int j) {
     case KIND_21: return Mats<KIND_21>::at(i, j);
     case KIND_22: return Mats<KIND_22>::at(i, j);
     case KIND_23: return Mats<KIND_23>::at(i, j);
+    case KIND_41: return Mats<KIND_41>::at(i, j);
+    case KIND_42: return Mats<KIND_42>::at(i, j);
     default: return Mats<KIND_43>::at(i, j);
   }
 }

@@ -6,7 +6,7 @@ wino_split; here the same functions run the HIP engine.  Differences: kernels la
 are decomposed into <= 3x3 pieces (DWM) instead of one large F(2,r) tile built from
 fractional interpolation points (matrix_conv.py:31-40) - the decomposition is the numerically
 better of the two; stride 2 is computed by the engine instead of falling back to
-F.conv2d (matrix_conv.py:71-75,93-95); output_block may be 2, or 4 for 3x3 kernels.
+F.conv2d (matrix_conv.py:71-75,93-95); output_block may be 2, or 4 for 2-D convolutions.
 """
 import numpy as np
 import torch
@@ -25,6 +25,13 @@ B[(2, 2)] = np.array([[1., -1., 0.], [0., 1., 0.], [0., -1., 1.]])
 A[(2, 3)] = np.array([[1., 1., 1., 0.], [0., 1., -1., -1.]])
 G[(2, 3)] = np.array([[1., 0., 0.], [.5, .5, .5], [.5, -.5, .5], [0., 0., 1.]])
 B[(2, 3)] = np.array([[1., 0., -1., 0.], [0., 1., 1., 0.], [0., -1., 1., 0.], [0., 1., 0., -1.]])
+A[(4, 1)] = np.eye(4)
+G[(4, 1)] = np.ones((4, 1))
+B[(4, 1)] = np.eye(4)
+A[(4, 2)] = np.array([[1., 1., 1., 1., 0.], [0., 1., -1., 2., 0.], [0., 1., 1., 4., 0.], [0., 1., -1., 8., 1.]])
+G[(4, 2)] = np.array([[1 / 2., 0.], [-1 / 2., -1 / 2.], [-1 / 6., 1 / 6.], [1 / 6., 1 / 3.], [0., 1.]])
+B[(4, 2)] = np.array([[2., -1., -2., 1., 0.], [0., -2., -1., 1., 0.], [0., 2., -3., 1., 0.],
+                      [0., -1., 0., 1., 0.], [0., 2., -1., -2., 1.]])
 A[(4, 3)] = np.array([[1., 1., 1., 1., 1., 0.], [0., 1., -1., 2., -2., 0.],
                       [0., 1., 1., 4., 4., 0.], [0., 1., -1., 8., -8., 1.]])
 G[(4, 3)] = np.array([[1 / 4., 0., 0.], [-1 / 6., -1 / 6., -1 / 6.], [-1 / 6., 1 / 6., -1 / 6.],
@@ -59,9 +66,10 @@ def _run(input, kernel, bias, stride, padding, groups, output_block, dtype):
     x = input.to(dtype)
     w = kernel.to(dtype)
     b = None if bias is None else bias.to(dtype)
-    big = any(int(k) > 3 for k in kernel.shape[2:])
     s = _same_stride(stride)
-    m = 2 if (big or s != 1) else int(output_block)
+    m = int(output_block)
+    if m == 4 and input.dim() != 4:
+        raise NotImplementedError("output_block 4 is available for 2-D convolutions only")
     return engine.conv_forward(x, w, b, s, padding, m)
 
 

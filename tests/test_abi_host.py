@@ -44,6 +44,7 @@ def test_wc_plan_dwm_matches_reference_table(key):
     ((1, 4, 20, 20), (4, 4, 3, 3), 1, 2), ((1, 4, 20, 20), (4, 4, 3, 3), 1, 4),
     ((1, 4, 20, 20), (4, 4, 7, 7), 1, 2), ((1, 4, 20, 20), (4, 4, 7, 7), 2, 2),
     ((1, 4, 20, 20), (4, 4, 3, 3), 2, 2), ((1, 4, 20, 20), (4, 4, 10, 9), 2, 2),
+    ((1, 4, 20, 20), (4, 4, 7, 7), 1, 4), ((1, 4, 20, 20), (4, 4, 5, 4), 2, 4),
     ((1, 4, 9, 20, 20), (4, 4, 3, 3, 3), 1, 2), ((1, 4, 9, 20, 20), (4, 4, 5, 7, 4), 1, 2),
 ])
 def test_wc_plan_conv_matches_oracle(xs, ws, stride, m):
@@ -73,9 +74,9 @@ def test_out_dims_follow_the_reference_arithmetic():
 
 def test_errors_are_status_codes_with_messages_not_exits():
     lib = _lib.load()
-    # unsupported: stride 3, tile 4 with a 5x5 kernel, kernel extent 11
-    for kw in (dict(stride=3), dict(m=4, w=(4, 4, 5, 5)), dict(w=(4, 4, 11, 3))):
-        desc = engine.make_desc((1, 4, 20, 20), kw.get("w", (4, 4, 3, 3)), torch.float32,
+    # unsupported: stride 3, tile 3, kernel extent 11, tile 4 in 3-D
+    for kw in (dict(stride=3), dict(m=3), dict(w=(4, 4, 11, 3)), dict(m=4, x=(1, 4, 9, 20, 20), w=(4, 4, 3, 3, 3))):
+        desc = engine.make_desc(kw.get("x", (1, 4, 20, 20)), kw.get("w", (4, 4, 3, 3)), torch.float32,
                                 kw.get("stride", 1), 0, kw.get("m", 2))
         with pytest.raises(NotImplementedError):
             engine.plan_conv(desc)
@@ -147,7 +148,7 @@ def test_reference_names_are_importable():
 def test_module_tables_equal_oracle_tables():
     import numpy as np
     from oracle import cook_toom
-    for key in ((2, 1), (2, 2), (2, 3), (4, 3)):
+    for key in ((2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3)):
         AT, G, BT = cook_toom.matrices(*key)
         assert np.allclose(pkg.matrix_conv.A[key], AT, atol=1e-16, rtol=0)
         assert np.allclose(pkg.matrix_conv.G[key], G, atol=1e-16, rtol=0)

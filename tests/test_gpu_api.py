@@ -54,6 +54,8 @@ def test_dwm2d_padding_bias_stride(dev, pad):
         ref = F.conv2d(x.double(), w.double(), b.double(), stride=stride, padding=pad)
         y = pkg.dwm.dwm2d(x.to(dev), w.to(dev), b.to(dev), (stride, stride), pad)
         assert y.shape == ref.shape and _nerr(y, ref) < 1e-3
+    y4 = pkg.dwm.dwm2d(x.to(dev), w.to(dev), b.to(dev), (1, 1), pad, output_block=4)
+    assert _nerr(y4, F.conv2d(x.double(), w.double(), b.double(), padding=pad)) < 1e-3
     yh = pkg.dwm.dwm2d(x.half().to(dev), w.half().to(dev), b.half().to(dev), (1, 1), pad)
     refh = F.conv2d(x.half().double(), w.half().double(), b.half().double(), padding=pad)
     assert yh.dtype == torch.float16 and _nerr(yh, refh) < 2e-2

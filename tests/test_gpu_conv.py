@@ -56,6 +56,10 @@ CASES = [
     ((2, 32, 28, 28), (32, 32, 7, 7), 1, 3, 2),
     ((2, 32, 28, 28), (32, 32, 3, 3), 2, 1, 2),
     ((2, 32, 28, 28), (32, 32, 7, 7), 2, 3, 2),
+    ((2, 32, 28, 28), (32, 32, 5, 5), 1, 2, 4),         # DWM with output tile 4
+    ((2, 32, 28, 28), (32, 32, 7, 7), 1, 3, 4),
+    ((2, 32, 28, 28), (32, 32, 3, 3), 2, 1, 4),
+    ((2, 32, 29, 27), (32, 32, 7, 7), 2, 3, 4),
     ((1, 224, 10, 10), (32, 224, 7, 7), 1, 0, 2),       # example.py:100-101
     ((1, 32, 10, 10, 10), (32, 32, 3, 3, 3), 1, 0, 2),  # example.py:112-113
     ((2, 32, 8, 14, 14), (32, 32, 3, 3, 3), 1, 1, 2),   # C3D-style

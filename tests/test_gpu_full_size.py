@@ -32,6 +32,9 @@ CONFIGS = [
     ("c3 512 @7", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, H16),
     ("c4 5x5 s1", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, H16),
     ("c4 7x7 s1", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, H16),
+    ("c4 5x5 s1 tile 4", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, H16),
+    ("c4 7x7 s1 tile 4", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, H16),
+    ("c4 7x7 s2 tile 4", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, H16),
     ("c4 3x3 s2", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, H16),
     ("c4 7x7 s2", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, H16),
     ("c5 3-D", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, H16),

@@ -62,6 +62,11 @@ CASES = [
     ((1, 8, 12, 12), (8, 8, 7, 7), 1, 3, 2),
     ((2, 8, 12, 13), (8, 8, 3, 3), 2, 1, 2),
     ((1, 8, 15, 14), (4, 8, 7, 7), 2, 3, 2),
+    ((2, 16, 12, 13), (8, 16, 5, 5), 1, 2, 4),
+    ((1, 8, 12, 12), (8, 8, 7, 7), 1, 3, 4),
+    ((2, 8, 12, 13), (8, 8, 3, 3), 2, 1, 4),
+    ((1, 8, 15, 14), (4, 8, 7, 7), 2, 3, 4),
+    ((1, 6, 14, 14), (5, 6, 4, 3), 1, 0, 4),
     ((2, 8, 6, 9, 11), (8, 8, 3, 3, 3), 1, 1, 2),
     ((1, 4, 7, 9, 8), (4, 4, 5, 5, 5), 1, 2, 2),
     ((1, 6, 6, 8, 8), (5, 6, 2, 3, 1), 1, 0, 2),

@@ -14,6 +14,9 @@ CASES = [
     ((1, 2, 11, 12), (3, 2, 6, 8), 1, 2, 2),
     ((2, 4, 12, 13), (3, 4, 3, 3), 2, 1, 2), ((1, 4, 15, 14), (3, 4, 7, 7), 2, 3, 2),
     ((1, 4, 15, 14), (3, 4, 5, 5), 2, 2, 2),
+    ((2, 4, 12, 13), (3, 4, 5, 5), 1, 2, 4), ((1, 4, 12, 12), (3, 4, 7, 7), 1, 3, 4),
+    ((1, 2, 11, 12), (3, 2, 4, 3), 1, 0, 4), ((1, 4, 15, 14), (3, 4, 7, 7), 2, 3, 4),
+    ((2, 4, 12, 13), (3, 4, 3, 3), 2, 1, 4),
     ((2, 4, 6, 9, 11), (3, 4, 3, 3, 3), 1, 1, 2), ((1, 3, 7, 9, 8), (2, 3, 5, 5, 5), 1, 2, 2),
     ((1, 3, 6, 8, 8), (2, 3, 2, 3, 1), 1, 0, 2), ((1, 2, 9, 9, 9), (2, 2, 3, 3, 3), 2, 1, 2),
 ]

@@ -41,7 +41,7 @@ def test_generator_satisfies_fir_identity_exactly(m, r, points):
     _fir_identity_exact(AT, G, BT, m, r)
 
 
-@pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 3)])
+@pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3)])
 def test_tables_in_use_satisfy_fir_identity_exactly(m, r):
     AT, G, BT = ct.matrices(m, r)
     as_frac = lambda M: [[Fraction(v).limit_denominator(1000) for v in row] for row in M]
