@@ -35,7 +35,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
 # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116734 KiB, x2.00 by the copy
 # probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
 # profiles/conv3x3_f16_n64_c256_56x56_all_kernels.md.
-GEMM_HBM_TRAFFIC_BYTES = int((116734 * 2.0 + 225792 * 1.0) * 1024)
+GEMM_HBM_TRAFFIC_BYTES = int((116716 * 2.0 + 225792 * 1.0) * 1024)
 
 
 def synthetic(n):
