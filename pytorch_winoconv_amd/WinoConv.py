@@ -4,9 +4,11 @@ nn.Conv2d / nn.Conv3d of the reference (conv.py:324-339, 465-480) a working form
 
 Routing rule of the modules: groups == 1 and dilation == 1 are required for the Winograd
 path; 3x3(x3) stride-1 kernels use plain Winograd, larger kernels and stride 2 the DWM
-decomposition (output tile 4 in 2-D, 2 in 3-D); anything else falls back to
-torch.nn.functional.conv2d/conv3d like the reference does (conv.py:326-332).  The transformed
-filter is cached and recomputed only when the weight changes.
+decomposition (output tile 4 in 2-D, 2 in 3-D); grouped, dilated, stride > 2 or kernel > 10
+convolutions, which the Winograd algorithm here does not cover, go to
+torch.nn.functional.conv2d/conv3d on the same device like the reference does (conv.py:326-332).
+There is no CPU path: a CPU tensor, or a missing HIP library, raises.  The transformed filter
+is cached and recomputed only when the weight changes.
 """
 import torch
 from torch import nn
@@ -60,8 +62,7 @@ class _WinoConvNd(nn.Module):
 
     def _winograd_ok(self, x):
         return (self.groups == 1 and set(self.dilation) == {1} and len(set(self.stride)) == 1
-                and self.stride[0] in (1, 2) and max(self.kernel_size) <= 10 and x.is_cuda
-                and x.dtype in (torch.float16, torch.float32))
+                and self.stride[0] in (1, 2) and max(self.kernel_size) <= 10)
 
     def _tile(self):
         if self.output_block is not None:
@@ -70,6 +71,10 @@ class _WinoConvNd(nn.Module):
 
     def forward(self, x):
         conv = F.conv2d if self.nd == 2 else F.conv3d
+        if not x.is_cuda:
+            raise ValueError("WinoConv: the engine runs on the GPU only; got a CPU tensor")
+        if x.dtype not in (torch.float16, torch.float32):
+            raise NotImplementedError(f"WinoConv: dtype {x.dtype} (float16 and float32 only)")
         if not self._winograd_ok(x):
             return conv(x, self.weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
         w = self.weight.to(x.dtype)

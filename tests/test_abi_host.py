@@ -130,6 +130,8 @@ def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
         engine.make_desc((1, 4, 8, 8), (4, 4, 3, 3), torch.float32, stride=(1, 2))
     with pytest.raises(NotImplementedError):
         pkg.dwm.dwm2d(x, w, groups=2)
+    with pytest.raises(ValueError, match="GPU only"):                       # modules have no CPU path either
+        pkg.WinoConv2d(4, 4, 3, 1, 1)(x)
 
 
 def test_reference_names_are_importable():
