@@ -82,3 +82,39 @@ def test_full_size_config(dev, cfg):
         lhs = engine.conv_forward(xd + x2, wd, None, stride, pad, m)
         rhs = y + engine.conv_forward(x2, wd, None, stride, pad, m)
         assert float((lhs - rhs).abs().max() / rhs.abs().max()) <= 1e-4, name
+
+
+def test_stage_calls_beyond_2g_elements(dev):
+    """Maximum sizes: V and M hold 2.47e9 elements each (more than 2^31), so every kernel's
+    offsets must be 64-bit.  Images are independent, so each stage's slice for one image must
+    equal, bit for bit, the same stage run on that image alone; the chunked one-call entry point
+    must reproduce the un-chunked stage pipeline; and the last image is checked against fp64."""
+    N, C, K, H = 96, 128, 128, 224
+    g = torch.Generator().manual_seed(3)
+    w = (torch.randn(K, C, 3, 3, generator=g) * (2.0 / (C * 9)) ** 0.5).half().to(dev)
+    x = torch.empty(N, H, H, C, dtype=H16, device=dev)                     # channel-last memory
+    for b in range(N):
+        x[b] = torch.randn(H, H, C, generator=g).half().to(dev)
+    desc = engine.make_desc((N, C, H, H), w.shape, H16, 1, 1, 2)
+    plan = engine.plan_conv(desc)
+    U = engine.filter_transform(desc, plan, w)
+    V = engine.input_transform(desc, plan, x)
+    assert V.numel() > 2 ** 31
+    M = engine.batched_gemm(V, U)
+    y = engine.output_transform(desc, plan, M, None, N)
+    tiles = V.shape[1] // N
+    d1 = engine.make_desc((1, C, H, H), w.shape, H16, 1, 1, 2)
+    for b in (0, 41, N - 1):
+        V1 = engine.input_transform(d1, plan, x[b:b + 1])
+        assert torch.equal(V[:, b * tiles:(b + 1) * tiles], V1), ("input transform", b)
+        M1 = engine.batched_gemm(V1, U)
+        assert torch.equal(M[:, b * tiles:(b + 1) * tiles], M1), ("batched gemm", b)
+        y1 = engine.output_transform(d1, plan, M1, None, 1)
+        assert torch.equal(y[b:b + 1], y1), ("output transform", b)
+    del V, M
+    x_nchw = x.permute(0, 3, 1, 2)                                         # channels_last view, no copy
+    yc = engine.conv_forward(x_nchw, w, None, 1, 1, 2)                     # chunked: V + M bounded at 2 GiB
+    assert torch.equal(yc.permute(0, 2, 3, 1), y[:, 0])                    # stage output keeps a depth axis of 1
+    ref = F.conv2d(x_nchw[N - 1:].double().cpu(), w.double().cpu(), padding=1)
+    err = float((yc[N - 1:].double().cpu() - ref).abs().max() / ref.abs().max())
+    assert err <= 2e-2, err
