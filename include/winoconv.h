@@ -47,7 +47,7 @@ typedef enum {
 /* One stride-1 sub-convolution of the DWM plan. */
 typedef struct {
   int tap0[3];   /* first kernel tap per axis (D, H, W)                      */
-  int r[3];      /* taps per axis, 1..3; taps are tap0 + i*tap_step          */
+  int r[3];      /* taps per axis, 1..3 (4..7 for a whole-kernel tile); taps are tap0 + i*tap_step */
   int t_offset;  /* first transform-domain element of this piece             */
 } wc_piece;
 
@@ -69,6 +69,10 @@ typedef struct {
   int m;           /* Winograd output tile: 2, or 4 (2-D problems only)         */
   int dtype;       /* wc_dtype                                                  */
   int chunk_images;/* images per pass of wc_conv_forward; 0 = choose automatically */
+  int whole_kernel;/* 0: kernels > 3 are decomposed into pieces of <= 3 taps (DWM, dwm.py:107-146);
+                    * 1: one F(2,k) x F(2,k) tile for the whole k x k kernel, k = 4..7, the arithmetic
+                    *    of the reference's PyTorch path (matrix_conv.py:112-135, tables :31-35):
+                    *    2-D, stride 1, m = 2 only; loses accuracy quickly with k, fp16 above all */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */

@@ -100,6 +100,11 @@ _LIT = {
         [[1., 0., -1., 0.], [0., 1., 1., 0.], [0., -1., 1., 0.], [0., 1., 0., -1.]]),
 }
 
+# the reference's long point set (matrix_conv.py:31), used for F(2,6) and F(2,7) (matrix_conv.py:34-35)
+POINTS_REF = (0, 1, -1, Fraction(1, 2), -Fraction(1, 2), Fraction(1, 3), -Fraction(1, 3),
+              Fraction(3, 2), -Fraction(3, 2), -3, 2, -2)
+# point sets of the whole-kernel tiles F(2,r), r = 4..7, as the reference builds them (matrix_conv.py:32-35)
+POINTS_F2R = {4: (0, 1, -1, 2), 5: (0, 1, -1, 2, -2), 6: POINTS_REF, 7: POINTS_REF}
 POINTS_F43 = (0, 1, -1, 2, -2)   # same point set the reference uses for F(2,5) (matrix_conv.py:33)
 POINTS_F42 = (0, 1, -1, 2)       # the reference's point set for F(2,4) (matrix_conv.py:32)
 _LIT[(4, 1)] = (                 # one tap: identity, like the reference's F(2,1) literal
@@ -109,7 +114,8 @@ _LIT[(4, 1)] = (                 # one tap: identity, like the reference's F(2,1
 
 
 def matrices(m, r):
-    """(AT, G, BT) float64 for F(m, r).  F(2,1..3) and F(4,1) literal, F(4,2), F(4,3) Cook-Toom."""
+    """(AT, G, BT) float64 for F(m, r).  F(2,1..3) and F(4,1) literal; F(4,2), F(4,3) and the
+    whole-kernel tiles F(2,4..7) Cook-Toom."""
     if (m, r) in _LIT:
         AT, G, BT = _LIT[(m, r)]
         return (np.array(AT, dtype=np.float64), np.array(G, dtype=np.float64),
@@ -118,4 +124,6 @@ def matrices(m, r):
         return cook_toom(POINTS_F43, 4, 3)
     if (m, r) == (4, 2):
         return cook_toom(POINTS_F42, 4, 2)
+    if m == 2 and r in POINTS_F2R:
+        return cook_toom(POINTS_F2R[r], 2, r)
     raise ValueError("F(%d,%d) not on the hot path" % (m, r))

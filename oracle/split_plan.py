@@ -65,7 +65,7 @@ def split_plan(kD, kH, kW):
     return plan
 
 
-def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False):
+def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=False):
     """General plan for a (kD, kH, kW) kernel with one stride for all axes.
 
     Each piece is one stride-1 sub-convolution: per axis (first_tap, tap_step,
@@ -73,9 +73,15 @@ def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False):
     (a 2-D problem, D = kD = 1) the depth axis is F(1,1) - one element - rather
     than the reference's zero-padded alpha = 2 depth tile (dwm.py:117,
     src/split_kernel.cu:93-97), which only multiplies zeros.
+    With `whole_kernel` the kernel is not decomposed: one piece, F(m, k) per axis - the
+    arithmetic of the reference's PyTorch path (matrix_conv.py:112-135), stride 1 only.
     Returns (pieces, T_total); pieces[i] = dict(axes, ms, alphas, t_offset).
     """
-    per_axis = [axis_pieces(k, stride) for k in kernel]
+    if whole_kernel:
+        assert stride == 1
+        per_axis = [[(0, 1, k)] for k in kernel]
+    else:
+        per_axis = [axis_pieces(k, stride) for k in kernel]
     ms = [1 if (ax == 0 and degenerate_depth) else m for ax in range(3)]
     out, t = [], 0
     for combo in product(*per_axis):

@@ -154,7 +154,7 @@ def _as_3d(x, w):
     return x, w, two_d
 
 
-def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2):
+def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
     """Shapes and pieces for an NC[D]HW x (K, C, [kD,] kH, kW) convolution."""
     two_d = len(x_shape) == 4
     sp = ([1] if two_d else []) + list(x_shape[2:])
@@ -162,19 +162,21 @@ def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2):
     if isinstance(padding, int):
         padding = [padding] * (len(x_shape) - 2)
     pads = ([0] if two_d else []) + list(padding)
-    pieces, T_total = conv_pieces(ks, stride, m, degenerate_depth=two_d)
+    pieces, T_total = conv_pieces(ks, stride, m, degenerate_depth=two_d, whole_kernel=whole_kernel)
     od = out_dims(sp, ks, pads, stride)
     grid = tile_grid(od, pieces[0]["ms"])
     return dict(spatial=sp, kernel=ks, pads=pads, pieces=pieces, T_total=T_total,
                 odims=od, grid=grid, two_d=two_d, stride=stride)
 
 
-def dwm_conv(x, w, bias=None, stride=1, padding=0, m=2, discipline="fp32", stages=None):
+def dwm_conv(x, w, bias=None, stride=1, padding=0, m=2, discipline="fp32", stages=None,
+             whole_kernel=False):
     """Native-layout Winograd/DWM convolution.  x NC[D]HW, w (K, C, [kD,] kH, kW).
     Returns y NC[D]HW in the storage type of `discipline`.  If `stages` is a dict the
-    intermediate buffers U, V, M and the plan are stored in it."""
+    intermediate buffers U, V, M and the plan are stored in it.  `whole_kernel`: one F(m, k) tile
+    per axis instead of the DWM pieces (the reference's matrix_conv arithmetic)."""
     st = _STORE[discipline]
-    plan = conv_plan(tuple(x.shape), tuple(w.shape), stride, padding, m)
+    plan = conv_plan(tuple(x.shape), tuple(w.shape), stride, padding, m, whole_kernel)
     x3, w3, two_d = _as_3d(x.to(st), w.to(st))
     xl = x3.permute(0, 2, 3, 4, 1).contiguous()                      # dwm.py:84, :132
     U = filter_transform(w3, plan["pieces"], plan["T_total"], discipline)

@@ -96,7 +96,8 @@ struct FilterArgs {
 };
 
 __device__ __forceinline__ int dev_kind(int m, int r) {
-  return m == 1 ? KIND_11 : (m == 4 ? (r == 3 ? KIND_43 : r == 2 ? KIND_42 : KIND_41) : KIND_21 + (r - 1));
+  return m == 1 ? KIND_11 : (m == 4 ? (r == 3 ? KIND_43 : r == 2 ? KIND_42 : KIND_41)
+                                   : (r <= 3 ? KIND_21 + (r - 1) : KIND_24 + (r - 4)));
 }
 
 template <typename T>

@@ -16,10 +16,10 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   const bool flat = plan->m[0] == 1;
   // Channels per thread.  Measured on MI355X at N=64, C=256, 56x56 fp16: F(4,3) tiles (36 live
   // elements per channel) run best with 2 channels per thread (more wavefronts in flight),
-  // F(2,r) tiles with 16-byte accesses; 3-D tiles (up to 64 elements) use 2.
+  // F(2,r) tiles with 16-byte accesses; 3-D tiles and whole-kernel tiles (up to 64 elements) use 2.
   int want;
   if (!flat) want = 2;
-  else if (plan->m[1] == 4) want = 2;
+  else if (plan->m[1] == 4 || plan->piece[0].r[1] > 3 || plan->piece[0].r[2] > 3) want = 2;
   else want = d->dtype == WC_F16 ? 8 : 4;
   int vec = 1;
   for (int v = want; v > 1; v /= 2)

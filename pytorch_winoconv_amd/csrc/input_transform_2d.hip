@@ -16,6 +16,7 @@ static InKernel pick2d_m2(int k1, int k2) {
 // output tile 2: 8 (fp16) / 4 (fp32) / 2 / 1 channels per thread
 InKernel pick_in_2d(int dtype, int k1, int k2, int vec) {
   if (kind_m(k1) == 4) return pick_in_2d_m4(dtype, k1, k2, vec);
+  if (k1 >= KIND_24 || k2 >= KIND_24) return pick_in_2d_whole(dtype, k1, k2, vec);
   if (dtype == WC_F16) {
     if (vec == 8) return pick2d_m2<half_t, 8>(k1, k2);
     if (vec == 4) return pick2d_m2<half_t, 4>(k1, k2);

@@ -98,6 +98,7 @@ constexpr InKernel in_kernel() { return &input_transform_kernel<T, K0, K1, K2, V
 // Kernel look-up, one translation unit per depth kind so that they compile in parallel.
 InKernel pick_in_2d(int dtype, int k1, int k2, int vec);          // depth kind KIND_11 (2-D problems)
 InKernel pick_in_2d_m4(int dtype, int k1, int k2, int vec);       // ... with output tile 4, vec 2 or 1
+InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec);    // ... whole-kernel tiles F(2,4..7), vec 2 or 1
 InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
 InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
 InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);

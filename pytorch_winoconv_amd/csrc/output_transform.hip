@@ -217,6 +217,12 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
   if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23)
     return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 2>
                     : &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 1>;
+  // whole-kernel tiles F(2,r) x F(2,r), r = 4..7
+#define WC_WHOLE(KD) \
+  if (k0 == KIND_11 && k1 == KD && k2 == KD) \
+    return vec == 4 ? &output_transform_kernel<T, KIND_11, KD, KD, 2> : &output_transform_kernel<T, KIND_11, KD, KD, 1>;
+  WC_WHOLE(KIND_24) WC_WHOLE(KIND_25) WC_WHOLE(KIND_26) WC_WHOLE(KIND_27)
+#undef WC_WHOLE
   return nullptr;
 }
 
@@ -258,9 +264,9 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
                                 : pick_single<float>(k[0], k[1], k[2], vec);
   }
   if (single) {
-    // 3-D tiles and F(4,3) tiles (36 live elements per channel) use 2 channels per thread:
+    // 3-D tiles, F(4,3) tiles (36 live elements per channel) and whole-kernel tiles use 2 channels per thread:
     // more wavefronts in flight (measured 64.8 vs 69.2 us at N=64, K=256, 56x56 fp16)
-    const int v = ((k[0] == KIND_23 || k[1] == KIND_43) && vec == 4) ? 2 : vec;
+    const int v = ((k[0] == KIND_23 || k[1] == KIND_43 || k[1] >= KIND_24) && vec == 4) ? 2 : vec;
     a.n_kvec = d->K / v;
     a.total = P * a.n_kvec;
     a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);

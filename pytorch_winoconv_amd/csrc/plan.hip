@@ -124,6 +124,14 @@ static int check_desc(const wc_conv_desc* d) {
   if (d->m == 4 && d->ndim != 2)
     return fail(WC_ERR_UNSUPPORTED, "output tile 4 is implemented for 2-D problems only");
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
+  WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
+  if (d->whole_kernel) {
+    if (d->ndim != 2 || d->stride != 1 || d->m != 2)
+      return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");
+    if (d->kernel[1] != d->kernel[2] || d->kernel[1] > 7)
+      return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles are built for square kernels up to 7x7, got %dx%d",
+                  d->kernel[1], d->kernel[2]);
+  }
   return WC_OK;
 }
 
@@ -133,7 +141,10 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   WC_CHECK_ARG(plan != nullptr, "wc_plan_conv: null plan");
   AxisPiece ax[3][8];
   int n[3];
-  for (int a = 0; a < 3; ++a) n[a] = axis_pieces(d->kernel[a], d->stride, ax[a]);
+  for (int a = 0; a < 3; ++a) {
+    if (d->whole_kernel) { ax[a][0].tap0 = 0; ax[a][0].r = d->kernel[a]; n[a] = 1; }
+    else n[a] = axis_pieces(d->kernel[a], d->stride, ax[a]);
+  }
   if (n[0] * n[1] * n[2] > WC_MAX_PIECES)
     return fail(WC_ERR_UNSUPPORTED, "%d pieces exceed %d", n[0] * n[1] * n[2], WC_MAX_PIECES);
   std::memset(plan, 0, sizeof(*plan));

@@ -40,8 +40,9 @@ def _triple(v, nd, fill):
     return ((fill,) if nd == 2 else ()) + v
 
 
-def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0):
-    """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter."""
+def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False):
+    """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter.  `whole_kernel`: one
+    F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces."""
     nd = len(x_shape) - 2
     if nd not in (2, 3) or len(w_shape) != nd + 2:
         raise ValueError("expected 4-D or 5-D input and matching filter, got %r and %r"
@@ -63,6 +64,7 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0)
     d.m = int(m)
     d.dtype = _DTYPES[dtype]
     d.chunk_images = int(chunk_images)
+    d.whole_kernel = int(bool(whole_kernel))
     return d
 
 
@@ -157,14 +159,14 @@ def output_transform(desc, plan, M, bias, n_images):
 
 
 # ---------------------------------------------------------------- whole convolution
-def transform_filter(w, x_shape, stride=1, padding=0, m=2):
+def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False):
     """Transformed filter U for later calls of conv_forward(..., U=U)."""
     _require_gpu(w)
-    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m)
+    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel)
     return filter_transform(desc, plan_conv(desc), w)
 
 
-def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0):
+def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False):
     """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
     without a copy, any other layout is permuted once."""
@@ -172,7 +174,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
-    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images)
+    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images, whole_kernel)
     out, _ = out_dims(desc)
     x_cl = channel_last(x)
     nbytes = ctypes.c_size_t()

@@ -2,16 +2,18 @@
 (reference: matrix_conv.py:70-254).
 
 The reference expresses the transforms and the product as torch matmuls on tiles produced by
-wino_split; here the same functions run the HIP engine.  Differences: kernels larger than 3
-are decomposed into <= 3x3 pieces (DWM) instead of one large F(2,r) tile built from
-fractional interpolation points (matrix_conv.py:31-40) - the decomposition is the numerically
-better of the two; stride 2 is computed by the engine instead of falling back to
-F.conv2d (matrix_conv.py:71-75,93-95); output_block may be 2, or 4 for 2-D convolutions.
+wino_split; here the same functions run the HIP engine.  Like the reference, a square 2-D
+kernel of 4..7 taps at stride 1 and output_block 2 is one whole-kernel tile F(2,k) x F(2,k)
+built from the reference's interpolation points (matrix_conv.py:31-35) - this is the
+arithmetic whose loss of accuracy in fp16 the DWM decomposition (dwm.py) avoids; pass
+decompose=True to get the decomposition here too.  Every other kernel larger than 3 (non-square,
+above 7 taps, 3-D, output_block 4) and stride 2 - for which the reference falls back to
+F.conv2d (matrix_conv.py:71-75,93-95) - is decomposed into pieces of <= 3 taps.
 """
 import numpy as np
 import torch
 
-from . import engine
+from . import engine, wincnn
 from .Split_and_Concat import wino_split, wino_concat  # noqa: F401  (re-exported like the reference)
 
 # transform tables under the reference's names: A = AT (m x alpha), G (alpha x r), B = BT
@@ -38,6 +40,12 @@ G[(4, 3)] = np.array([[1 / 4., 0., 0.], [-1 / 6., -1 / 6., -1 / 6.], [-1 / 6., 1
                       [1 / 24., 1 / 12., 1 / 6.], [1 / 24., -1 / 12., 1 / 6.], [0., 0., 1.]])
 B[(4, 3)] = np.array([[4., 0., -5., 0., 1., 0.], [0., -4., -4., 1., 1., 0.], [0., 4., -4., -1., 1., 0.],
                       [0., -2., -1., 2., 1., 0.], [0., 2., -1., -2., 1., 0.], [0., 4., 0., -5., 0., 1.]])
+# whole-kernel tiles, generated like the reference does (matrix_conv.py:31-35)
+points = (0, 1, -1, "1/2", "-1/2", "1/3", "-1/3", "3/2", "-3/2", -3, 2, -2)
+A[(2, 4)], G[(2, 4)], B[(2, 4)] = wincnn.showCookToomFilter((0, 1, -1, 2), 2, 4)
+A[(2, 5)], G[(2, 5)], B[(2, 5)] = wincnn.showCookToomFilter((0, 1, -1, 2, -2), 2, 5)
+A[(2, 6)], G[(2, 6)], B[(2, 6)] = wincnn.showCookToomFilter(points, 2, 6)
+A[(2, 7)], G[(2, 7)], B[(2, 7)] = wincnn.showCookToomFilter(points, 2, 7)
 
 
 def matrix_alloc(m, r):
@@ -60,7 +68,13 @@ def _same_stride(stride):
     return s[0]
 
 
-def _run(input, kernel, bias, stride, padding, groups, output_block, dtype):
+def _whole_kernel(kernel, stride, m, decompose):
+    ks = tuple(kernel.shape[2:])
+    return (not decompose and len(ks) == 2 and ks[0] == ks[1] and 4 <= ks[0] <= 7
+            and stride == 1 and m == 2)
+
+
+def _run(input, kernel, bias, stride, padding, groups, output_block, dtype, decompose=False):
     if groups != 1:
         raise NotImplementedError("groups != 1 is not supported")
     x = input.to(dtype)
@@ -70,23 +84,23 @@ def _run(input, kernel, bias, stride, padding, groups, output_block, dtype):
     m = int(output_block)
     if m == 4 and input.dim() != 4:
         raise NotImplementedError("output_block 4 is available for 2-D convolutions only")
-    return engine.conv_forward(x, w, b, s, padding, m)
+    return engine.conv_forward(x, w, b, s, padding, m, whole_kernel=_whole_kernel(w, s, m, decompose))
 
 
-def conv16(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2):
+def conv16(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2, decompose=False):
     """Half-precision Winograd convolution returning float32 (reference: matrix_conv.py:70-90)."""
-    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float16).float()
+    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float16, decompose).float()
 
 
-def conv32(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2):
+def conv32(input, kernel, bias=None, stride=(1, 1), padding=0, groups=1, output_block=2, decompose=False):
     """Single-precision Winograd convolution (reference: matrix_conv.py:92-110)."""
-    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float32)
+    return _run(input, kernel, bias, stride, padding, groups, output_block, torch.float32, decompose)
 
 
-def conv(input, kernel, output_block, stride, fp16=False):
+def conv(input, kernel, output_block, stride, fp16=False, decompose=False):
     """VALID stride-1 convolution (reference: matrix_conv.py:112-135)."""
     dtype = torch.float16 if fp16 else torch.float32
-    out = _run(input, kernel, None, 1, 0, 1, output_block, dtype)
+    out = _run(input, kernel, None, 1, 0, 1, output_block, dtype, decompose)
     return out.float() if fp16 else out
 
 
@@ -99,4 +113,5 @@ def base_conv32(input, kernel, fp16, m, r):
     if list(input.shape[2:]) != [mi + ri - 1 for mi, ri in zip(m, r)]:
         raise ValueError("base_conv32: tiles of shape %r do not match F(%r, %r)" % (tuple(input.shape[2:]), m, r))
     dtype = torch.float16 if fp16 else input.dtype
-    return engine.conv_forward(input.to(dtype), kernel.to(dtype), None, 1, 0, int(m[0])).contiguous()
+    return engine.conv_forward(input.to(dtype), kernel.to(dtype), None, 1, 0, int(m[0]),
+                               whole_kernel=_whole_kernel(kernel, 1, int(m[0]), False)).contiguous()

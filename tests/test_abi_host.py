@@ -134,6 +134,50 @@ def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
         pkg.WinoConv2d(4, 4, 3, 1, 1)(x)
 
 
+def test_whole_kernel_plans():
+    """One F(2,k) x F(2,k) piece for a k x k kernel (the reference's matrix_conv tile,
+    matrix_conv.py:112-135) and the descriptor checks around it."""
+    lib = _lib.load()
+    for k in (4, 5, 6, 7):
+        d = engine.make_desc((2, 8, 20, 20), (4, 8, k, k), torch.float32, 1, 0, 2, whole_kernel=True)
+        plan = engine.plan_conv(d)
+        assert plan.n_pieces == 1 and plan.t_total == (k + 1) ** 2
+        assert list(plan.piece[0].r) == [1, k, k] and list(plan.piece[0].tap0) == [0, 0, 0]
+        assert list(plan.m) == [1, 2, 2]
+    d3 = engine.make_desc((2, 8, 20, 20), (4, 8, 3, 3), torch.float32, 1, 1, 2, whole_kernel=True)
+    assert engine.plan_conv(d3).t_total == 16                       # 3x3 is a whole-kernel tile anyway
+    for bad in (dict(x=(2, 8, 20, 20), w=(4, 8, 5, 5), stride=2, m=2),
+                dict(x=(2, 8, 20, 20), w=(4, 8, 5, 5), stride=1, m=4),
+                dict(x=(2, 8, 20, 20), w=(4, 8, 5, 7), stride=1, m=2),
+                dict(x=(2, 8, 20, 20), w=(4, 8, 9, 9), stride=1, m=2),
+                dict(x=(2, 8, 9, 20, 20), w=(4, 8, 5, 5, 5), stride=1, m=2)):
+        d = engine.make_desc(bad["x"], bad["w"], torch.float32, bad["stride"], 0, bad["m"], whole_kernel=True)
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(d)
+
+
+def test_product_generator_equals_oracle_generator():
+    """pytorch_winoconv_amd.wincnn (Lagrange-basis form) against oracle.cook_toom (the
+    reference generator's steps), exact rationals, and against the reference's F(2,9) literals."""
+    import json, os
+    from fractions import Fraction
+    from oracle import cook_toom
+    from pytorch_winoconv_amd import wincnn
+    cases = [((0, 1, -1), 2, 3), ((0, 1, -1, 2, -2), 4, 3), ((0, 1, -1, 2), 4, 2), ((0, 1, -1, 2), 2, 4),
+             (cook_toom.POINTS_REF, 2, 6), (cook_toom.POINTS_REF, 2, 7), (cook_toom.POINTS_REF, 9, 5)]
+    for pts, m, r in cases:
+        a = wincnn.cookToomFilter(pts, m, r)
+        b = cook_toom.cook_toom_exact(pts, m, r)
+        assert a[0] == b[0] and a[1] == b[1] and a[2] == b[2], (m, r)
+    with open(os.path.join(os.path.dirname(__file__), "golden", "cook_toom_f29.json")) as f:
+        g = json.load(f)
+    AT, G, BT = wincnn.cookToomFilter(g["points"], g["m"], g["r"])
+    frac = lambda M: [[Fraction(v) for v in row] for row in M]
+    assert AT == frac(g["AT"]) and G == frac(g["G"]) and BT == frac(g["BT"])
+    with pytest.raises(ValueError):
+        wincnn.cookToomFilter((0, 1), 2, 3)                          # too few points
+
+
 def test_reference_names_are_importable():
     for name in ("AddGPU", "Foo", "WinoSplit", "WinoConcat", "DWM", "add_gpu", "wino_split", "wino_concat",
                  "winograd_conv", "split_and_concat", "Wino", "Dwm", "WinoConv2d", "WinoConv3d"):
@@ -150,7 +194,7 @@ def test_reference_names_are_importable():
 def test_module_tables_equal_oracle_tables():
     import numpy as np
     from oracle import cook_toom
-    for key in ((2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3)):
+    for key in ((2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3), (2, 4), (2, 5), (2, 6), (2, 7)):
         AT, G, BT = cook_toom.matrices(*key)
         assert np.allclose(pkg.matrix_conv.A[key], AT, atol=1e-16, rtol=0)
         assert np.allclose(pkg.matrix_conv.G[key], G, atol=1e-16, rtol=0)

@@ -76,6 +76,27 @@ def test_matrix_conv_functions(dev):
     assert _nerr(pkg.matrix_conv3d.conv32(x3.to(dev), w3.to(dev), b3.to(dev), (1, 1, 1), (1, 1, 1)), ref3) < 1e-3
 
 
+def test_matrix_conv_whole_kernel_tile_and_decompose_switch(dev):
+    """matrix_conv.conv32 on a 5x5 kernel is one F(2,5) x F(2,5) tile like the reference
+    (matrix_conv.py:112-135): bit-identical to the engine's whole-kernel plan; decompose=True
+    is bit-identical to the DWM plan; wino_split -> base_conv32 -> wino_concat with 6x6 tiles
+    gives the whole-kernel result too."""
+    x, w, _ = _mk((2, 16, 18, 17), (8, 16, 5, 5))
+    xd, wd = x.to(dev), w.to(dev)
+    ref = F.conv2d(x.double(), w.double())
+    y = pkg.matrix_conv.conv32(xd, wd)
+    assert torch.equal(y, pkg.engine.conv_forward(xd, wd, whole_kernel=True))
+    assert _nerr(y, ref) < 1e-3
+    yd = pkg.matrix_conv.conv32(xd, wd, decompose=True)
+    assert torch.equal(yd, pkg.engine.conv_forward(xd, wd))
+    assert not torch.equal(y, yd)
+    tiles = pkg.wino_split(xd, list(w.shape), 2)
+    assert tuple(tiles.shape[2:]) == (6, 6)
+    out = pkg.matrix_conv.base_conv32(tiles, wd, False, [2, 2], [5, 5])
+    yc = pkg.wino_concat(out, [14, 13], 2)
+    assert _nerr(yc, ref) < 1e-3 and _nerr(yc, y.double().cpu()) < 1e-5
+
+
 def test_split_base_conv_concat_pipeline_like_the_reference(dev):
     """matrix_conv.conv's own sequence (matrix_conv.py:126-134): wino_split -> base_conv32 ->
     wino_concat, against the oracle's restatement of that path and fp64 convolution."""

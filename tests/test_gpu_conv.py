@@ -118,6 +118,47 @@ def test_integer_exactness(dev, dtype, case):
     assert torch.equal(y.double().cpu(), ref)
 
 
+WHOLE = [
+    # x shape, w shape, pad; whole-kernel tile F(2,k) x F(2,k) (reference: matrix_conv.py:112-135)
+    ((2, 32, 28, 28), (32, 32, 4, 4), 1),
+    ((2, 32, 28, 28), (32, 32, 5, 5), 2),
+    ((2, 32, 27, 29), (32, 32, 6, 6), 0),
+    ((2, 32, 28, 28), (32, 32, 7, 7), 3),
+    ((1, 224, 10, 10), (32, 224, 7, 7), 0),             # example.py:100-101
+]
+
+
+@pytest.mark.parametrize("case", WHOLE)
+def test_whole_kernel_tile_fp32(dev, case):
+    """fp32 whole-kernel tiles against fp64 convolution and against the oracle run in the same
+    discipline.  The tile's own rounding error grows with k (the oracle shows 1e-6 at k = 4 to
+    5e-4 at k = 7 on these inputs), so the bound against fp64 is 2e-3, and the engine's error
+    must stay within 3x that of the oracle's fp32 evaluation of the same formula (the two
+    differ in summation order, so at k = 7 they differ from each other as much as from fp64)."""
+    xs, ws, pad = case
+    x, w, b = _data(xs, ws, torch.float32)
+    ref = _conv64(x, w, b, 1, pad)
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2, whole_kernel=True)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert _nerr(y, ref) <= 2e-3
+    yo = ow.dwm_conv(x, w, b, 1, pad, 2, "fp32", whole_kernel=True)
+    assert _nerr(y, ref) <= 3 * _nerr(yo, ref) + 1e-6
+
+
+def test_decomposition_keeps_fp16_accurate_where_the_whole_kernel_tile_does_not(dev):
+    """The reference's claim (example.py:99-109): for a 7x7 kernel in half precision the DWM
+    pieces stay accurate while one F(2,7) tile does not.  Same uniform inputs as the demo."""
+    x, w, _ = _data((1, 224, 10, 10), (32, 224, 7, 7), torch.float16, uniform=True)
+    ref = _conv64(x, w, None, 1, 0)
+    xd, wd = x.to(dev), w.to(dev)
+    e_dwm = _nerr(engine.conv_forward(xd, wd, None, 1, 0, 2), ref)
+    e_whole = _nerr(engine.conv_forward(xd, wd, None, 1, 0, 2, whole_kernel=True), ref)
+    e_oracle = _nerr(ow.dwm_conv(x, w, None, 1, 0, 2, "fp16", whole_kernel=True), ref)
+    assert e_dwm <= 2e-3
+    assert e_whole >= 20 * e_dwm                         # the tile really is that much worse
+    assert 0.25 * e_oracle <= e_whole <= 4 * e_oracle    # and as bad as the same formula on the CPU
+
+
 def test_reference_statistic(dev):
     """The reference's own accuracy statistic mean(|(y - y64) / y64|) on U(0,1) data at its own
     shapes (example.py:99-119); recorded for continuity, bounded loosely."""

@@ -8,6 +8,8 @@ Independent facts used (none is a retyped copy of the generator's formula):
     (what wincnn.filterVerify checks symbolically, wincnn.py:73-87), on basis vectors;
   * the published Lavin & Gray F(4x4,3x3) matrices, equal to the reference's commented B25 / G25
     literals (transform.py:29-40);
+  * the reference's commented F(2,9) literals A29 / G29 / B29 (transform.py:41-61), kept as data
+    in tests/golden/cook_toom_f29.json: a 10 x 10 case with the sign and scaling convention;
   * spot formulas of the reference's unrolled kernels (transform_kernels.cu:1191,1587-1588,
     transform_kernels_3d.cu:4998).
 """
@@ -41,7 +43,8 @@ def test_generator_satisfies_fir_identity_exactly(m, r, points):
     _fir_identity_exact(AT, G, BT, m, r)
 
 
-@pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3)])
+@pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3),
+                                 (2, 4), (2, 5), (2, 6), (2, 7)])
 def test_tables_in_use_satisfy_fir_identity_exactly(m, r):
     AT, G, BT = ct.matrices(m, r)
     as_frac = lambda M: [[Fraction(v).limit_denominator(1000) for v in row] for row in M]
@@ -74,6 +77,36 @@ def test_f25_generator_reproduces_the_reference_literals():
     assert np.array_equal(AT, np.array(A25, dtype=np.float64))
     assert np.allclose(G, np.array(G25), rtol=0, atol=1e-16)
     assert np.array_equal(BT, np.array(B25, dtype=np.float64))
+
+
+def _golden_f29():
+    import json, os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "cook_toom_f29.json")) as f:
+        g = json.load(f)
+    frac = lambda M: [[Fraction(v) for v in row] for row in M]
+    return g["points"], g["m"], g["r"], frac(g["AT"]), frac(g["G"]), frac(g["BT"])
+
+
+def test_f29_generator_reproduces_the_reference_literals():
+    """A 10 x 10 known answer: the generator over the points 0, +-1 .. +-4 must give the
+    reference's commented A29 / G29 / B29 exactly (rational arithmetic, no tolerance)."""
+    points, m, r, AT, G, BT = _golden_f29()
+    got = ct.cook_toom_exact(points, m, r)
+    assert got[0] == AT and got[1] == G and got[2] == BT
+    _fir_identity_exact(AT, G, BT, m, r)          # and the literals themselves are a valid F(2,9)
+
+
+def test_whole_kernel_tables_use_the_reference_point_sets():
+    """F(2,4..7) as the reference builds them (matrix_conv.py:31-35): the first alpha-1 entries of
+    its point tuples.  AT rows are the powers of those points, which fixes the choice of points;
+    the FIR identity above fixes the rest up to the scaling that the F(2,5)/F(2,9) literals fix."""
+    long_points = [0, 1, -1, Fraction(1, 2), Fraction(-1, 2), Fraction(1, 3), Fraction(-1, 3)]
+    want = {4: [0, 1, -1, 2], 5: [0, 1, -1, 2, -2], 6: long_points[:6], 7: long_points[:7]}
+    for r, pts in want.items():
+        AT, G, BT = ct.matrices(2, r)
+        assert np.array_equal(AT[0], np.array([1.] * r + [0.]))
+        assert np.allclose(AT[1], np.array([float(p) for p in pts] + [1.]), rtol=0, atol=0)
+        assert np.array_equal(G[-1], np.eye(r)[-1]) and BT[-1][-1] == 1.0
 
 
 def test_kernel_spot_formulas():
