@@ -155,33 +155,42 @@ __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
   }
 
   // Epilogue through LDS so that global stores are whole rows.  Accumulator (i, j), register
-  // 4q + e holds output channel 32j + 8q + 4*lhi + e of tile row 32i + l32.
+  // 4q + e holds output channel 32j + 8q + 4*lhi + e of tile row 32i + l32.  The tile is staged
+  // EI accumulator rows at a time (all of them for fp16; one for fp32, whose full tile would need
+  // 135 KB and leave room for only one workgroup per CU).
+  constexpr int EI = sizeof(T) == 4 ? 1 : WM;
   constexpr int CS = BN + EPC;                     // padded row of the staged output tile
+  constexpr int SROWS = 64 * EI;                   // staged rows per pass: 2 wavefront rows x EI x 32
   T* cs = lds;   // operand stages are free after the last barrier; the launch sizes LDS for both uses
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        Pack<T, 4> o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
-        *reinterpret_cast<Pack<T, 4>*>(cs + (wp * WM * 32 + i * 32 + l32) * CS + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi) = o;
-      }
-  __syncthreads();
   T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
   constexpr int CPRO = BN / EPC;                   // 16-byte chunks per output row
   constexpr int RPPO = 256 / CPRO;                 // rows per pass
-  static_assert(256 % CPRO == 0 && BM % RPPO == 0, "output tile shape");
+  static_assert(256 % CPRO == 0 && SROWS % RPPO == 0, "output tile shape");
   const int orow = tid / CPRO, ocol = (tid % CPRO) * EPC;
-  if (k0 + ocol < g.ldm) {
 #pragma unroll
-    for (int r = 0; r < BM / RPPO; ++r) {
-      const int row = orow + r * RPPO;
-      if (p0 + row < g.P)
-        *reinterpret_cast<Chunk16*>(Mt + (long long)(p0 + row) * g.ldm + k0 + ocol) =
-            *reinterpret_cast<const Chunk16*>(cs + row * CS + ocol);
+  for (int i0 = 0; i0 < WM; i0 += EI) {
+    if (i0 > 0) __syncthreads();                   // the previous pass has been read out
+#pragma unroll
+    for (int ii = 0; ii < EI; ++ii)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          Pack<T, 4> o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i0 + ii][j][4 * q + e]);
+          *reinterpret_cast<Pack<T, 4>*>(cs + (wp * EI * 32 + ii * 32 + l32) * CS + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi) = o;
+        }
+    __syncthreads();
+    if (k0 + ocol < g.ldm) {
+#pragma unroll
+      for (int r = 0; r < SROWS / RPPO; ++r) {
+        const int srow = orow + r * RPPO;            // staged row: wavefront row, then (ii, l32)
+        const int row = (srow / (EI * 32)) * WM * 32 + i0 * 32 + srow % (EI * 32);
+        if (p0 + row < g.P)
+          *reinterpret_cast<Chunk16*>(Mt + (long long)(p0 + row) * g.ldm + k0 + ocol) =
+              *reinterpret_cast<const Chunk16*>(cs + srow * CS + ocol);
+      }
     }
   }
 }
@@ -198,7 +207,7 @@ template <typename T, int WM, int WN, int BK>
 static GemmConfig make_config() {
   constexpr int EPC = 16 / sizeof(T);
   constexpr size_t stages = (size_t)2 * (64 * WM + 64 * WN) * (BK + EPC) * sizeof(T);
-  constexpr size_t out_tile = (size_t)64 * WM * (64 * WN + EPC) * sizeof(T);
+  constexpr size_t out_tile = (size_t)64 * (sizeof(T) == 4 ? 1 : WM) * (64 * WN + EPC) * sizeof(T);
   return GemmConfig{&gemm_kernel<T, WM, WN, BK>, 64 * WM, 64 * WN, BK,
                     stages > out_tile ? stages : out_tile};
 }
@@ -235,16 +244,23 @@ template <> struct Configs<float> {
   }
 };
 
-// Picks the largest tile that still gives the 256 CUs about two workgroups each and does not
-// waste more than half a tile on the channel axis.
+// fp16: the largest tile that still gives the 256 CUs about two workgroups each and does not
+// waste more than half a tile on the channel axis (the big tile moves the fewest bytes, and the
+// fp16 product is bound by memory).  fp32: always the 64 x 64 tile.  One reduction step of an
+// fp32 stage is only 16 deep, so a big tile has too little work per stage to cover the load
+// latency with one or two workgroups per CU; the small tile runs 4+ workgroups per CU and
+// measured 1.0-1.3x faster than every larger tile on all VGG-16 layer shapes (N = 8), within 4 %
+// of the best tile on each.
 template <typename T>
-static GemmConfig choose(int T_, int P, int K) {
+static GemmConfig choose(int T_, int P, int K, int Cp) {
   const char* force = std::getenv("WINOCONV_GEMM_CONFIG");
   if (force) {
     const int i = std::atoi(force);
     if (i >= 0 && i < Configs<T>::n) return Configs<T>::get(i);
   }
   constexpr int n_auto = 5;
+  // (a reduction of <= 64 channels is one or two stages: the same argument holds for fp16)
+  if (sizeof(T) == 4 || Cp <= 64) return Configs<T>::get(n_auto - 1);
   GemmConfig best = Configs<T>::get(n_auto - 1);
   for (int i = 0; i < n_auto; ++i) {
     GemmConfig c = Configs<T>::get(i);
@@ -266,7 +282,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(Cp > 0 && Cp % 32 == 0, "wc_batched_gemm: reduction extent %d is not a multiple of 32", Cp);
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "wc_batched_gemm: row stride %d (needs >= K, multiple of 8)", ldm);
   WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32, "wc_batched_gemm: dtype %d", dtype);
-  GemmConfig c = dtype == WC_F16 ? choose<half_t>(T_, P, K) : choose<float>(T_, P, K);
+  GemmConfig c = dtype == WC_F16 ? choose<half_t>(T_, P, K, Cp) : choose<float>(T_, P, K, Cp);
   GemmArgs g;
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;
