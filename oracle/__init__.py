@@ -20,13 +20,17 @@ winograd    filter / input / output transforms, batched product, the
 
 Pinning status (what independent facts each function is checked against lives
 in tests/test_oracle_*.py):
-  cook_toom.*          pinned: literal tables in the reference source, exact
-                       rational FIR identity, textbook F(4,3) matrices.
+  cook_toom.*          pinned: literal tables in the reference source (F(2,1..3),
+                       commented F(2,5) and F(2,9)), exact rational FIR identity,
+                       textbook F(4,3) matrices, and - for the whole-kernel tiles
+                       F(2,4..7) and F(9,5), fractional points included - the output
+                       of the reference's own generator, kept as exact rationals in
+                       tests/golden/cook_toom_reference_tables.json (written once by
+                       tests/golden/make_cook_toom_tables.py).
   split_plan.*         pinned: all 36 keys of the reference LUT (golden JSON).
   tiles.*              pinned: torch unfold / brute-force loops, odd edges.
   winograd.*           pinned: fp64 torch conv2d/conv3d, integer-exact KATs,
                        the reference kernels' unrolled spot formulas.
-  Large-tile F(2,r>=4) matrices with the reference's fractional point set
-  (matrix_conv.py:31-40): parity unpinned (only an import of the reference's
-  wincnn could fix the AT/G/BT scaling split; they are off the hot path).
+  Tables F(2,8..11) of the reference (matrix_conv.py:36-39) are not restated:
+  nothing here uses them.
 """

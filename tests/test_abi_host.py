@@ -174,6 +174,10 @@ def test_product_generator_equals_oracle_generator():
     AT, G, BT = wincnn.cookToomFilter(g["points"], g["m"], g["r"])
     frac = lambda M: [[Fraction(v) for v in row] for row in M]
     assert AT == frac(g["AT"]) and G == frac(g["G"]) and BT == frac(g["BT"])
+    with open(os.path.join(os.path.dirname(__file__), "golden", "cook_toom_reference_tables.json")) as f:
+        for t in json.load(f)["tables"]:                             # the reference generator's own output
+            got = wincnn.cookToomFilter(t["points"], t["m"], t["r"])
+            assert got[0] == frac(t["AT"]) and got[1] == frac(t["G"]) and got[2] == frac(t["BT"])
     with pytest.raises(ValueError):
         wincnn.cookToomFilter((0, 1), 2, 3)                          # too few points
 

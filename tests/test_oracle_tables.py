@@ -10,6 +10,10 @@ Independent facts used (none is a retyped copy of the generator's formula):
     literals (transform.py:29-40);
   * the reference's commented F(2,9) literals A29 / G29 / B29 (transform.py:41-61), kept as data
     in tests/golden/cook_toom_f29.json: a 10 x 10 case with the sign and scaling convention;
+  * the output of the reference's own generator (wincnn.py:49-70) for the point sets it uses at
+    import (matrix_conv.py:31-36), fractional points included, written once in the build
+    container by tests/golden/make_cook_toom_tables.py into
+    tests/golden/cook_toom_reference_tables.json (exact rationals);
   * spot formulas of the reference's unrolled kernels (transform_kernels.cu:1191,1587-1588,
     transform_kernels_3d.cu:4998).
 """
@@ -94,6 +98,25 @@ def test_f29_generator_reproduces_the_reference_literals():
     got = ct.cook_toom_exact(points, m, r)
     assert got[0] == AT and got[1] == G and got[2] == BT
     _fir_identity_exact(AT, G, BT, m, r)          # and the literals themselves are a valid F(2,9)
+
+
+def test_generator_reproduces_the_reference_generator_output():
+    """F(2,4), F(2,5), F(2,6), F(2,7) and F(9,5) exactly as the reference's generator returns
+    them for its own point tuples - the split of the scaling between AT, G and BT for
+    fractional points is a convention only that output shows."""
+    import json, os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "cook_toom_reference_tables.json")) as f:
+        tables = json.load(f)["tables"]
+    assert sorted((t["m"], t["r"]) for t in tables) == [(2, 4), (2, 5), (2, 6), (2, 7), (9, 5)]
+    frac = lambda M: [[Fraction(v) for v in row] for row in M]
+    for t in tables:
+        got = ct.cook_toom_exact([Fraction(p) for p in t["points"]], t["m"], t["r"])
+        assert got[0] == frac(t["AT"]) and got[1] == frac(t["G"]) and got[2] == frac(t["BT"]), (t["m"], t["r"])
+        if t["m"] == 2:                      # and these are the tables in use for whole-kernel tiles
+            AT, G, BT = ct.matrices(2, t["r"])
+            as_f = lambda M: np.array([[float(v) for v in row] for row in M])
+            assert np.array_equal(AT, as_f(got[0])) and np.array_equal(G, as_f(got[1]))
+            assert np.array_equal(BT, as_f(got[2]))
 
 
 def test_whole_kernel_tables_use_the_reference_point_sets():
