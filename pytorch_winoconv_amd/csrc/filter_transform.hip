@@ -8,7 +8,8 @@
 // its operands along contiguous rows (the reference keeps (T, C, K): split_kernel.cu:51).
 // Arithmetic in fp32, one rounding to the storage type.  Tiny (K*C*T outputs); run once per
 // weight update by callers that cache U.  Single-piece plans of the common shapes take a
-// compile-time kernel (taps loaded once per (k, c)); anything else the generic one.
+// compile-time kernel (taps loaded once per (k, c)), DWM plans one launch whose workgroups pick the
+// compile-time body of their piece; anything else (whole-kernel tiles) the generic kernel.
 #include "wc_transform.h"
 
 namespace wc {
@@ -36,27 +37,22 @@ struct FilterFastArgs {
   int t_offset;
 };
 
-// Single piece with compile-time kinds: one thread per (k, c) loads its taps once, transforms
-// in registers and writes the alpha^d elements with lanes along c (coalesced rows of U).
+// One (k, c) of one piece with compile-time kinds: loads the taps once, transforms in registers
+// and writes the alpha^d elements (lanes along c: coalesced rows of U).
 template <typename T, int K0, int K1, int K2>
-__global__ __launch_bounds__(256) void filter_transform_fast_kernel(const FilterFastArgs a) {
+__device__ __forceinline__ void transform_taps(const T* __restrict__ w, const long long (&s)[5], int k, int c,
+                                               bool ok, const int (&tap0)[3], int step, T* __restrict__ U,
+                                               long long plane) {
   constexpr int R0 = Mats<K0>::r, R1 = Mats<K1>::r, R2 = Mats<K2>::r;
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
-  const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= a.K * a.Cp) return;
-  const int c = idx % a.Cp, k = idx / a.Cp;
-  T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + idx;
-  const long long plane = (long long)a.K * a.Cp;
   float g[R0 * R1 * R2][1];
-  const bool ok = c < a.C;
-  const T* w = static_cast<const T*>(a.w) + k * a.s[0] + (ok ? c : 0) * a.s[1];
+  const T* wp = w + k * s[0] + (ok ? c : 0) * s[1];
   static_for<0, R0>([&](auto j0_) {
     static_for<0, R1>([&](auto j1_) {
       static_for<0, R2>([&](auto j2_) {
         constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
-        const float v = static_cast<float>(w[(a.tap0[0] + j0 * a.step) * a.s[2] +
-                                            (a.tap0[1] + j1 * a.step) * a.s[3] +
-                                            (a.tap0[2] + j2 * a.step) * a.s[4]]);
+        const float v = static_cast<float>(wp[(tap0[0] + j0 * step) * s[2] + (tap0[1] + j1 * step) * s[3] +
+                                             (tap0[2] + j2 * step) * s[4]]);
         g[(j0 * R1 + j1) * R2 + j2][0] = ok ? v : 0.f;
       });
     });
@@ -71,6 +67,17 @@ __global__ __launch_bounds__(256) void filter_transform_fast_kernel(const Filter
     constexpr int e = decltype(e_)::value;
     U[e * plane] = static_cast<T>(u0[e][0]);
   });
+}
+
+// Single piece with compile-time kinds: one thread per (k, c).
+template <typename T, int K0, int K1, int K2>
+__global__ __launch_bounds__(256) void filter_transform_fast_kernel(const FilterFastArgs a) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.K * a.Cp) return;
+  const int c = idx % a.Cp, k = idx / a.Cp;
+  T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + idx;
+  transform_taps<T, K0, K1, K2>(static_cast<const T*>(a.w), a.s, k, c, c < a.C, a.tap0, a.step, U,
+                                (long long)a.K * a.Cp);
 }
 
 using FilterFastKernel = void (*)(FilterFastArgs);
@@ -98,6 +105,35 @@ struct FilterArgs {
 __device__ __forceinline__ int dev_kind(int m, int r) {
   return m == 1 ? KIND_11 : (m == 4 ? (r == 3 ? KIND_43 : r == 2 ? KIND_42 : KIND_41)
                                    : (r <= 3 ? KIND_21 + (r - 1) : KIND_24 + (r - 4)));
+}
+
+// Any plan whose pieces have 1..3 taps per axis (every DWM plan): blockIdx.y is the piece, one
+// thread per (k, c); the piece's taps-per-axis select one of the compile-time bodies (a branch
+// that is uniform over the workgroup).  FLAT: one-element depth axis; MO: output tile 2 or 4.
+template <typename T, bool FLAT, int MO>
+__global__ __launch_bounds__(256) void filter_transform_pieces_kernel(const FilterArgs a) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.K * a.Cp) return;
+  const wc_piece& pc = a.piece[blockIdx.y];
+  const int c = idx % a.Cp, k = idx / a.Cp;
+  const long long plane = (long long)a.K * a.Cp;
+  T* U = static_cast<T*>(a.U) + (long long)pc.t_offset * plane + idx;
+  const T* w = static_cast<const T*>(a.w);
+  const bool ok = c < a.C;
+  constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
+#define WC_BODY(K0, K1, K2) transform_taps<T, K0, K1, K2>(w, a.s, k, c, ok, pc.tap0, a.step, U, plane)
+#define WC_ROW(K0, K1) \
+  switch (pc.r[2]) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
+#define WC_PLANE(K0) \
+  switch (pc.r[1]) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
+  if constexpr (FLAT) {
+    WC_PLANE(KIND_11)
+  } else {
+    switch (pc.r[0]) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
+  }
+#undef WC_PLANE
+#undef WC_ROW
+#undef WC_BODY
 }
 
 template <typename T>
@@ -174,6 +210,26 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   a.n_pieces = plan->n_pieces;
   for (int i = 0; i < plan->n_pieces; ++i) a.piece[i] = plan->piece[i];
   a.total = (long long)plan->t_total * d->K * a.Cp;
+  bool small_taps = true;
+  for (int i = 0; i < plan->n_pieces; ++i)
+    for (int q = 0; q < 3; ++q) small_taps = small_taps && plan->piece[i].r[q] >= 1 && plan->piece[i].r[q] <= 3;
+  const bool flat = plan->m[0] == 1;
+  const int mo = plan->m[1];
+  if (small_taps && plan->m[2] == mo && (flat ? (mo == 2 || mo == 4) : (mo == 2 && plan->m[0] == 2))) {
+    const long long n = (long long)d->K * a.Cp;
+    WC_CHECK_ARG(n < (1ll << 31), "wc_filter_transform: problem too large");
+    const dim3 grid((unsigned)ceil_div_ll(n, 256), (unsigned)plan->n_pieces);
+    void (*fn)(FilterArgs);
+    if (d->dtype == WC_F16)
+      fn = !flat ? &filter_transform_pieces_kernel<half_t, false, 2>
+                 : (mo == 4 ? &filter_transform_pieces_kernel<half_t, true, 4> : &filter_transform_pieces_kernel<half_t, true, 2>);
+    else
+      fn = !flat ? &filter_transform_pieces_kernel<float, false, 2>
+                 : (mo == 4 ? &filter_transform_pieces_kernel<float, true, 4> : &filter_transform_pieces_kernel<float, true, 2>);
+    hipLaunchKernelGGL(fn, grid, dim3(256), 0, as_stream(stream), a);
+    WC_CHECK_LAUNCH("filter_transform_pieces_kernel");
+    return WC_OK;
+  }
   const long long blocks = ceil_div_ll(a.total, 256);
   WC_CHECK_ARG(blocks < (1ll << 31), "wc_filter_transform: problem too large");
   if (d->dtype == WC_F16)
