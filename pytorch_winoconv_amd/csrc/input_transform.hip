@@ -24,12 +24,48 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   int vec = 1;
   for (int v = want; v > 1; v /= 2)
     if (d->C % v == 0) { vec = v; break; }
+  InArgs a;
+  a.x = x; a.V = V;
+  a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = Cp;
+  a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
+  a.step = plan->tap_step;
+  a.t_stride = P * Cp;
+  a.n_cvec = Cp / vec;
+  a.total = P * a.n_cvec;
+  const long long blocks = ceil_div_ll(a.total, 256);
+  a.per_xcd = (int)ceil_div_ll(blocks, kXcds);
+  WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
+  const dim3 launch_grid((unsigned)(a.per_xcd * kXcds));
+
+  // 2-D DWM plans: all pieces in one launch
+  bool small_taps = plan->n_pieces > 1 && flat && plan->t_total <= 0xffff;
+  for (int s = 0; s < plan->n_pieces && small_taps; ++s) {
+    const wc_piece& pc = plan->piece[s];
+    small_taps = pc.r[1] >= 1 && pc.r[1] <= 3 && pc.r[2] >= 1 && pc.r[2] <= 3 && pc.tap0[1] < 16 && pc.tap0[2] < 16;
+  }
+  if (small_taps && plan->m[1] == plan->m[2]) {
+    InPiecesKernel fn = pick_in_2d_pieces(d->dtype, plan->m[1], vec);
+    if (fn) {
+      InPiecesArgs g;
+      a.base0 = a.base1 = a.base2 = 0; a.t_offset = 0;
+      g.o = a;
+      g.n_pieces = plan->n_pieces;
+      g.pad1 = d->pad[1]; g.pad2 = d->pad[2];
+      for (int s = 0; s < plan->n_pieces; ++s) {
+        const wc_piece& pc = plan->piece[s];
+        g.info[s] = pc.t_offset | (pc.tap0[1] << 16) | (pc.tap0[2] << 20) | (pc.r[1] << 24) | (pc.r[2] << 28);
+      }
+      hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), g);
+      WC_CHECK_LAUNCH("input_transform_pieces_kernel");
+      return WC_OK;
+    }
+  }
   for (int s = 0; s < plan->n_pieces; ++s) {
     const wc_piece& pc = plan->piece[s];
     int k[3];
-    for (int a = 0; a < 3; ++a) {
-      k[a] = kind_of(plan->m[a], pc.r[a]);
-      if (k[a] < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[a], pc.r[a]);
+    for (int q = 0; q < 3; ++q) {
+      k[q] = kind_of(plan->m[q], pc.r[q]);
+      if (k[q] < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[q], pc.r[q]);
     }
     InKernel fn = nullptr;
     switch (k[0]) {
@@ -40,20 +76,9 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       default: break;
     }
     if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for kinds (%d,%d,%d) not built", k[0], k[1], k[2]);
-    InArgs a;
-    a.x = x; a.V = V;
-    a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = Cp;
-    a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
     a.base0 = pc.tap0[0] - d->pad[0]; a.base1 = pc.tap0[1] - d->pad[1]; a.base2 = pc.tap0[2] - d->pad[2];
-    a.step = plan->tap_step;
-    a.t_stride = P * Cp;
     a.t_offset = pc.t_offset;
-    a.n_cvec = Cp / vec;
-    a.total = P * a.n_cvec;
-    const long long blocks = ceil_div_ll(a.total, 256);
-    a.per_xcd = (int)ceil_div_ll(blocks, kXcds);
-    WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
-    hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, as_stream(stream), a);
+    hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("input_transform_kernel");
   }
   return WC_OK;

@@ -1,0 +1,39 @@
+// Input transform of every piece of a 2-D DWM plan (pieces of 1..3 taps per axis) in one launch.
+#include "input_transform_impl.h"
+
+namespace wc {
+
+template <typename T, int MO, int VEC>
+__global__ __launch_bounds__(256) void input_transform_pieces_kernel(InPiecesArgs g) {
+  const InArgs& a = g.o;
+  InWhere w;
+  if (!in_decode(a, xcd_remap(blockIdx.x, a.per_xcd), VEC, w)) return;
+  constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
+  for (int s = 0; s < g.n_pieces; ++s) {
+    const int info = g.info[s];
+    const int t_offset = info & 0xffff;
+    const int base1 = ((info >> 16) & 15) - g.pad1, base2 = ((info >> 20) & 15) - g.pad2;
+    const int r1 = (info >> 24) & 15, r2 = (info >> 28) & 15;
+#define WC_BODY(K1, K2) transform_window<T, KIND_11, K1, K2, VEC>(a, w, 0, base1, base2, t_offset)
+#define WC_ROW(K1) \
+  switch (r2) { case 1: WC_BODY(K1, KA); break; case 2: WC_BODY(K1, KB); break; default: WC_BODY(K1, KC); }
+    switch (r1) { case 1: WC_ROW(KA) break; case 2: WC_ROW(KB) break; default: WC_ROW(KC) }
+#undef WC_ROW
+#undef WC_BODY
+  }
+}
+
+template <typename T>
+static InPiecesKernel pick(int m, int vec) {
+  if (m == 4) return vec == 2 ? &input_transform_pieces_kernel<T, 4, 2> : vec == 1 ? &input_transform_pieces_kernel<T, 4, 1> : nullptr;
+  if (vec == 8 && sizeof(T) == 2) return &input_transform_pieces_kernel<T, 2, 8>;
+  if (vec == 4) return &input_transform_pieces_kernel<T, 2, 4>;
+  if (vec == 2) return &input_transform_pieces_kernel<T, 2, 2>;
+  return vec == 1 ? &input_transform_pieces_kernel<T, 2, 1> : nullptr;
+}
+
+InPiecesKernel pick_in_2d_pieces(int dtype, int m, int vec) {
+  return dtype == WC_F16 ? pick<half_t>(m, vec) : pick<float>(m, vec);
+}
+
+}  // namespace wc

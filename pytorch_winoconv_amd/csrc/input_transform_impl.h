@@ -1,5 +1,6 @@
 // Input transform kernel (included by the per-shape translation units).
-// Input transform V = (BT_d x BT_h x BT_w) d, channel-last input, one launch per piece.
+// Input transform V = (BT_d x BT_h x BT_w) d, channel-last input; one launch per piece, or one
+// launch for all pieces of a 2-D DWM plan.
 //
 // Replaces inputNorm2WinoTransform + inputNorm2WinoCalculation of the reference
 // (src/split_kernel.cu:60-120, src/calculation_kernels.cu:763-1522).  Window of tile t,
@@ -29,43 +30,56 @@ struct InArgs {
   int per_xcd;
 };
 
+// Tile coordinates and channel offset of one thread
+struct InWhere {
+  int td, th, tw, c;
+  long long b, p;
+  bool c_ok;
+};
+
+// blk: logical workgroup index (after the XCD remap)
+__device__ __forceinline__ bool in_decode(const InArgs& a, int blk, int vec, InWhere& w) {
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return false;
+  const int cv = (int)(idx % a.n_cvec);
+  w.p = idx / a.n_cvec;
+  w.tw = (int)(w.p % a.nW); long long q = w.p / a.nW;
+  w.th = (int)(q % a.nH); q /= a.nH;
+  w.td = (int)(q % a.nD);
+  w.b = q / a.nD;
+  w.c = cv * vec;
+  w.c_ok = w.c < a.C;
+  return true;
+}
+
+// One window (tile x VEC channels) of one piece: load, transform, store.
 template <typename T, int K0, int K1, int K2, int VEC>
-__global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
+__device__ __forceinline__ void transform_window(const InArgs& a, const InWhere& w, int base0, int base1,
+                                                 int base2, int t_offset) {
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
   constexpr int m0 = Mats<K0>::m, m1 = Mats<K1>::m, m2 = Mats<K2>::m;
-  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
-  const long long idx = (long long)blk * 256 + threadIdx.x;
-  if (idx >= a.total) return;
-  const int cv = (int)(idx % a.n_cvec);
-  const long long p = idx / a.n_cvec;
-  const int tw = (int)(p % a.nW); long long q = p / a.nW;
-  const int th = (int)(q % a.nH); q /= a.nH;
-  const int td = (int)(q % a.nD);
-  const long long b = q / a.nD;
-  const int c = cv * VEC;
-  const bool c_ok = c < a.C;
   const T* x = static_cast<const T*>(a.x);
 
   // Every load is issued unconditionally from a clamped address and zeroed afterwards if the
   // window element lies outside the image: the loads of a tile are then all in flight together
   // instead of one per divergent branch.
   float d[A0 * A1 * A2][VEC];
-  const int cc = c_ok ? c : 0;
+  const int cc = w.c_ok ? w.c : 0;
   static_for<0, A0>([&](auto i0_) {
     constexpr int i0 = decltype(i0_)::value;
-    const int z = a.step * (m0 * td + i0) + a.base0;
-    const bool z_ok = c_ok && (unsigned)z < (unsigned)a.D;
+    const int z = a.step * (m0 * w.td + i0) + base0;
+    const bool z_ok = w.c_ok && (unsigned)z < (unsigned)a.D;
     const int zc = min(max(z, 0), a.D - 1);
     static_for<0, A1>([&](auto i1_) {
       constexpr int i1 = decltype(i1_)::value;
-      const int yy = a.step * (m1 * th + i1) + a.base1;
+      const int yy = a.step * (m1 * w.th + i1) + base1;
       const bool y_ok = z_ok && (unsigned)yy < (unsigned)a.H;
       const int yc = min(max(yy, 0), a.H - 1);
-      const long long row = ((b * a.D + zc) * a.H + yc) * a.W;
+      const long long row = ((w.b * a.D + zc) * a.H + yc) * a.W;
       static_for<0, A2>([&](auto i2_) {
         constexpr int i2 = decltype(i2_)::value;
         constexpr int e = (i0 * A1 + i1) * A2 + i2;
-        const int xx = a.step * (m2 * tw + i2) + a.base2;
+        const int xx = a.step * (m2 * w.tw + i2) + base2;
         const bool ok = y_ok && (unsigned)xx < (unsigned)a.W;
         const int xc = min(max(xx, 0), a.W - 1);
         load_pack<T, VEC>(x + (row + xc) * a.C + cc, d[e]);
@@ -82,13 +96,33 @@ __global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
   if constexpr (A0 > 1) {
     apply_axis<MatSel<K0, false>, 0, A0, A1, A2, VEC>(d, t2);
   }
-  T* V = static_cast<T*>(a.V) + (long long)a.t_offset * a.t_stride + p * a.Cp + c;
+  T* V = static_cast<T*>(a.V) + (long long)t_offset * a.t_stride + w.p * a.Cp + w.c;
   static_for<0, A0 * A1 * A2>([&](auto e_) {
     constexpr int e = decltype(e_)::value;
     if constexpr (A0 > 1) store_pack<T, VEC>(V + e * a.t_stride, t2[e]);
     else store_pack<T, VEC>(V + e * a.t_stride, d[e]);
   });
 }
+
+template <typename T, int K0, int K1, int K2, int VEC>
+__global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
+  InWhere w;
+  if (!in_decode(a, xcd_remap(blockIdx.x, a.per_xcd), VEC, w)) return;
+  transform_window<T, K0, K1, K2, VEC>(a, w, a.base0, a.base1, a.base2, a.t_offset);
+}
+
+// All pieces of a 2-D DWM plan in one launch: a thread transforms the windows of its tile piece
+// after piece, so the overlapping windows of the pieces are read from HBM once and then served
+// by the caches (a launch per piece reads the whole input once per piece; giving each piece its
+// own workgroup next to the others on one XCD measured 8-16 % slower than this loop).
+struct InPiecesArgs {
+  InArgs o;                       // base0/1/2 and t_offset unused
+  int n_pieces;
+  int pad1, pad2;
+  int info[WC_MAX_PIECES];        // t_offset | tap0_h << 16 | tap0_w << 20 | r_h << 24 | r_w << 28
+};
+using InPiecesKernel = void (*)(InPiecesArgs);
+InPiecesKernel pick_in_2d_pieces(int dtype, int m, int vec);     // nullptr if the combination is not built
 
 using InKernel = void (*)(InArgs);
 
