@@ -8,11 +8,13 @@
 // written iff it lies inside (oD, oH, oW).
 //
 // HBM-bound: a thread owns one tile x VEC consecutive output channels (lanes along K).
-// Two kernels: a separable compile-time one for single-piece plans (F(2,3)^2, F(4,3)^2,
-// F(2,3)^3) and a streaming one for any other plan (F(2,r) pieces, or F(4,r) pieces in 2-D),
-// where each loaded tile row is transformed along the width and then scattered into the m^d
+// Three kernels: a separable compile-time one for single-piece plans (F(2,3)^2, F(4,3)^2,
+// F(2,3)^3, whole-kernel tiles); one for 2-D DWM plans that runs the same compile-time body for
+// every piece and sums the pieces in registers; and a streaming one for 3-D DWM plans, where
+// each loaded tile row is transformed along the width and then scattered into the m^d
 // accumulators with coefficients from a constant table.
 #include "wc_transform.h"
+#include <type_traits>
 
 namespace wc {
 
@@ -203,6 +205,66 @@ __global__ __launch_bounds__(256) void output_multi_kernel(OutMultiArgs g) {
   write_tile<T, M0, MO, MO, VEC>(a, w, k, acc);
 }
 
+// ---- all pieces of a 2-D DWM plan, compile-time body per piece ------------------------------------
+// Each piece is handled like a single-piece plan (all alpha_h x alpha_w loads of the tile issued
+// together, separable AT passes in registers) and added to the m x m accumulators; the piece's
+// taps per axis select the body, a branch that is uniform over the launch.
+template <typename T, int MO, int VEC>
+__global__ __launch_bounds__(256) void output_pieces_kernel(OutMultiArgs g) {
+  const OutArgs& a = g.o;
+  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int k = (int)(idx % a.n_kvec) * VEC;
+  const long long p = idx / a.n_kvec;
+  const Where w = decode_tile(p, a.nD, a.nH, a.nW);
+  const T* M = static_cast<const T*>(a.M) + p * a.ldm + k;
+  constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
+
+  float acc[MO * MO][VEC];
+#pragma unroll
+  for (int e = 0; e < MO * MO; ++e)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[e][v] = 0.f;
+
+  auto piece = [&](auto k1_, auto k2_, const T* Ms) {
+    constexpr int K1 = decltype(k1_)::value, K2 = decltype(k2_)::value;
+    constexpr int A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
+    float m[A1 * A2][VEC];
+    static_for<0, A1 * A2>([&](auto e_) {
+      constexpr int e = decltype(e_)::value;
+      load_pack<T, VEC>(Ms + e * a.t_stride, m[e]);
+    });
+    float s2[A1 * MO][VEC];
+    apply_axis<MatSel<K2, true>, 2, 1, A1, A2, VEC>(m, s2);
+    float s1[MO * MO][VEC];
+    apply_axis<MatSel<K1, true>, 1, 1, A1, MO, VEC>(s2, s1);
+#pragma unroll
+    for (int e = 0; e < MO * MO; ++e)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[e][v] += s1[e][v];
+  };
+  using IA = std::integral_constant<int, KA>;
+  using IB = std::integral_constant<int, KB>;
+  using IC = std::integral_constant<int, KC>;
+  for (int s = 0; s < g.n_pieces; ++s) {
+    const int info = g.info[s];
+    const int r1 = (info >> 20) & 15, r2 = (info >> 24) & 15;
+    const T* Ms = M + (long long)(info & 0xffff) * a.t_stride;
+#define WC_ROW(I1) \
+  switch (r2) { case 1: piece(I1{}, IA{}, Ms); break; case 2: piece(I1{}, IB{}, Ms); break; default: piece(I1{}, IC{}, Ms); }
+    switch (r1) { case 1: WC_ROW(IA) break; case 2: WC_ROW(IB) break; default: WC_ROW(IC) }
+#undef WC_ROW
+  }
+  write_tile<T, 1, MO, MO, VEC>(a, w, k, acc);
+}
+
+template <typename T>
+static void (*pick_pieces(int m, int vec))(OutMultiArgs) {
+  if (m == 4) return vec == 2 ? &output_pieces_kernel<T, 4, 2> : &output_pieces_kernel<T, 4, 1>;
+  return vec == 4 ? &output_pieces_kernel<T, 2, 4> : &output_pieces_kernel<T, 2, 1>;
+}
+
 using OutKernel = void (*)(OutArgs);
 using OutMultiKernel = void (*)(OutMultiArgs);
 
@@ -293,6 +355,17 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
     for (int q = 0; q < 3; ++q)
       if (pc.r[q] < 1 || pc.r[q] > 3) return fail(WC_ERR_UNSUPPORTED, "piece with %d taps", pc.r[q]);
     g.info[i] = pc.t_offset | ((flat ? 0 : pc.r[0]) << 16) | (pc.r[1] << 20) | (pc.r[2] << 24);
+  }
+  if (flat) {
+    // 2-D plans: compile-time body per piece; F(4,r) tiles use 2 channels per thread
+    const int v = (tile4 && vec == 4) ? 2 : vec;
+    g.o.n_kvec = d->K / v;
+    g.o.total = P * g.o.n_kvec;
+    g.o.per_xcd = (int)ceil_div_ll(ceil_div_ll(g.o.total, 256), kXcds);
+    OutMultiKernel fp = d->dtype == WC_F16 ? pick_pieces<half_t>(plan->m[1], v) : pick_pieces<float>(plan->m[1], v);
+    hipLaunchKernelGGL(fp, dim3((unsigned)(g.o.per_xcd * kXcds)), dim3(256), 0, s, g);
+    WC_CHECK_LAUNCH("output_pieces_kernel");
+    return WC_OK;
   }
   OutMultiKernel fn = d->dtype == WC_F16 ? pick_multi<half_t>(flat, plan->m[1], vec) : pick_multi<float>(flat, plan->m[1], vec);
   hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, g);
