@@ -32,7 +32,8 @@
 extern "C" {
 #endif
 
-typedef enum { WC_F32 = 0, WC_F16 = 1 } wc_dtype;
+/* storage type of every tensor of a call; arithmetic inside the kernels is always fp32 */
+typedef enum { WC_F32 = 0, WC_F16 = 1, WC_BF16 = 2 } wc_dtype;
 
 typedef enum {
   WC_OK = 0,

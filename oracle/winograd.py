@@ -26,7 +26,8 @@ transform_kernels_3d.cu:4987).
   "fp16"  float16 storage of x, w, U, V, M, y with float32 arithmetic inside each
           stage and one rounding per stored value (the engine's fp16 contract;
           the reference's own half path rounds after every matmul,
-          matrix_conv.py:160-251).
+          matrix_conv.py:160-251),
+  "bf16"  the same contract with bfloat16 storage (the reference has no bfloat16 path).
 """
 import math
 import torch
@@ -34,8 +35,8 @@ import torch
 from . import cook_toom
 from .split_plan import conv_pieces
 
-_STORE = {"fp64": torch.float64, "fp32": torch.float32, "fp16": torch.float16}
-_MATH = {"fp64": torch.float64, "fp32": torch.float32, "fp16": torch.float32}
+_STORE = {"fp64": torch.float64, "fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+_MATH = {"fp64": torch.float64, "fp32": torch.float32, "fp16": torch.float32, "bf16": torch.float32}
 
 
 def _mats(m, r, dtype):

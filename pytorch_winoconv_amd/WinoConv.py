@@ -69,16 +69,22 @@ class _WinoConvNd(nn.Module):
             return int(self.output_block)
         return 4 if self.nd == 2 else 2
 
+    def _tile_for(self, dtype):
+        # F(4,r) tiles lose about 1e-1 of the output range in bfloat16 (8 mantissa bits): tile 2 there
+        if self.output_block is None and dtype == torch.bfloat16:
+            return 2
+        return self._tile()
+
     def forward(self, x):
         conv = F.conv2d if self.nd == 2 else F.conv3d
         if not x.is_cuda:
             raise ValueError("WinoConv: the engine runs on the GPU only; got a CPU tensor")
-        if x.dtype not in (torch.float16, torch.float32):
-            raise NotImplementedError(f"WinoConv: dtype {x.dtype} (float16 and float32 only)")
+        if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"WinoConv: dtype {x.dtype} (float32, float16 and bfloat16 only)")
         if not self._winograd_ok(x):
             return conv(x, self.weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
         w = self.weight.to(x.dtype)
-        m = self._tile()
+        m = self._tile_for(x.dtype)
         key = (self.weight._version, self.weight.data_ptr(), tuple(x.shape[2:]), x.dtype, m)
         if self._cache is None or self._cache[0] != key:
             U = engine.transform_filter(w.detach(), x.shape, self.stride[0], self.padding, m)

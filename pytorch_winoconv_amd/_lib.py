@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libwinoconv_hip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
-WC_F32, WC_F16 = 0, 1
+WC_F32, WC_F16, WC_BF16 = 0, 1, 2
 WC_OK, WC_ERR_BAD_ARG, WC_ERR_UNSUPPORTED, WC_ERR_WORKSPACE, WC_ERR_HIP = 0, -1, -2, -3, -4
 WC_MAX_PIECES = 64
 

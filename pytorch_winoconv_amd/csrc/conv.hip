@@ -32,7 +32,7 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   if (rc) return rc;
   L->Cp = wc_padded_channels(d->C);
   L->ldm = wc_padded_channels8(d->K);
-  L->es = d->dtype == WC_F16 ? 2 : 4;
+  L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
   const long long T = L->plan.t_total;
   int chunk = d->chunk_images;

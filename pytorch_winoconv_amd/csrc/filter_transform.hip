@@ -185,7 +185,7 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   if (plan->n_pieces == 1) {
     const wc_piece& pc = plan->piece[0];
     const int k0 = kind_of(plan->m[0], pc.r[0]), k1 = kind_of(plan->m[1], pc.r[1]), k2 = kind_of(plan->m[2], pc.r[2]);
-    FilterFastKernel fn = d->dtype == WC_F16 ? pick_fast<half_t>(k0, k1, k2) : pick_fast<float>(k0, k1, k2);
+    FilterFastKernel fn = dispatch_dtype(d->dtype, [&](auto t) { return pick_fast<decltype(t)>(k0, k1, k2); });
     if (fn) {
       FilterFastArgs f;
       f.w = w; f.U = U;
@@ -219,23 +219,21 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
     const long long n = (long long)d->K * a.Cp;
     WC_CHECK_ARG(n < (1ll << 31), "wc_filter_transform: problem too large");
     const dim3 grid((unsigned)ceil_div_ll(n, 256), (unsigned)plan->n_pieces);
-    void (*fn)(FilterArgs);
-    if (d->dtype == WC_F16)
-      fn = !flat ? &filter_transform_pieces_kernel<half_t, false, 2>
-                 : (mo == 4 ? &filter_transform_pieces_kernel<half_t, true, 4> : &filter_transform_pieces_kernel<half_t, true, 2>);
-    else
-      fn = !flat ? &filter_transform_pieces_kernel<float, false, 2>
-                 : (mo == 4 ? &filter_transform_pieces_kernel<float, true, 4> : &filter_transform_pieces_kernel<float, true, 2>);
+    void (*fn)(FilterArgs) = dispatch_dtype(d->dtype, [&](auto t) -> void (*)(FilterArgs) {
+      using T = decltype(t);
+      return !flat ? &filter_transform_pieces_kernel<T, false, 2>
+                   : (mo == 4 ? &filter_transform_pieces_kernel<T, true, 4> : &filter_transform_pieces_kernel<T, true, 2>);
+    });
     hipLaunchKernelGGL(fn, grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("filter_transform_pieces_kernel");
     return WC_OK;
   }
   const long long blocks = ceil_div_ll(a.total, 256);
   WC_CHECK_ARG(blocks < (1ll << 31), "wc_filter_transform: problem too large");
-  if (d->dtype == WC_F16)
-    filter_transform_kernel<half_t><<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(a);
-  else
-    filter_transform_kernel<float><<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(a);
+  void (*gen)(FilterArgs) = dispatch_dtype(d->dtype, [](auto t) -> void (*)(FilterArgs) {
+    return &filter_transform_kernel<decltype(t)>;
+  });
+  hipLaunchKernelGGL(gen, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), a);
   WC_CHECK_LAUNCH("filter_transform_kernel");
   return WC_OK;
 }

@@ -13,13 +13,14 @@
 // fragment reads of 8 consecutive rows hit 32 distinct banks.  The MFMA "A" operand is the
 // filter block and "B" the input block: a lane then holds 4 consecutive output channels of
 // one tile row per accumulator group and stores them as one 8-byte (fp16) / 16-byte (fp32)
-// write.  fp16 accumulates in fp32; fp32 uses v_mfma_f32_32x32x2_f32.
+// write.  fp16 and bf16 accumulate in fp32; fp32 uses v_mfma_f32_32x32x2_f32.
 #include "wc_common.h"
 #include <cstdlib>
 
 namespace wc {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 template <typename T> struct Mfma;
@@ -29,6 +30,14 @@ template <> struct Mfma<half_t> {
   static constexpr int kstep = 16;   // reduction elements per instruction
   __device__ static __forceinline__ floatx16 run(Frag a, Frag b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<bf16_t> {
+  using Frag = bf16x8;
+  static constexpr int kpack = 8;
+  static constexpr int kstep = 16;
+  __device__ static __forceinline__ floatx16 run(Frag a, Frag b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mfma<float> {
@@ -231,6 +240,18 @@ template <> struct Configs<half_t> {
     }
   }
 };
+template <> struct Configs<bf16_t> {
+  static constexpr int n = 5;
+  static GemmConfig get(int i) {
+    switch (i) {
+      case 0: return make_config<bf16_t, 4, 2, 32>();
+      case 1: return make_config<bf16_t, 2, 2, 32>();
+      case 2: return make_config<bf16_t, 4, 1, 32>();
+      case 3: return make_config<bf16_t, 2, 1, 32>();
+      default: return make_config<bf16_t, 1, 1, 32>();
+    }
+  }
+};
 template <> struct Configs<float> {
   static constexpr int n = 5;
   static GemmConfig get(int i) {
@@ -281,8 +302,8 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(T_ > 0 && P > 0 && K > 0, "wc_batched_gemm: T %d, P %d, K %d", T_, P, K);
   WC_CHECK_ARG(Cp > 0 && Cp % 32 == 0, "wc_batched_gemm: reduction extent %d is not a multiple of 32", Cp);
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "wc_batched_gemm: row stride %d (needs >= K, multiple of 8)", ldm);
-  WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32, "wc_batched_gemm: dtype %d", dtype);
-  GemmConfig c = dtype == WC_F16 ? choose<half_t>(T_, P, K, Cp) : choose<float>(T_, P, K, Cp);
+  WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32 || dtype == WC_BF16, "wc_batched_gemm: dtype %d", dtype);
+  GemmConfig c = dispatch_dtype(dtype, [&](auto t) { return choose<decltype(t)>(T_, P, K, Cp); });
   GemmArgs g;
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;

@@ -20,7 +20,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   int want;
   if (!flat) want = 2;
   else if (plan->m[1] == 4 || plan->piece[0].r[1] > 3 || plan->piece[0].r[2] > 3) want = 2;
-  else want = d->dtype == WC_F16 ? 8 : 4;
+  else want = d->dtype == WC_F32 ? 4 : 8;
   int vec = 1;
   for (int v = want; v > 1; v /= 2)
     if (d->C % v == 0) { vec = v; break; }

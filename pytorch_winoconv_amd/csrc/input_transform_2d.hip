@@ -17,10 +17,17 @@ static InKernel pick2d_m2(int k1, int k2) {
 InKernel pick_in_2d(int dtype, int k1, int k2, int vec) {
   if (kind_m(k1) == 4) return pick_in_2d_m4(dtype, k1, k2, vec);
   if (k1 >= KIND_24 || k2 >= KIND_24) return pick_in_2d_whole(dtype, k1, k2, vec);
-  if (dtype == WC_F16) {
-    if (vec == 8) return pick2d_m2<half_t, 8>(k1, k2);
-    if (vec == 4) return pick2d_m2<half_t, 4>(k1, k2);
-    return vec == 2 ? pick2d_m2<half_t, 2>(k1, k2) : pick2d_m2<half_t, 1>(k1, k2);
+  if (dtype == WC_F16 || dtype == WC_BF16) {
+    return dispatch_dtype(dtype, [&](auto t) -> InKernel {
+      using T = decltype(t);
+      if constexpr (sizeof(T) == 2) {
+        if (vec == 8) return pick2d_m2<T, 8>(k1, k2);
+        if (vec == 4) return pick2d_m2<T, 4>(k1, k2);
+        return vec == 2 ? pick2d_m2<T, 2>(k1, k2) : pick2d_m2<T, 1>(k1, k2);
+      } else {
+        return nullptr;
+      }
+    });
   }
   if (vec == 4) return pick2d_m2<float, 4>(k1, k2);
   return vec == 2 ? pick2d_m2<float, 2>(k1, k2) : pick2d_m2<float, 1>(k1, k2);

@@ -33,7 +33,7 @@ static InPiecesKernel pick(int m, int vec) {
 }
 
 InPiecesKernel pick_in_2d_pieces(int dtype, int m, int vec) {
-  return dtype == WC_F16 ? pick<half_t>(m, vec) : pick<float>(m, vec);
+  return dispatch_dtype(dtype, [&](auto t) { return pick<decltype(t)>(m, vec); });
 }
 
 }  // namespace wc

@@ -14,8 +14,10 @@ static InKernel pick2d_whole(int k1, int k2) {
 
 // 2 channels per thread (1 when C is odd): up to 64 live elements per channel
 InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec) {
-  if (dtype == WC_F16) return vec == 2 ? pick2d_whole<half_t, 2>(k1, k2) : pick2d_whole<half_t, 1>(k1, k2);
-  return vec == 2 ? pick2d_whole<float, 2>(k1, k2) : pick2d_whole<float, 1>(k1, k2);
+  return dispatch_dtype(dtype, [&](auto t) -> InKernel {
+    using T = decltype(t);
+    return vec == 2 ? pick2d_whole<T, 2>(k1, k2) : pick2d_whole<T, 1>(k1, k2);
+  });
 }
 
 }  // namespace wc

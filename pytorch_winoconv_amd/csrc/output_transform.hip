@@ -322,8 +322,7 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
   OutKernel single = nullptr;
   if (plan->n_pieces == 1) {
     for (int q = 0; q < 3; ++q) k[q] = kind_of(plan->m[q], plan->piece[0].r[q]);
-    single = d->dtype == WC_F16 ? pick_single<half_t>(k[0], k[1], k[2], vec)
-                                : pick_single<float>(k[0], k[1], k[2], vec);
+    single = dispatch_dtype(d->dtype, [&](auto t) { return pick_single<decltype(t)>(k[0], k[1], k[2], vec); });
   }
   if (single) {
     // 3-D tiles, F(4,3) tiles (36 live elements per channel) and whole-kernel tiles use 2 channels per thread:
@@ -362,12 +361,12 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, c
     g.o.n_kvec = d->K / v;
     g.o.total = P * g.o.n_kvec;
     g.o.per_xcd = (int)ceil_div_ll(ceil_div_ll(g.o.total, 256), kXcds);
-    OutMultiKernel fp = d->dtype == WC_F16 ? pick_pieces<half_t>(plan->m[1], v) : pick_pieces<float>(plan->m[1], v);
+    OutMultiKernel fp = dispatch_dtype(d->dtype, [&](auto t) { return pick_pieces<decltype(t)>(plan->m[1], v); });
     hipLaunchKernelGGL(fp, dim3((unsigned)(g.o.per_xcd * kXcds)), dim3(256), 0, s, g);
     WC_CHECK_LAUNCH("output_pieces_kernel");
     return WC_OK;
   }
-  OutMultiKernel fn = d->dtype == WC_F16 ? pick_multi<half_t>(flat, plan->m[1], vec) : pick_multi<float>(flat, plan->m[1], vec);
+  OutMultiKernel fn = dispatch_dtype(d->dtype, [&](auto t) { return pick_multi<decltype(t)>(flat, plan->m[1], vec); });
   hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, g);
   WC_CHECK_LAUNCH("output_multi_kernel");
   return WC_OK;

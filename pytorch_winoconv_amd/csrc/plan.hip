@@ -104,7 +104,7 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d != nullptr, "null descriptor");
   WC_CHECK_ARG(d->ndim == 2 || d->ndim == 3, "ndim must be 2 or 3, got %d", d->ndim);
   WC_CHECK_ARG(d->N > 0 && d->C > 0 && d->K > 0, "N, C, K must be positive (%d, %d, %d)", d->N, d->C, d->K);
-  WC_CHECK_ARG(d->dtype == WC_F32 || d->dtype == WC_F16, "unknown dtype %d", d->dtype);
+  WC_CHECK_ARG(d->dtype == WC_F32 || d->dtype == WC_F16 || d->dtype == WC_BF16, "unknown dtype %d", d->dtype);
   for (int a = 0; a < 3; ++a) {
     WC_CHECK_ARG(d->in[a] > 0 && d->kernel[a] > 0 && d->pad[a] >= 0,
                  "axis %d: input %d, kernel %d, pad %d", a, d->in[a], d->kernel[a], d->pad[a]);

@@ -48,6 +48,17 @@ struct alignas(sizeof(T) * N) Pack {
 };
 
 using half_t = _Float16;
+using bf16_t = __bf16;
+
+// f(T{}) with the storage type that `dtype` (a wc_dtype) names
+template <typename F>
+inline auto dispatch_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case WC_F16: return f(half_t{});
+    case WC_BF16: return f(bf16_t{});
+    default: return f(float{});
+  }
+}
 
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;

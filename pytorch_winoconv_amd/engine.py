@@ -10,7 +10,7 @@ import torch
 from . import _lib
 from ._lib import ConvDesc, Plan, check
 
-_DTYPES = {torch.float32: _lib.WC_F32, torch.float16: _lib.WC_F16}
+_DTYPES = {torch.float32: _lib.WC_F32, torch.float16: _lib.WC_F16, torch.bfloat16: _lib.WC_BF16}
 
 
 def _ptr(t):
@@ -28,7 +28,7 @@ def _require_gpu(*tensors):
         if not t.is_cuda:
             raise ValueError("winoconv runs on the GPU only: got a %s tensor" % t.device)
         if t.dtype not in _DTYPES:
-            raise TypeError("winoconv supports float32 and float16, got %s" % t.dtype)
+            raise TypeError("winoconv supports float32, float16 and bfloat16, got %s" % t.dtype)
 
 
 def _triple(v, nd, fill):

@@ -134,6 +134,14 @@ def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
         pkg.WinoConv2d(4, 4, 3, 1, 1)(x)
 
 
+def test_bfloat16_is_a_storage_type():
+    d = engine.make_desc((2, 8, 20, 20), (4, 8, 3, 3), torch.bfloat16, 1, 1, 2)
+    assert d.dtype == _lib.WC_BF16 == 2 and engine.plan_conv(d).t_total == 16
+    d.dtype = 3
+    with pytest.raises(ValueError):
+        engine.plan_conv(d)
+
+
 def test_whole_kernel_plans():
     """One F(2,k) x F(2,k) piece for a k x k kernel (the reference's matrix_conv tile,
     matrix_conv.py:112-135) and the descriptor checks around it."""
