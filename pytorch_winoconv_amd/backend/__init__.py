@@ -106,14 +106,20 @@ def split_and_concat(direction, in_a, out, *args):
     raise ValueError("split_and_concat: direction must be 'split' or 'concat'")
 
 
-def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0):
+def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, algo="dwm", U=None,
+                  chunk_images=0):
     """Whole convolution on channel-last tensors, written into `Output`.
 
     Input (B, D, H, W, C) contiguous; Weight any strided view whose dims are (kD, kH, kW, C, K)
     (the reference's layout, dwm.py:85,133); Output (B, oD, oH, oW, K) contiguous.  A 2-D
     problem has D = kD = 1.  `padding` is (pD, pH, pW) or one int; `m` is the Winograd output
     tile (4 allowed for 2-D 3x3 stride 1); kernels larger than 3 or stride 2 are decomposed
-    (DWM).  `U` is an optional filter transformed earlier by engine.transform_filter."""
+    (algo "dwm"); algo "whole" keeps a square 2-D kernel of 4..7 taps as one F(2,k) x F(2,k) tile,
+    the arithmetic of the reference's matrix_conv path (matrix_conv.py:112-135).  `U` is an
+    optional filter transformed earlier by engine.transform_filter."""
+    if algo not in ("dwm", "whole"):
+        raise ValueError("winograd_conv: algo must be 'dwm' or 'whole', got %r" % (algo,))
+    whole = algo == "whole"
     _require_gpu(Input, Weight, Output, bias, U)
     if Input.dim() != 5 or Weight.dim() != 5 or Output.dim() != 5:
         raise ValueError("winograd_conv: expected 5-D channel-last Input/Output and a 5-D Weight")
@@ -131,9 +137,9 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, U=
         padding = (0 if flat else padding, padding, padding)
     w_kc = Weight.permute(4, 3, 0, 1, 2)                 # (K, C, kD, kH, kW) view, no copy
     if flat:
-        desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images)
+        desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole)
     else:
-        desc = make_desc((B, C, D, H, W), (K, C, kD, kH, kW), Input.dtype, stride, padding, m, chunk_images)
+        desc = make_desc((B, C, D, H, W), (K, C, kD, kH, kW), Input.dtype, stride, padding, m, chunk_images, whole)
     out, _ = out_dims(desc)
     _check_out(Output, (B, out[0], out[1], out[2], K), Input, "winograd_conv")
     nbytes = ctypes.c_size_t()
@@ -153,4 +159,4 @@ def DWM(Input, Weight, Output, stride, tmp_input_buffer=None, tmp_weight_buffer=
     (B, oD, oH, oW, K).  The four scratch tensors of the reference signature are accepted and
     ignored: the engine sizes its own workspace (transformed buffers are laid out differently
     and no pointer table is needed)."""
-    winograd_conv(Input, Weight, Output, None, int(stride), 0, 2)
+    winograd_conv(Input, Weight, Output, None, int(stride), 0, 2, "dwm")

@@ -134,6 +134,16 @@ def test_backend_entry_points_with_reference_layouts(dev):
     out3 = torch.zeros(2, 1, 10, 11, 6, device=dev)
     pkg.DWM(xin, w3.to(dev).unsqueeze(2).permute(2, 3, 4, 1, 0).contiguous(), out3, 1)
     assert _nerr(out3[:, 0].permute(0, 3, 1, 2), F.conv2d(x.double(), w3.double())) < 1e-3
+    # winograd_conv(x, w, out, bias, stride, padding, m, algo): padding, bias, tile 4 and the
+    # whole-kernel algorithm on the same channel-last tensors
+    b = torch.randn(6)
+    refp = F.conv2d(x.double(), w.double(), b.double(), padding=2)
+    for m, algo in ((2, "dwm"), (4, "dwm"), (2, "whole")):
+        o = torch.zeros(2, 1, 12, 13, 6, device=dev)
+        pkg.winograd_conv(xin, win, o, b.to(dev), 1, 2, m, algo)
+        assert _nerr(o[:, 0].permute(0, 3, 1, 2), refp) < 1e-3, (m, algo)
+    with pytest.raises(ValueError):
+        pkg.winograd_conv(xin, win, out, None, 1, 0, 2, "fft")
     # tile copies
     a = xd.permute(0, 2, 3, 1).contiguous()
     tiles = torch.zeros(2 * 5 * 6, 8, 4, 4, device=dev)
