@@ -190,3 +190,46 @@ def test_winoconv3d_module(dev):
     x = torch.randn(1, 8, 6, 10, 10, device=dev)
     ref = F.conv3d(x.double().cpu(), mod.weight.detach().double().cpu(), mod.bias.detach().double().cpu(), padding=1)
     assert _nerr(mod(x), ref) < 1e-3
+
+
+def test_forward_is_capturable_in_a_hip_graph(dev):
+    """The library allocates nothing, never synchronises and takes its stream from the caller, so a
+    whole forward pass (four kernels) can be captured once and replayed.  The graph is replayed
+    three times with new input contents, eager work and synchronisation between the replays, and
+    every replay must equal the eager result bit for bit."""
+    import ctypes
+    from pytorch_winoconv_amd import _lib
+    lib = _lib.load()
+    xs, ws = (2, 32, 20, 20), (48, 32, 5, 5)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(*xs, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    w = (torch.randn(*ws, generator=g) * 0.05).half().to(dev)
+    desc = pkg.engine.make_desc(xs, ws, torch.float16, 1, 2, 4)
+    nbytes = ctypes.c_size_t()
+    _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+    wsp = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+    x_cl = pkg.engine.channel_last(x)
+    y = torch.empty(2, 20, 20, 48, dtype=torch.float16, device=dev)
+    strides = pkg.engine._w_strides(w)
+
+    def forward():
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.wc_conv_forward(ctypes.byref(desc), x_cl.data_ptr(), w.data_ptr(), strides, None, None,
+                                       y.data_ptr(), wsp.data_ptr(), nbytes.value, st))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        forward()                                         # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        forward()
+    for i in range(3):
+        x_cl.copy_(torch.randn(x_cl.shape, generator=g).half().to(dev))
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, 2, 4)     # eager, own buffers
+        assert torch.equal(got.permute(0, 3, 1, 2), want), i
