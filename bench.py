@@ -87,6 +87,7 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
+    ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)xF(4,3)^2", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, "f16"),
     ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
 ]
 VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),

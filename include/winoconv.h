@@ -67,7 +67,7 @@ typedef struct {
   int kernel[3];   /* kD, kH, kW (kD = 1 when ndim == 2)                        */
   int pad[3];      /* symmetric zero padding per axis                           */
   int stride;      /* 1 or 2, same on every axis                                */
-  int m;           /* Winograd output tile: 2, or 4 (2-D problems only)         */
+  int m;           /* Winograd output tile: 2, or 4 (2-D: 4 x 4; 3-D: 2 x 4 x 4, 3x3x3 stride 1 only) */
   int dtype;       /* wc_dtype                                                  */
   int chunk_images;/* images per pass of wc_conv_forward; 0 = choose automatically */
   int whole_kernel;/* 0: kernels > 3 are decomposed into pieces of <= 3 taps (DWM, dwm.py:107-146);

@@ -82,7 +82,9 @@ def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=Fals
         per_axis = [[(0, 1, k)] for k in kernel]
     else:
         per_axis = [axis_pieces(k, stride) for k in kernel]
-    ms = [1 if (ax == 0 and degenerate_depth) else m for ax in range(3)]
+    # m: one output tile extent for all axes, or one per axis (depth, height, width)
+    mt = [m] * 3 if isinstance(m, int) else list(m)
+    ms = [1 if (ax == 0 and degenerate_depth) else mt[ax] for ax in range(3)]
     out, t = [], 0
     for combo in product(*per_axis):
         alphas = [ms[ax] + combo[ax][2] - 1 for ax in range(3)]

@@ -87,6 +87,7 @@ static FilterFastKernel pick_fast(int k0, int k1, int k2) {
   if (k0 == KIND_11 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_11, KIND_43, KIND_43>;
   if (k0 == KIND_11 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_11, KIND_23, KIND_23>;
   if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_23, KIND_23, KIND_23>;
+  if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_23, KIND_43, KIND_43>;
   return nullptr;
 }
 

@@ -1,5 +1,6 @@
 // Host entry of the input transform: picks the kernel of each piece and launches it.
 #include "input_transform_impl.h"
+#include <algorithm>
 
 using namespace wc;
 
@@ -34,6 +35,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   a.total = P * a.n_cvec;
   const long long blocks = ceil_div_ll(a.total, 256);
   a.per_xcd = (int)ceil_div_ll(blocks, kXcds);
+  a.x_bytes = 0;
   WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
   const dim3 launch_grid((unsigned)(a.per_xcd * kXcds));
 
@@ -68,6 +70,35 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       if (k[q] < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[q], pc.r[q]);
     }
     InKernel fn = nullptr;
+    if (!flat && plan->m[1] == 4) {
+      // tile 2 x 4 x 4 of a 3x3x3 kernel: the kernel reads x through a buffer descriptor with 32-bit
+      // offsets, so the batch is cut into launches of images that together stay below 2 GiB
+      if (!(k[0] == KIND_23 && k[1] == KIND_43 && k[2] == KIND_43))
+        return fail(WC_ERR_UNSUPPORTED, "3-D output tile 4 is built for 3x3x3 kernels only");
+      const int v3 = d->dtype == WC_F32 ? 1 : vec;   // channels per thread of this kernel
+      InKernel f3 = pick_in_3d_m4(d->dtype, v3);
+      a.n_cvec = Cp / v3;
+      const long long es = d->dtype == WC_F32 ? 4 : 2;
+      const long long image_bytes = (long long)d->in[0] * d->in[1] * d->in[2] * d->C * es;
+      if (image_bytes >= (1ll << 31))
+        return fail(WC_ERR_UNSUPPORTED, "3-D output tile 4 needs images below 2 GiB (%lld bytes)", image_bytes);
+      const int per_launch = (int)std::max<long long>(1, ((1ll << 31) - 1) / image_bytes);
+      const long long tiles_per_image = (long long)grid[0] * grid[1] * grid[2];
+      a.base0 = pc.tap0[0] - d->pad[0]; a.base1 = pc.tap0[1] - d->pad[1]; a.base2 = pc.tap0[2] - d->pad[2];
+      a.t_offset = pc.t_offset;
+      for (int b0 = 0; b0 < n_images; b0 += per_launch) {
+        const int nb = std::min(per_launch, n_images - b0);
+        InArgs c = a;
+        c.x = static_cast<const char*>(x) + (long long)b0 * image_bytes;
+        c.V = static_cast<char*>(V) + (long long)b0 * tiles_per_image * Cp * es;
+        c.x_bytes = (int)(nb * image_bytes);
+        c.total = (long long)nb * tiles_per_image * c.n_cvec;
+        c.per_xcd = (int)ceil_div_ll(ceil_div_ll(c.total, 256), kXcds);
+        hipLaunchKernelGGL(f3, dim3((unsigned)(c.per_xcd * kXcds)), dim3(256), 0, as_stream(stream), c);
+        WC_CHECK_LAUNCH("input_transform_3d_m4_kernel");
+      }
+      continue;
+    }
     switch (k[0]) {
       case KIND_11: fn = pick_in_2d(d->dtype, k[1], k[2], vec); break;
       case KIND_21: fn = pick_in_3d_21(d->dtype, k[1], k[2], vec); break;

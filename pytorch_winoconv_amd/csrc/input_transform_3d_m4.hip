@@ -1,0 +1,115 @@
+// Input transform for the 3-D tile 2 x 4 x 4 of a 3x3x3 kernel: F(2,3) along depth, F(4,3) along
+// height and width (4 x 6 x 6 = 144 elements per channel).
+//
+// The depth pass of F(2,3) only adds or subtracts two input planes
+//   o0 = p0 - p2,  o1 = p1 + p2,  o2 = p2 - p1,  o3 = p1 - p3      (BT of matrix_conv.py:27-30)
+// so it is done first on two 6 x 6 planes at a time (kept in storage precision until combined),
+// and each resulting plane goes through the height / width passes and is stored at once.  Plane p1
+// is read twice (the second time from cache).
+#include "input_transform_impl.h"
+
+namespace wc {
+
+// VEC consecutive elements through one buffer load: the buffer descriptor carries the base and
+// the size of the input, the per-lane address is one 32-bit offset (half the registers of a 64-bit
+// pointer per load), and an offset beyond the size - which is how a window element outside the
+// image is encoded - reads as zero in hardware, so no select is needed afterwards.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> buffer_load_pack(__amdgpu_buffer_rsrc_t rsrc, unsigned off) {
+  if constexpr (sizeof(T) * VEC == 2) {
+    const unsigned short raw = __builtin_amdgcn_raw_buffer_load_b16(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  } else if constexpr (sizeof(T) * VEC == 4) {
+    const unsigned raw = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  } else {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  }
+}
+
+constexpr unsigned kOutside = 0x80000000u;   // >= the descriptor's size (the host keeps it below 2 GiB)
+
+// One 6 x 6 plane in storage precision (a 16-bit pair stays packed in one register until it is used)
+template <typename T, int VEC>
+__device__ __forceinline__ void load_plane(const InArgs& a, __amdgpu_buffer_rsrc_t rsrc, const InWhere& w, int i0,
+                                           Pack<T, VEC> (&d)[36]) {
+  const int cc = w.c_ok ? w.c : 0;
+  const int z = 2 * w.td + i0 + a.base0;
+  const bool z_ok = w.c_ok && (unsigned)z < (unsigned)a.D;
+  static_for<0, 6>([&](auto i1_) {
+    constexpr int i1 = decltype(i1_)::value;
+    const int yy = 4 * w.th + i1 + a.base1;
+    const bool y_ok = z_ok && (unsigned)yy < (unsigned)a.H;
+    const unsigned row = (((unsigned)w.b * a.D + z) * a.H + yy) * a.W;
+    static_for<0, 6>([&](auto i2_) {
+      constexpr int i2 = decltype(i2_)::value;
+      const int xx = 4 * w.tw + i2 + a.base2;
+      const bool ok = y_ok && (unsigned)xx < (unsigned)a.W;
+      const unsigned off = ok ? ((row + xx) * a.C + cc) * (unsigned)sizeof(T) : kOutside;
+      d[i1 * 6 + i2] = buffer_load_pack<T, VEC>(rsrc, off);
+    });
+  });
+}
+
+// o = sp * p + sq * q in fp32
+template <typename T, int VEC>
+__device__ __forceinline__ void combine(const Pack<T, VEC> (&p)[36], const Pack<T, VEC> (&q)[36], float sp, float sq,
+                                        float (&o)[36][VEC]) {
+#pragma unroll
+  for (int e = 0; e < 36; ++e)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[e][v] = sp * static_cast<float>(p[e].v[v]) + sq * static_cast<float>(q[e].v[v]);
+}
+
+// height / width passes of one plane (in place, `tmp` is scratch) and store as depth element i0
+template <typename T, int VEC>
+__device__ __forceinline__ void finish_plane(const InArgs& a, const InWhere& w, int i0, float (&d)[36][VEC],
+                                             float (&tmp)[36][VEC]) {
+  apply_axis<MatSel<KIND_43, false>, 2, 1, 6, 6, VEC>(d, tmp);
+  apply_axis<MatSel<KIND_43, false>, 1, 1, 6, 6, VEC>(tmp, d);
+  T* V = static_cast<T*>(a.V) + (long long)(a.t_offset + i0 * 36) * a.t_stride + w.p * a.Cp + w.c;
+  static_for<0, 36>([&](auto e_) {
+    constexpr int e = decltype(e_)::value;
+    store_pack<T, VEC>(V + e * a.t_stride, d[e]);
+  });
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256, 2) void input_transform_3d_m4_kernel(InArgs a) {
+  InWhere w;
+  if (!in_decode(a, xcd_remap(blockIdx.x, a.per_xcd), VEC, w)) return;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.x), 0, a.x_bytes, 0x00020000);
+  Pack<T, VEC> p[36], q[36];
+  float o[36][VEC], tmp[36][VEC];
+  load_plane<T, VEC>(a, rsrc, w, 1, p);
+  load_plane<T, VEC>(a, rsrc, w, 2, q);
+  combine<T, VEC>(p, q, 1.f, 1.f, o);            // o1 = p1 + p2
+  finish_plane<T, VEC>(a, w, 1, o, tmp);
+  combine<T, VEC>(p, q, -1.f, 1.f, o);           // o2 = p2 - p1
+  finish_plane<T, VEC>(a, w, 2, o, tmp);
+  // (compiler fences: without them the loads of the later planes are hoisted and the register
+  // count grows to one wavefront per SIMD)
+  asm volatile("" ::: "memory");
+  load_plane<T, VEC>(a, rsrc, w, 0, p);          // q still holds p2
+  combine<T, VEC>(p, q, 1.f, -1.f, o);           // o0 = p0 - p2
+  finish_plane<T, VEC>(a, w, 0, o, tmp);
+  asm volatile("" ::: "memory");
+  load_plane<T, VEC>(a, rsrc, w, 1, p);
+  load_plane<T, VEC>(a, rsrc, w, 3, q);
+  combine<T, VEC>(p, q, 1.f, -1.f, o);           // o3 = p1 - p3
+  finish_plane<T, VEC>(a, w, 3, o, tmp);
+}
+
+InKernel pick_in_3d_m4(int dtype, int vec) {
+  return dispatch_dtype(dtype, [&](auto t) -> InKernel {
+    using T = decltype(t);
+    // 16-bit types: 2 channels per thread (one 4-byte access); fp32: 1
+    if constexpr (sizeof(T) == 2) return vec == 2 ? &input_transform_3d_m4_kernel<T, 2> : &input_transform_3d_m4_kernel<T, 1>;
+    else return &input_transform_3d_m4_kernel<T, 1>;
+  });
+}
+
+}  // namespace wc

@@ -28,6 +28,7 @@ struct InArgs {
   int n_cvec;                // Cp / VEC
   long long total;           // P * n_cvec
   int per_xcd;
+  int x_bytes;               // bytes of the images one launch covers (kernels that read x through a buffer descriptor)
 };
 
 // Tile coordinates and channel offset of one thread
@@ -136,5 +137,6 @@ InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec);    // ... whole-k
 InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
 InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
 InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);
+InKernel pick_in_3d_m4(int dtype, int vec);                       // tile 2 x 4 x 4 of a 3x3x3 kernel, vec 2 or 1
 
 }  // namespace wc

@@ -205,6 +205,50 @@ __global__ __launch_bounds__(256) void output_multi_kernel(OutMultiArgs g) {
   write_tile<T, M0, MO, MO, VEC>(a, w, k, acc);
 }
 
+// ---- 3-D tile 2 x 4 x 4 of a 3x3x3 kernel ---------------------------------------------------------
+// One depth plane (36 elements) at a time: height / width passes of F(4,3), then the plane is
+// added to the two output planes with the coefficients of A^T of F(2,3)
+// ([[1, 1, 1, 0], [0, 1, -1, -1]], matrix_conv.py:21-22).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void output_transform_3d_m4_kernel(OutArgs a) {
+  const int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  const long long idx = (long long)blk * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int k = (int)(idx % a.n_kvec) * VEC;
+  const long long p = idx / a.n_kvec;
+  const Where w = decode_tile(p, a.nD, a.nH, a.nW);
+  const T* M = static_cast<const T*>(a.M) + (long long)a.t_offset * a.t_stride + p * a.ldm + k;
+  float acc[32][VEC];
+#pragma unroll
+  for (int e = 0; e < 32; ++e)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[e][v] = 0.f;
+  static_for<0, 4>([&](auto i0_) {
+    constexpr int i0 = decltype(i0_)::value;
+    float m[36][VEC];
+    static_for<0, 36>([&](auto e_) {
+      constexpr int e = decltype(e_)::value;
+      load_pack<T, VEC>(M + (long long)(i0 * 36 + e) * a.t_stride, m[e]);
+    });
+    float s2[24][VEC];
+    apply_axis<MatSel<KIND_43, true>, 2, 1, 6, 6, VEC>(m, s2);
+    float s1[16][VEC];
+    apply_axis<MatSel<KIND_43, true>, 1, 1, 6, 4, VEC>(s2, s1);
+    constexpr float c0 = Mats<KIND_23>::at(0, i0), c1 = Mats<KIND_23>::at(1, i0);
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        if constexpr (c0 != 0.f) acc[e][v] += c0 * s1[e][v];
+        if constexpr (c1 != 0.f) acc[16 + e][v] += c1 * s1[e][v];
+      }
+    // compiler fence: keeps the loads of the next plane below this point (hoisted, all 144 loads
+    // of the tile are live at once and the kernel runs at one wavefront per SIMD)
+    asm volatile("" ::: "memory");
+  });
+  write_tile<T, 2, 4, 4, VEC>(a, w, k, acc);
+}
+
 // ---- all pieces of a 2-D DWM plan, compile-time body per piece ------------------------------------
 // Each piece is handled like a single-piece plan (all alpha_h x alpha_w loads of the tile issued
 // together, separable AT passes in registers) and added to the m x m accumulators; the piece's
@@ -279,6 +323,8 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
   if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23)
     return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 2>
                     : &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 1>;
+  if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43)
+    return vec == 4 ? &output_transform_3d_m4_kernel<T, 2> : &output_transform_3d_m4_kernel<T, 1>;
   // whole-kernel tiles F(2,r) x F(2,r), r = 4..7
 #define WC_WHOLE(KD) \
   if (k0 == KIND_11 && k1 == KD && k2 == KD) \

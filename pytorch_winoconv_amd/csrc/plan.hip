@@ -121,8 +121,9 @@ static int check_desc(const wc_conv_desc* d) {
     return fail(WC_ERR_UNSUPPORTED, "stride %d not implemented (1 or 2)", d->stride);
   if (d->m != 2 && d->m != 4)
     return fail(WC_ERR_UNSUPPORTED, "output tile %d not implemented (2 or 4)", d->m);
-  if (d->m == 4 && d->ndim != 2)
-    return fail(WC_ERR_UNSUPPORTED, "output tile 4 is implemented for 2-D problems only");
+  if (d->m == 4 && d->ndim == 3 &&
+      !(d->stride == 1 && d->kernel[0] == 3 && d->kernel[1] == 3 && d->kernel[2] == 3))
+    return fail(WC_ERR_UNSUPPORTED, "output tile 4 in 3-D (2 x 4 x 4) is implemented for 3x3x3 kernels at stride 1");
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
   if (d->whole_kernel) {
@@ -150,7 +151,7 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   std::memset(plan, 0, sizeof(*plan));
   plan->tap_step = d->stride;
   const bool flat_depth = (d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0);
-  plan->m[0] = flat_depth ? 1 : d->m;
+  plan->m[0] = flat_depth ? 1 : (d->m == 4 ? 2 : d->m);   // 3-D tile 4 is 2 x 4 x 4
   plan->m[1] = d->m;
   plan->m[2] = d->m;
   int np = 0, t = 0;
@@ -182,7 +183,7 @@ int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
   const bool flat_depth = (d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0);
   for (int a = 0; a < 3; ++a) {
     out[a] = (d->in[a] + 2 * d->pad[a] - d->kernel[a]) / d->stride + 1;
-    int m = (a == 0 && flat_depth) ? 1 : d->m;
+    int m = a == 0 ? (flat_depth ? 1 : (d->m == 4 ? 2 : d->m)) : d->m;
     grid[a] = (out[a] + m - 1) / m;
   }
   return WC_OK;

@@ -82,8 +82,6 @@ def _run(input, kernel, bias, stride, padding, groups, output_block, dtype, deco
     b = None if bias is None else bias.to(dtype)
     s = _same_stride(stride)
     m = int(output_block)
-    if m == 4 and input.dim() != 4:
-        raise NotImplementedError("output_block 4 is available for 2-D convolutions only")
     return engine.conv_forward(x, w, b, s, padding, m, whole_kernel=_whole_kernel(w, s, m, decompose))
 
 

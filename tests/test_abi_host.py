@@ -74,8 +74,8 @@ def test_out_dims_follow_the_reference_arithmetic():
 
 def test_errors_are_status_codes_with_messages_not_exits():
     lib = _lib.load()
-    # unsupported: stride 3, tile 3, kernel extent 11, tile 4 in 3-D
-    for kw in (dict(stride=3), dict(m=3), dict(w=(4, 4, 11, 3)), dict(m=4, x=(1, 4, 9, 20, 20), w=(4, 4, 3, 3, 3))):
+    # unsupported: stride 3, tile 3, kernel extent 11, tile 4 in 3-D for a kernel that is not 3x3x3
+    for kw in (dict(stride=3), dict(m=3), dict(w=(4, 4, 11, 3)), dict(m=4, x=(1, 4, 9, 20, 20), w=(4, 4, 3, 3, 5))):
         desc = engine.make_desc(kw.get("x", (1, 4, 20, 20)), kw.get("w", (4, 4, 3, 3)), torch.float32,
                                 kw.get("stride", 1), 0, kw.get("m", 2))
         with pytest.raises(NotImplementedError):
@@ -140,6 +140,17 @@ def test_bfloat16_is_a_storage_type():
     d.dtype = 3
     with pytest.raises(ValueError):
         engine.plan_conv(d)
+
+
+def test_3d_tile_4_is_2x4x4_for_3x3x3_only():
+    d = engine.make_desc((2, 8, 7, 18, 21), (4, 8, 3, 3, 3), torch.float16, 1, 1, 4)
+    plan = engine.plan_conv(d)
+    assert list(plan.m) == [2, 4, 4] and plan.n_pieces == 1 and plan.t_total == 4 * 6 * 6
+    out, grid = engine.out_dims(d)
+    assert out == [7, 18, 21] and grid == [4, 5, 6]
+    for ws, stride in (((4, 8, 5, 5, 5), 1), ((4, 8, 3, 3, 3), 2), ((4, 8, 1, 3, 3), 1)):
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(engine.make_desc((2, 8, 7, 18, 21), ws, torch.float16, stride, 1, 4))
 
 
 def test_whole_kernel_plans():

@@ -38,6 +38,7 @@ CONFIGS = [
     ("c4 3x3 s2", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, H16),
     ("c4 7x7 s2", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, H16),
     ("c5 3-D", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, H16),
+    ("c5 3-D tile 2x4x4", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, H16),
 ]
 
 

@@ -70,6 +70,8 @@ CASES = [
     ((2, 8, 6, 9, 11), (8, 8, 3, 3, 3), 1, 1, 2),
     ((1, 4, 7, 9, 8), (4, 4, 5, 5, 5), 1, 2, 2),
     ((1, 6, 6, 8, 8), (5, 6, 2, 3, 1), 1, 0, 2),
+    ((2, 8, 6, 9, 11), (8, 8, 3, 3, 3), 1, 1, 4),       # 3-D tile 2 x 4 x 4
+    ((1, 5, 5, 10, 7), (6, 5, 3, 3, 3), 1, 0, 4),
     # whole-kernel tiles F(2,k) x F(2,k) (sixth entry), the reference's matrix_conv arithmetic
     ((2, 8, 12, 13), (8, 8, 4, 4), 1, 1, 2, True),
     ((2, 6, 12, 13), (8, 6, 5, 5), 1, 2, 2, True),
@@ -93,7 +95,8 @@ def _setup(case, dtype, dev, seed=0, integer=False):
         w = torch.randn(*ws, generator=g) * (2.0 / fan_in) ** 0.5
     x, w = x.to(dtype), w.to(dtype)
     stages = {}
-    ow.dwm_conv(x, w, None, stride, pad, m, DISC[dtype], stages, whole_kernel=whole)
+    om = (2, 4, 4) if (m == 4 and len(xs) == 5) else m        # the engine's 3-D "tile 4" is 2 x 4 x 4
+    ow.dwm_conv(x, w, None, stride, pad, om, DISC[dtype], stages, whole_kernel=whole)
     desc = engine.make_desc(xs, ws, dtype, stride, pad, m, whole_kernel=whole)
     plan = engine.plan_conv(desc)
     return x, w, stages, desc, plan
