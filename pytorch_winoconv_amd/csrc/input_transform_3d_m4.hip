@@ -53,26 +53,58 @@ __device__ __forceinline__ void load_plane(const InArgs& a, __amdgpu_buffer_rsrc
   });
 }
 
-// o = sp * p + sq * q in fp32
+// One output depth plane: o = sp * p + sq * q (fp32), width pass row by row as the rows are
+// combined, height pass column by column with each result stored at once - the fp32 copy of the
+// combined plane never exists as a whole.
 template <typename T, int VEC>
-__device__ __forceinline__ void combine(const Pack<T, VEC> (&p)[36], const Pack<T, VEC> (&q)[36], float sp, float sq,
-                                        float (&o)[36][VEC]) {
+__device__ __forceinline__ void emit_plane(const InArgs& a, const InWhere& w, int i0, const Pack<T, VEC> (&p)[36],
+                                           const Pack<T, VEC> (&q)[36], float sp, float sq) {
+  using BT = MatSel<KIND_43, false>;
+  float t[36][VEC];
+  static_for<0, 6>([&](auto r_) {
+    constexpr int r = decltype(r_)::value;
+    float in[6][VEC];
 #pragma unroll
-  for (int e = 0; e < 36; ++e)
+    for (int i = 0; i < 6; ++i)
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) o[e][v] = sp * static_cast<float>(p[e].v[v]) + sq * static_cast<float>(q[e].v[v]);
-}
-
-// height / width passes of one plane (in place, `tmp` is scratch) and store as depth element i0
-template <typename T, int VEC>
-__device__ __forceinline__ void finish_plane(const InArgs& a, const InWhere& w, int i0, float (&d)[36][VEC],
-                                             float (&tmp)[36][VEC]) {
-  apply_axis<MatSel<KIND_43, false>, 2, 1, 6, 6, VEC>(d, tmp);
-  apply_axis<MatSel<KIND_43, false>, 1, 1, 6, 6, VEC>(tmp, d);
+      for (int v = 0; v < VEC; ++v)
+        in[i][v] = sp * static_cast<float>(p[r * 6 + i].v[v]) + sq * static_cast<float>(q[r * 6 + i].v[v]);
+    static_for<0, 6>([&](auto j_) {
+      constexpr int j = decltype(j_)::value;
+      constexpr int first = BT::first_nz(j);
+      static_for<0, 6>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        constexpr float c = BT::get(j, i);
+        if constexpr (c != 0.f) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            if constexpr (i == first) t[r * 6 + j][v] = c * in[i][v];
+            else t[r * 6 + j][v] = __builtin_fmaf(c, in[i][v], t[r * 6 + j][v]);
+          }
+        }
+      });
+    });
+  });
   T* V = static_cast<T*>(a.V) + (long long)(a.t_offset + i0 * 36) * a.t_stride + w.p * a.Cp + w.c;
-  static_for<0, 36>([&](auto e_) {
-    constexpr int e = decltype(e_)::value;
-    store_pack<T, VEC>(V + e * a.t_stride, d[e]);
+  static_for<0, 6>([&](auto j_) {           // column j of the plane
+    constexpr int j = decltype(j_)::value;
+    static_for<0, 6>([&](auto o_) {         // output row o
+      constexpr int o = decltype(o_)::value;
+      constexpr int first = BT::first_nz(o);
+      float acc[VEC];
+      static_for<0, 6>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        constexpr float c = BT::get(o, i);
+        if constexpr (c != 0.f) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            if constexpr (i == first) acc[v] = c * t[i * 6 + j][v];
+            else acc[v] = __builtin_fmaf(c, t[i * 6 + j][v], acc[v]);
+          }
+        }
+      });
+      store_pack<T, VEC>(V + (long long)(o * 6 + j) * a.t_stride, acc);
+    });
   });
 }
 
@@ -83,24 +115,19 @@ __global__ __launch_bounds__(256, 2) void input_transform_3d_m4_kernel(InArgs a)
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.x), 0, a.x_bytes, 0x00020000);
   Pack<T, VEC> p[36], q[36];
-  float o[36][VEC], tmp[36][VEC];
   load_plane<T, VEC>(a, rsrc, w, 1, p);
   load_plane<T, VEC>(a, rsrc, w, 2, q);
-  combine<T, VEC>(p, q, 1.f, 1.f, o);            // o1 = p1 + p2
-  finish_plane<T, VEC>(a, w, 1, o, tmp);
-  combine<T, VEC>(p, q, -1.f, 1.f, o);           // o2 = p2 - p1
-  finish_plane<T, VEC>(a, w, 2, o, tmp);
+  emit_plane<T, VEC>(a, w, 1, p, q, 1.f, 1.f);    // o1 = p1 + p2
+  emit_plane<T, VEC>(a, w, 2, p, q, -1.f, 1.f);   // o2 = p2 - p1
   // (compiler fences: without them the loads of the later planes are hoisted and the register
   // count grows to one wavefront per SIMD)
   asm volatile("" ::: "memory");
-  load_plane<T, VEC>(a, rsrc, w, 0, p);          // q still holds p2
-  combine<T, VEC>(p, q, 1.f, -1.f, o);           // o0 = p0 - p2
-  finish_plane<T, VEC>(a, w, 0, o, tmp);
+  load_plane<T, VEC>(a, rsrc, w, 0, p);           // q still holds p2
+  emit_plane<T, VEC>(a, w, 0, p, q, 1.f, -1.f);   // o0 = p0 - p2
   asm volatile("" ::: "memory");
   load_plane<T, VEC>(a, rsrc, w, 1, p);
   load_plane<T, VEC>(a, rsrc, w, 3, q);
-  combine<T, VEC>(p, q, 1.f, -1.f, o);           // o3 = p1 - p3
-  finish_plane<T, VEC>(a, w, 3, o, tmp);
+  emit_plane<T, VEC>(a, w, 3, p, q, 1.f, -1.f);   // o3 = p1 - p3
 }
 
 InKernel pick_in_3d_m4(int dtype, int vec) {
