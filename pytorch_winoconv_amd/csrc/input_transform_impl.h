@@ -137,6 +137,6 @@ InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec);    // ... whole-k
 InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
 InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
 InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);
-InKernel pick_in_3d_m4(int dtype, int vec);                       // tile 2 x 4 x 4 of a 3x3x3 kernel, vec 2 or 1
+InKernel pick_in_3d_planes(int dtype, int vec);                   // tile 2 x 4 x 4 of a 3x3x3 kernel, plane by plane, vec 2 or 1
 
 }  // namespace wc
