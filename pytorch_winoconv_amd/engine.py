@@ -174,6 +174,11 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
+    if x.shape[0] == 0:
+        # empty batch: the shape arithmetic is checked on one image, nothing is launched
+        out, _ = out_dims(make_desc((1,) + tuple(x.shape[1:]), w.shape, x.dtype, stride, padding, m, 0, whole_kernel))
+        osp = out[1:] if x.dim() == 4 else out
+        return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
     desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images, whole_kernel)
     out, _ = out_dims(desc)
     x_cl = channel_last(x)

@@ -194,3 +194,19 @@ def test_channels_last_input_and_cached_filter(dev):
     y1 = engine.conv_forward(xcl, w.to(dev), b.to(dev), 1, 1, 4, U=U)
     assert torch.equal(y0, y1)
     assert y1.is_contiguous(memory_format=torch.channels_last)
+
+
+def test_empty_batch_and_single_pixel_outputs(dev):
+    """Empty input (N = 0) gives an empty output of the right shape, like torch; outputs of one
+    pixel and inputs smaller than a tile are handled by the edge rules."""
+    w = torch.randn(6, 4, 3, 3).half().to(dev)
+    y = engine.conv_forward(torch.empty(0, 4, 9, 7, dtype=torch.float16, device=dev), w, None, 1, 1, 4)
+    assert tuple(y.shape) == (0, 6, 9, 7) and y.dtype == torch.float16
+    y3 = engine.conv_forward(torch.empty(0, 4, 5, 9, 7, device=dev), torch.randn(6, 4, 3, 3, 3, device=dev), None, 2, 1, 2)
+    assert tuple(y3.shape) == (0, 6, 3, 5, 4)
+    for xs, ws, stride, pad, m in (((2, 4, 3, 3), (6, 4, 3, 3), 1, 0, 4), ((1, 4, 1, 1), (6, 4, 3, 3), 1, 1, 2),
+                                   ((2, 4, 7, 7), (6, 4, 7, 7), 2, 0, 4), ((1, 4, 2, 3, 3), (6, 4, 3, 3, 3), 1, (1, 0, 0), 2)):
+        x, wt, b = _data(xs, ws, torch.float32)
+        ref = _conv64(x, wt, b, stride, pad)
+        yy = engine.conv_forward(x.to(dev), wt.to(dev), b.to(dev), stride, pad, m)
+        assert tuple(yy.shape) == tuple(ref.shape) and _nerr(yy, ref) <= 1e-3
