@@ -156,6 +156,19 @@ int wc_conv_forward(const wc_conv_desc* desc, const void* x,
                     const void* w, const int64_t w_strides[5], const void* U_cached,
                     const void* bias, void* y, void* workspace, size_t workspace_bytes,
                     void* stream);
+
+/* ---- weight gradient -------------------------------------------------------------------------- */
+/* No counterpart in the reference: it never implemented a backward pass (only a pointer-assign
+ * helper exists for one, src/back/utils.cu:15-24; include/split_functions_grad.h:3-6 is empty).
+ * dw[k][c][taps] = gradient of sum(y * dy) with respect to the filter, for the same descriptor as
+ * the forward call: x (N, D, H, W, C) and dy (N, oD, oH, oW, K) channel-last contiguous, dw written
+ * through element strides for the axes (K, C, kD, kH, kW).  Computed in the transform domain
+ * (dU = sum over tiles of dM x V, dw = G^T dU G) with every sum in fp32.  The input gradient needs
+ * no entry point of its own: it is wc_conv_forward of dy with the flipped, transposed filter. */
+int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
+int wc_conv_backward_weight(const wc_conv_desc* desc, const void* x, const void* dy, void* dw,
+                            const int64_t dw_strides[5], void* workspace, size_t workspace_bytes,
+                            void* stream);
 #ifdef __cplusplus
 }
 #endif

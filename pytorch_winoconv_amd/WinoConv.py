@@ -41,6 +41,31 @@ class Wino:
         return self._mod(input).conv(input, kernel, output_block, stride, fp16)
 
 
+class WinoConvFunction(torch.autograd.Function):
+    """conv_forward with gradients.  The reference has no backward pass (src/back/ holds only a
+    pointer-assign helper, src/back/utils.cu:15-24); here the input gradient is a convolution run by
+    the same engine and the weight gradient is computed in the transform domain."""
+
+    @staticmethod
+    def forward(ctx, x, w, bias, stride, padding, m, U):
+        ctx.save_for_backward(x, w)
+        ctx.conf = (stride, padding, m, bias is not None)
+        return engine.conv_forward(x, w, bias, stride, padding, m, U=U)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        stride, padding, m, has_bias = ctx.conf
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = engine.conv_backward_input(dy, w, x.shape[2:], stride, padding, m)
+        if ctx.needs_input_grad[1]:
+            dw = engine.conv_backward_weight(x, dy, w.shape, stride, padding, m)
+        if has_bias and ctx.needs_input_grad[2]:
+            db = dy.sum(dim=[0] + list(range(2, dy.dim())))
+        return dx, dw, db, None, None, None, None
+
+
 class _WinoConvNd(nn.Module):
     nd = 2
 
@@ -90,6 +115,8 @@ class _WinoConvNd(nn.Module):
             U = engine.transform_filter(w.detach(), x.shape, self.stride[0], self.padding, m)
             self._cache = (key, U)
         b = None if self.bias is None else self.bias.to(x.dtype)
+        if torch.is_grad_enabled() and (x.requires_grad or w.requires_grad or (b is not None and b.requires_grad)):
+            return WinoConvFunction.apply(x, w, b, self.stride[0], self.padding, m, self._cache[1])
         return engine.conv_forward(x, w.detach(), b, self.stride[0], self.padding, m, U=self._cache[1])
 
 

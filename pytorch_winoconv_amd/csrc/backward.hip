@@ -1,0 +1,464 @@
+// Weight gradient of the Winograd / DWM convolution, in the transform domain.
+//
+// The reference never implemented a backward pass (it holds only a pointer-assign helper for one,
+// src/back/utils.cu:15-24, and an empty header, include/split_functions_grad.h:3-6).  With
+// y = sum over pieces of A^T [ (G g G^T) . (B^T d B) ] A, the gradient with respect to g is
+//
+//   dU[t][k][c] = sum over tiles p of dM[t][p][k] * V[t][p][c]     dM = A dy A^T per tile
+//   dg          = G^T dU G                                         per piece, onto its taps
+//
+// V is the forward input transform (same kernels).  dM comes from a small gather kernel, the
+// contraction over the tiles runs on the batched GEMM after both operands have been transposed to
+// tile-contiguous fp32 (the sum over up to millions of tiles is kept in fp32 from the first
+// product to the last addition, whatever the storage type), and a last kernel applies G^T . G and
+// accumulates over image chunks.  Plain design throughout: this path is not performance-critical.
+#include "wc_transform.h"
+#include <algorithm>
+
+namespace wc {
+
+__device__ __forceinline__ int dev_kind_of(int m, int r) {
+  return m == 1 ? KIND_11 : (m == 4 ? (r == 3 ? KIND_43 : r == 2 ? KIND_42 : KIND_41)
+                                   : (r <= 3 ? KIND_21 + (r - 1) : KIND_24 + (r - 4)));
+}
+
+struct GradOutArgs {
+  const void* dy;
+  void* dM;
+  int oD, oH, oW, K, ldm;
+  int nD, nH, nW;
+  long long P;
+  int m[3];
+  int n_pieces;
+  long long total;           // T * P * ldm
+  wc_piece piece[WC_MAX_PIECES];
+};
+
+// dM[t][p][k] = sum_a AT[a0][i0] AT[a1][i1] AT[a2][i2] dy[b, m0 td + a0, m1 th + a1, m2 tw + a2, k]
+template <typename T>
+__global__ __launch_bounds__(256) void grad_output_transform_kernel(const GradOutArgs a) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int k = (int)(idx % a.ldm);
+  long long q = idx / a.ldm;
+  const long long p = q % a.P;
+  const int t = (int)(q / a.P);
+  T* dM = static_cast<T*>(a.dM);
+  if (k >= a.K) { dM[idx] = static_cast<T>(0.f); return; }
+  int s = 0;
+  while (s + 1 < a.n_pieces && a.piece[s + 1].t_offset <= t) ++s;
+  const wc_piece& pc = a.piece[s];
+  const int e = t - pc.t_offset;
+  const int a1n = a.m[1] + pc.r[1] - 1, a2n = a.m[2] + pc.r[2] - 1;
+  const int i2 = e % a2n, i1 = (e / a2n) % a1n, i0 = e / (a2n * a1n);
+  const int k0 = dev_kind_of(a.m[0], pc.r[0]), k1 = dev_kind_of(a.m[1], pc.r[1]), k2 = dev_kind_of(a.m[2], pc.r[2]);
+  const int tw = (int)(p % a.nW); long long r = p / a.nW;
+  const int th = (int)(r % a.nH); r /= a.nH;
+  const int td = (int)(r % a.nD);
+  const long long b = r / a.nD;
+  const T* dy = static_cast<const T*>(a.dy);
+  float acc = 0.f;
+  for (int a0 = 0; a0 < a.m[0]; ++a0) {
+    const int od = a.m[0] * td + a0;
+    if (od >= a.oD) continue;
+    const float c0 = table_at(k0, a0, i0);
+    for (int a1 = 0; a1 < a.m[1]; ++a1) {
+      const int oh = a.m[1] * th + a1;
+      if (oh >= a.oH) continue;
+      const float c01 = c0 * table_at(k1, a1, i1);
+      for (int a2 = 0; a2 < a.m[2]; ++a2) {
+        const int ow = a.m[2] * tw + a2;
+        if (ow >= a.oW) continue;
+        const float c = c01 * table_at(k2, a2, i2);
+        if (c != 0.f)
+          acc = __builtin_fmaf(c, static_cast<float>(dy[(((b * a.oD + od) * a.oH + oh) * a.oW + ow) * a.K + k]), acc);
+      }
+    }
+  }
+  dM[idx] = static_cast<T>(acc);
+}
+
+// A (alpha x m) = transpose of A^T, as an apply_axis matrix
+template <int KIND>
+struct MatA {
+  static constexpr int rows = Mats<KIND>::alpha;
+  static constexpr int cols = Mats<KIND>::m;
+  __host__ __device__ static constexpr float get(int i, int j) { return Mats<KIND>::at(j, i); }
+  __host__ __device__ static constexpr int first_nz(int i) {
+    for (int j = 0; j < cols; ++j)
+      if (get(i, j) != 0.f) return j;
+    return cols;
+  }
+};
+
+// The same for plans whose pieces have 1..3 taps per axis (every DWM plan): a thread owns one tile x
+// VEC output channels, loads its m^d values of dy once and writes dM = (A x A x A) dy for every
+// piece; the piece's taps select a compile-time body (a branch that is uniform over the launch).
+// M0 x MO x MO is the output tile: 1 x 2 x 2, 1 x 4 x 4, 2 x 2 x 2 or 2 x 4 x 4.
+template <typename T, int M0, int MO, int VEC>
+__global__ __launch_bounds__(256) void grad_output_pieces_kernel(const GradOutArgs a) {
+  const int n_kvec = a.ldm / VEC;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.P * n_kvec) return;
+  const int k = (int)(idx % n_kvec) * VEC;
+  const long long p = idx / n_kvec;
+  const int tw = (int)(p % a.nW); long long r = p / a.nW;
+  const int th = (int)(r % a.nH); r /= a.nH;
+  const int td = (int)(r % a.nD);
+  const long long b = r / a.nD;
+  const T* dy = static_cast<const T*>(a.dy);
+  const bool k_ok = k < a.K;                       // ldm - K padding columns are written as zeros
+  float g[M0 * MO * MO][VEC];
+  static_for<0, M0>([&](auto a0_) {
+    constexpr int a0 = decltype(a0_)::value;
+    const int od = M0 * td + a0;
+    static_for<0, MO>([&](auto a1_) {
+      constexpr int a1 = decltype(a1_)::value;
+      const int oh = MO * th + a1;
+      static_for<0, MO>([&](auto a2_) {
+        constexpr int a2 = decltype(a2_)::value;
+        const int ow = MO * tw + a2;
+        constexpr int e = (a0 * MO + a1) * MO + a2;
+        const bool ok = k_ok && od < a.oD && oh < a.oH && ow < a.oW;
+        const long long off = (((b * a.oD + min(od, a.oD - 1)) * a.oH + min(oh, a.oH - 1)) * a.oW + min(ow, a.oW - 1)) * a.K + (k_ok ? k : 0);
+        if constexpr (VEC == 1) {
+          g[e][0] = ok ? static_cast<float>(dy[off]) : 0.f;
+        } else {
+          load_pack<T, VEC>(dy + off, g[e]);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) g[e][v] = ok ? g[e][v] : 0.f;
+        }
+      });
+    });
+  });
+  T* dM = static_cast<T*>(a.dM) + p * a.ldm + k;
+  const long long t_stride = a.P * a.ldm;
+  auto piece = [&](auto k0_, auto k1_, auto k2_, int t_offset) {
+    constexpr int K0 = decltype(k0_)::value, K1 = decltype(k1_)::value, K2 = decltype(k2_)::value;
+    constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
+    float s2[M0 * MO * A2][VEC];
+    apply_axis<MatA<K2>, 2, M0, MO, MO, VEC>(g, s2);
+    float s1[M0 * A1 * A2][VEC];
+    apply_axis<MatA<K1>, 1, M0, MO, A2, VEC>(s2, s1);
+    T* out = dM + (long long)t_offset * t_stride;
+    if constexpr (M0 > 1) {
+      float s0[A0 * A1 * A2][VEC];
+      apply_axis<MatA<K0>, 0, M0, A1, A2, VEC>(s1, s0);
+      static_for<0, A0 * A1 * A2>([&](auto e_) {
+        constexpr int e = decltype(e_)::value;
+        store_pack<T, VEC>(out + e * t_stride, s0[e]);
+      });
+    } else {
+      static_for<0, A1 * A2>([&](auto e_) {
+        constexpr int e = decltype(e_)::value;
+        store_pack<T, VEC>(out + e * t_stride, s1[e]);
+      });
+    }
+  };
+  constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
+  using IA = ic<KA>; using IB = ic<KB>; using IC = ic<KC>;
+  for (int s = 0; s < a.n_pieces; ++s) {
+    const wc_piece& pc = a.piece[s];
+    const int t0 = pc.t_offset;
+    if constexpr (M0 == 1) {
+#define WC_ROW(I1) \
+  switch (pc.r[2]) { case 1: piece(ic<KIND_11>{}, I1{}, IA{}, t0); break; case 2: piece(ic<KIND_11>{}, I1{}, IB{}, t0); break; \
+                     default: piece(ic<KIND_11>{}, I1{}, IC{}, t0); }
+      switch (pc.r[1]) { case 1: WC_ROW(IA) break; case 2: WC_ROW(IB) break; default: WC_ROW(IC) }
+#undef WC_ROW
+    } else if constexpr (MO == 4) {
+      piece(ic<KIND_23>{}, IC{}, IC{}, t0);        // the only 3-D plan with tile 4: one 3x3x3 piece
+    } else {
+#define WC_ROW(I0, I1) \
+  switch (pc.r[2]) { case 1: piece(I0{}, I1{}, IA{}, t0); break; case 2: piece(I0{}, I1{}, IB{}, t0); break; \
+                     default: piece(I0{}, I1{}, IC{}, t0); }
+#define WC_PLANE(I0) \
+  switch (pc.r[1]) { case 1: WC_ROW(I0, IA) break; case 2: WC_ROW(I0, IB) break; default: WC_ROW(I0, IC) }
+      switch (pc.r[0]) { case 1: WC_PLANE(IA) break; case 2: WC_PLANE(IB) break; default: WC_PLANE(IC) }
+#undef WC_PLANE
+#undef WC_ROW
+    }
+  }
+}
+
+// src (T, P, ld) of type T -> dst (T, S, n, Pq) fp32: dst[t][s][j][q] = src[t][s Pq + q][j], zero
+// where s Pq + q >= P.  64 x 64 tiles through LDS; grid (ceil(n / 64), S * Pq / 64, T).
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_to_f32_kernel(const T* __restrict__ src, float* __restrict__ dst,
+                                                               long long P, int ld, int n, int S, int Pq) {
+  __shared__ float tile[64][65];
+  const int j0 = blockIdx.x * 64;
+  const int qblocks = Pq / 64;
+  const int s = blockIdx.y / qblocks, q0 = (blockIdx.y % qblocks) * 64;
+  const int t = blockIdx.z;
+  const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
+  const T* st = src + (long long)t * P * ld;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = ly + 4 * i;                       // tile-local p
+    const long long p = (long long)s * Pq + q0 + row;
+    const int j = j0 + lx;
+    tile[row][lx] = (p < P && j < n) ? static_cast<float>(st[p * ld + j]) : 0.f;
+  }
+  __syncthreads();
+  float* dt = dst + (((long long)t * S + s) * n) * Pq;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int jrow = ly + 4 * i;
+    const int j = j0 + jrow;
+    if (j < n) dt[(long long)j * Pq + q0 + lx] = tile[lx][jrow];
+  }
+}
+
+struct GradFilterArgs {
+  const float* dU;           // (T, S, K, ldc)
+  float* acc;                // (taps, K, C) running sum over image chunks
+  int K, C, ldc, S;
+  int kernel[3];
+  int step;
+  int m[3];
+  int n_pieces;
+  int first;                 // 1: overwrite acc, 0: add to it
+  long long total;           // taps * K * C
+  wc_piece piece[WC_MAX_PIECES];
+};
+
+// acc[tap][k][c] (+)= sum_i G[i0][j0] G[i1][j1] G[i2][j2] sum_s dU[t_off + e(i)][s][k][c] for the piece owning the tap
+__global__ __launch_bounds__(256) void grad_filter_transform_kernel(const GradFilterArgs a) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.total) return;
+  const int c = (int)(idx % a.C);
+  long long q = idx / a.C;
+  const int k = (int)(q % a.K);
+  const int tap = (int)(q / a.K);
+  const int x2 = tap % a.kernel[2], x1 = (tap / a.kernel[2]) % a.kernel[1], x0 = tap / (a.kernel[2] * a.kernel[1]);
+  // the piece that owns this tap and the tap's index inside it
+  int s = -1, j0 = 0, j1 = 0, j2 = 0;
+  for (int i = 0; i < a.n_pieces && s < 0; ++i) {
+    const wc_piece& pc = a.piece[i];
+    const int d0 = x0 - pc.tap0[0], d1 = x1 - pc.tap0[1], d2 = x2 - pc.tap0[2];
+    if (d0 < 0 || d1 < 0 || d2 < 0 || d0 % a.step || d1 % a.step || d2 % a.step) continue;
+    j0 = d0 / a.step; j1 = d1 / a.step; j2 = d2 / a.step;
+    if (j0 < pc.r[0] && j1 < pc.r[1] && j2 < pc.r[2]) s = i;
+  }
+  float val = 0.f;
+  if (s >= 0) {
+    const wc_piece& pc = a.piece[s];
+    const int n0 = a.m[0] + pc.r[0] - 1, n1 = a.m[1] + pc.r[1] - 1, n2 = a.m[2] + pc.r[2] - 1;
+    const int k0 = dev_kind_of(a.m[0], pc.r[0]), k1 = dev_kind_of(a.m[1], pc.r[1]), k2 = dev_kind_of(a.m[2], pc.r[2]);
+    for (int i0 = 0; i0 < n0; ++i0) {
+      const float g0 = table_g(k0, i0, j0);
+      if (g0 == 0.f) continue;
+      for (int i1 = 0; i1 < n1; ++i1) {
+        const float g01 = g0 * table_g(k1, i1, j1);
+        if (g01 == 0.f) continue;
+        for (int i2 = 0; i2 < n2; ++i2) {
+          const float g = g01 * table_g(k2, i2, j2);
+          if (g == 0.f) continue;
+          const long long t = pc.t_offset + (i0 * n1 + i1) * n2 + i2;
+          float u = 0.f;
+          for (int sp = 0; sp < a.S; ++sp) u += a.dU[((t * a.S + sp) * a.K + k) * a.ldc + c];
+          val = __builtin_fmaf(g, u, val);
+        }
+      }
+    }
+  }
+  a.acc[idx] = a.first ? val : a.acc[idx] + val;
+}
+
+// dw[k][c][tap] through element strides <- acc (taps, K, C)
+template <typename T>
+__global__ __launch_bounds__(256) void grad_filter_store_kernel(const float* __restrict__ acc, T* __restrict__ dw,
+                                                               long long s0, long long s1, long long s2, long long s3,
+                                                               long long s4, int K, int C, int kD, int kH, int kW,
+                                                               long long total) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)(idx % C);
+  long long q = idx / C;
+  const int k = (int)(q % K);
+  const int tap = (int)(q / K);
+  const int x2 = tap % kW, x1 = (tap / kW) % kH, x0 = tap / (kW * kH);
+  dw[k * s0 + c * s1 + x0 * s2 + x1 * s3 + x2 * s4] = static_cast<T>(acc[idx]);
+}
+
+}  // namespace wc
+
+using namespace wc;
+
+namespace {
+
+size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+struct BwdLayout {
+  wc_plan plan;
+  int out[3], grid[3];
+  int Cp, ldm, ldc, chunk, S, Pq;
+  long long tiles_per_image;
+  size_t es;
+  size_t v_bytes, dm_bytes, vt_bytes, dmt_bytes, du_bytes, acc_bytes;
+};
+
+int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
+  int rc = wc_plan_conv(d, &L->plan);
+  if (rc) return rc;
+  rc = wc_conv_out_dims(d, L->out, L->grid);
+  if (rc) return rc;
+  if (L->plan.t_total > 0xffff) return fail(WC_ERR_UNSUPPORTED, "plan with %d transform elements is too large", L->plan.t_total);
+  L->Cp = wc_padded_channels(d->C);
+  L->ldm = wc_padded_channels8(d->K);
+  L->ldc = wc_padded_channels8(d->C);
+  L->es = d->dtype == WC_F32 ? 4 : 2;
+  L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
+  const long long T = L->plan.t_total;
+  // images per pass: the four large buffers of one pass stay below about 2 GiB
+  const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * (L->es + 4.0) * 1.1;
+  int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(2048.0 * 1024 * 1024 / per_image);
+  chunk = std::max(1, std::min(chunk, d->N));
+  L->chunk = chunk;
+  const long long Pc = L->tiles_per_image * chunk;
+  if (Pc >= (1ll << 31)) return fail(WC_ERR_UNSUPPORTED, "chunk of %d images has too many tiles", chunk);
+  // split of the tile axis: enough 64 x 64 output tiles for the whole chip, every part >= 64 tiles
+  const long long tiles = T * ((d->K + 63) / 64) * ((d->C + 63) / 64);
+  long long S = (1024 + tiles - 1) / tiles;
+  S = std::max(1ll, std::min(S, std::min(64ll, (Pc + 63) / 64)));
+  L->S = (int)S;
+  L->Pq = (int)(((Pc + S - 1) / S + 63) / 64 * 64);
+  L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
+  L->dm_bytes = round256((size_t)T * Pc * L->ldm * L->es);
+  L->vt_bytes = round256((size_t)T * S * d->C * L->Pq * 4);
+  L->dmt_bytes = round256((size_t)T * S * d->K * L->Pq * 4);
+  L->du_bytes = round256((size_t)T * S * d->K * L->ldc * 4);
+  L->acc_bytes = round256((size_t)d->kernel[0] * d->kernel[1] * d->kernel[2] * d->K * d->C * 4);
+  return WC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* d, size_t* bytes) {
+  WC_CHECK_ARG(bytes != nullptr, "wc_conv_backward_weight_workspace_bytes: null output");
+  BwdLayout L;
+  int rc = make_bwd_layout(d, &L);
+  if (rc) return rc;
+  *bytes = L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes + L.acc_bytes;
+  return WC_OK;
+}
+
+int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy, void* dw,
+                            const int64_t dw_strides[5], void* workspace, size_t workspace_bytes, void* stream) {
+  BwdLayout L;
+  int rc = make_bwd_layout(d, &L);
+  if (rc) return rc;
+  WC_CHECK_ARG(x && dy && dw && dw_strides, "wc_conv_backward_weight: null pointer");
+  if (!workspace) return fail(WC_ERR_WORKSPACE, "wc_conv_backward_weight: null workspace");
+  const size_t need = L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes + L.acc_bytes;
+  if (workspace_bytes < need)
+    return fail(WC_ERR_WORKSPACE, "wc_conv_backward_weight: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
+    return fail(WC_ERR_WORKSPACE, "wc_conv_backward_weight: workspace must be 256-byte aligned");
+  hipStream_t s = as_stream(stream);
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  void* V = ws;
+  void* dM = ws + L.v_bytes;
+  float* Vt = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes);
+  float* dMt = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes);
+  float* dU = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes);
+  float* acc = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes);
+  const int T = L.plan.t_total;
+  const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L.es;
+  const size_t y_image = (size_t)L.out[0] * L.out[1] * L.out[2] * d->K * L.es;
+  const int taps = d->kernel[0] * d->kernel[1] * d->kernel[2];
+
+  for (int b0 = 0; b0 < d->N; b0 += L.chunk) {
+    const int n = std::min(L.chunk, d->N - b0);
+    const long long P = L.tiles_per_image * n;
+    rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);
+    if (rc) return rc;
+    {
+      GradOutArgs a;
+      a.dy = static_cast<const unsigned char*>(dy) + b0 * y_image;
+      a.dM = dM;
+      a.oD = L.out[0]; a.oH = L.out[1]; a.oW = L.out[2]; a.K = d->K; a.ldm = L.ldm;
+      a.nD = L.grid[0]; a.nH = L.grid[1]; a.nW = L.grid[2];
+      a.P = P;
+      for (int i = 0; i < 3; ++i) a.m[i] = L.plan.m[i];
+      a.n_pieces = L.plan.n_pieces;
+      for (int i = 0; i < L.plan.n_pieces; ++i) a.piece[i] = L.plan.piece[i];
+      a.total = (long long)T * P * L.ldm;
+      const long long blocks = ceil_div_ll(a.total, 256);
+      WC_CHECK_ARG(blocks < (1ll << 31), "wc_conv_backward_weight: problem too large");
+      bool small_taps = true;
+      for (int i = 0; i < L.plan.n_pieces; ++i)
+        for (int q = 0; q < 3; ++q) small_taps = small_taps && L.plan.piece[i].r[q] <= 3;
+      const int m0 = L.plan.m[0], mo = L.plan.m[1];
+      void (*fn)(GradOutArgs) = nullptr;
+      long long threads = a.total;
+      if (small_taps && L.plan.m[2] == mo && (mo == 2 || mo == 4) && (m0 == 1 || m0 == 2)) {
+        // 2 channels per thread when K is even, except for the 144-element tile of the 3-D tile 4
+        const int vec = ((m0 == 2 && mo == 4) || d->K % 2) ? 1 : 2;
+        threads = P * (L.ldm / vec);
+        fn = dispatch_dtype(d->dtype, [&](auto t) -> void (*)(GradOutArgs) {
+          using TT = decltype(t);
+          if (m0 == 2 && mo == 4) return &grad_output_pieces_kernel<TT, 2, 4, 1>;
+          if (vec == 2) {
+            if (m0 == 1) return mo == 4 ? &grad_output_pieces_kernel<TT, 1, 4, 2> : &grad_output_pieces_kernel<TT, 1, 2, 2>;
+            return &grad_output_pieces_kernel<TT, 2, 2, 2>;
+          }
+          if (m0 == 1) return mo == 4 ? &grad_output_pieces_kernel<TT, 1, 4, 1> : &grad_output_pieces_kernel<TT, 1, 2, 1>;
+          return &grad_output_pieces_kernel<TT, 2, 2, 1>;
+        });
+      } else {
+        fn = dispatch_dtype(d->dtype, [](auto t) -> void (*)(GradOutArgs) {
+          return &grad_output_transform_kernel<decltype(t)>;
+        });
+      }
+      const long long nblocks = ceil_div_ll(threads, 256);
+      hipLaunchKernelGGL(fn, dim3((unsigned)nblocks), dim3(256), 0, s, a);
+      WC_CHECK_LAUNCH("grad_output_transform_kernel");
+    }
+    // the part length of this pass (the last pass may hold fewer images)
+    const int Pq = (int)(((P + L.S - 1) / L.S + 63) / 64 * 64);
+    dispatch_dtype(d->dtype, [&](auto t) {
+      using TT = decltype(t);
+      const dim3 gv((unsigned)ceil_div(d->C, 64), (unsigned)(L.S * (Pq / 64)), (unsigned)T);
+      hipLaunchKernelGGL(transpose_to_f32_kernel<TT>, gv, dim3(256), 0, s, static_cast<const TT*>(V), Vt, P, L.Cp,
+                         d->C, L.S, Pq);
+      const dim3 gm((unsigned)ceil_div(d->K, 64), (unsigned)(L.S * (Pq / 64)), (unsigned)T);
+      hipLaunchKernelGGL(transpose_to_f32_kernel<TT>, gm, dim3(256), 0, s, static_cast<const TT*>(dM), dMt, P, L.ldm,
+                         d->K, L.S, Pq);
+      return 0;
+    });
+    WC_CHECK_LAUNCH("transpose_to_f32_kernel");
+    // dU[(t, s)] (K x C) = dMt[(t, s)] (K x Pq) . Vt[(t, s)] (C x Pq)^T, fp32
+    rc = wc_batched_gemm(dMt, Vt, dU, T * L.S, d->K, Pq, d->C, L.ldc, WC_F32, stream);
+    if (rc) return rc;
+    {
+      GradFilterArgs g;
+      g.dU = dU; g.acc = acc;
+      g.K = d->K; g.C = d->C; g.ldc = L.ldc; g.S = L.S;
+      for (int i = 0; i < 3; ++i) { g.kernel[i] = d->kernel[i]; g.m[i] = L.plan.m[i]; }
+      g.step = L.plan.tap_step;
+      g.n_pieces = L.plan.n_pieces;
+      for (int i = 0; i < L.plan.n_pieces; ++i) g.piece[i] = L.plan.piece[i];
+      g.first = b0 == 0;
+      g.total = (long long)taps * d->K * d->C;
+      hipLaunchKernelGGL(grad_filter_transform_kernel, dim3((unsigned)ceil_div_ll(g.total, 256)), dim3(256), 0, s, g);
+      WC_CHECK_LAUNCH("grad_filter_transform_kernel");
+    }
+  }
+  const long long total = (long long)taps * d->K * d->C;
+  dispatch_dtype(d->dtype, [&](auto t) {
+    using TT = decltype(t);
+    hipLaunchKernelGGL(grad_filter_store_kernel<TT>, dim3((unsigned)ceil_div_ll(total, 256)), dim3(256), 0, s, acc,
+                       static_cast<TT*>(dw), (long long)dw_strides[0], (long long)dw_strides[1],
+                       (long long)dw_strides[2], (long long)dw_strides[3], (long long)dw_strides[4], d->K, d->C,
+                       d->kernel[0], d->kernel[1], d->kernel[2], total);
+    return 0;
+  });
+  WC_CHECK_LAUNCH("grad_filter_store_kernel");
+  return WC_OK;
+}
+
+}  // extern "C"

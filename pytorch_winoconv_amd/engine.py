@@ -194,3 +194,65 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_cl), _ptr(w), _w_strides(w), _ptr(U),
                               _ptr(bias), _ptr(y), _ptr(ws), nbytes.value, _stream(x)))
     return channel_first_view(y)
+
+
+# ---------------------------------------------------------------- gradients
+def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
+    """Gradient of sum(y * dy) with respect to the filter of conv_forward(x, w, ...): a tensor of
+    shape `w_shape` (K, C, [kD,] kH, kW) in x's dtype.  The reference has no backward pass; this one
+    works in the transform domain (see include/winoconv.h)."""
+    _require_gpu(x, dy)
+    if dy.dtype != x.dtype:
+        raise TypeError("x and dy must share one dtype")
+    lib = _lib.load()
+    desc = make_desc(x.shape, w_shape, x.dtype, stride, padding, m, 0, whole_kernel)
+    out, _ = out_dims(desc)
+    osp = out[1:] if desc.ndim == 2 else out
+    if tuple(dy.shape) != (x.shape[0], w_shape[0]) + tuple(osp):
+        raise ValueError("dy has shape %r, the convolution gives %r"
+                         % (tuple(dy.shape), (x.shape[0], w_shape[0]) + tuple(osp)))
+    dw = torch.empty(tuple(w_shape), dtype=x.dtype, device=x.device)
+    if x.shape[0] == 0:
+        return dw.zero_()
+    x_cl, dy_cl = channel_last(x), channel_last(dy)
+    nbytes = ctypes.c_size_t()
+    check(lib.wc_conv_backward_weight_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+    check(lib.wc_conv_backward_weight(ctypes.byref(desc), _ptr(x_cl), _ptr(dy_cl), _ptr(dw), _w_strides(dw),
+                                      _ptr(ws), nbytes.value, _stream(x)))
+    return dw
+
+
+def conv_backward_input(dy, w, x_spatial, stride=1, padding=0, m=2):
+    """Gradient of sum(y * dy) with respect to the input: the convolution of dy (with zeros between
+    its elements when stride is 2) with the filter flipped along every spatial axis and its two
+    channel axes exchanged, padded by k - 1 - p - so it runs through conv_forward."""
+    _require_gpu(dy, w)
+    nd = w.dim() - 2
+    ks = tuple(w.shape[2:])
+    pads = _triple(padding, nd, 0)[3 - nd:]
+    if isinstance(stride, (tuple, list)):
+        stride = int(stride[0])
+    if any(k - 1 - p < 0 for k, p in zip(ks, pads)):
+        raise NotImplementedError("input gradient needs padding <= kernel - 1 on every axis")
+    want = tuple(int(v) for v in x_spatial)
+    if stride == 2:
+        # zeros between the elements of dy, and at the end as many as it takes for the result to have
+        # the input's extent (one more when the strided forward pass left an odd remainder)
+        up = [X - (k - 1 - 2 * p) for X, k, p in zip(want, ks, pads)]
+        if any(u < 2 * (o - 1) + 1 for u, o in zip(up, dy.shape[2:])):
+            raise ValueError("dy of shape %r does not belong to an input of extent %r" % (tuple(dy.shape), want))
+        dyu = torch.zeros(tuple(dy.shape[:2]) + tuple(up), dtype=dy.dtype, device=dy.device)
+        dyu[(slice(None), slice(None)) + tuple(slice(0, 2 * (o - 1) + 1, 2) for o in dy.shape[2:])] = dy
+        dy = dyu
+    elif stride != 1:
+        raise NotImplementedError("stride must be 1 or 2")
+    w_rot = w.flip(tuple(range(2, 2 + nd))).transpose(0, 1)
+    # output tile: the caller's, except where the 3-D tile 4 does not exist and for stride 2, where
+    # three quarters of the zero-filled dy are zeros and the F(4,r) rounding error is not averaged
+    # down (fp16: 2.6e-2 of the gradient's range against 2e-3 with tile 2)
+    mm = m if (stride == 1 and (m == 2 or nd == 2 or ks == (3, 3, 3))) else 2
+    dx = conv_forward(dy, w_rot, None, 1, tuple(k - 1 - p for k, p in zip(ks, pads)), mm)
+    if tuple(dx.shape[2:]) != want:
+        raise ValueError("dy of shape %r does not belong to an input of extent %r" % (tuple(dy.shape), want))
+    return dx
