@@ -28,8 +28,8 @@ def test_rule_reproduces_every_lut_key(key):
 
 def test_kernel_stride_and_total_follow_the_launcher():
     """kernel_stride is the running sum of prod(size + 1) (base_conv_launchers.cu:307-313); the
-    totals the survey quotes: 7x7 -> 200 and 5x5 -> 98 with the reference's doubled depth,
-    3x3x3 -> 64."""
+    totals that follow from the table by hand: 7x7 -> 9 boxes of (1+1)(a+1)(b+1) = 200 and 5x5 -> 98
+    with the reference's doubled depth, 3x3x3 -> 4^3 = 64."""
     p = sp.split_plan(1, 7, 7)
     assert p["kernel_stride"] == [0, 32, 64, 80, 112, 144, 160, 176, 192] and p["T_total"] == 200
     assert sp.split_plan(1, 5, 5)["T_total"] == 98
