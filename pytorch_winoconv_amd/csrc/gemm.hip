@@ -9,8 +9,9 @@
 // Workgroup = 4 wavefronts (2 x 2), each owning WM x WN MFMA blocks of 32 x 32, so the
 // macro tile is (64 WM) tiles x (64 WN) output channels.  Operand tiles go global -> registers ->
 // LDS with two LDS stages (one barrier per reduction step; the global loads of step k+1 are in
-// flight while step k is multiplied).  LDS rows are padded by 16 bytes, which makes the 16-byte
-// fragment reads of 8 consecutive rows hit 32 distinct banks.  The MFMA "A" operand is the
+// flight while step k is multiplied).  LDS rows are 64 bytes with their 16-byte chunks swizzled
+// by row, which keeps both the row-wise stores and the column-wise fragment reads free of bank
+// conflicts.  The MFMA "A" operand is the
 // filter block and "B" the input block: a lane then holds 4 consecutive output channels of
 // one tile row per accumulator group and stores them as one 8-byte (fp16) / 16-byte (fp32)
 // write.  fp16 and bf16 accumulate in fp32; fp32 uses v_mfma_f32_32x32x2_f32.
@@ -22,6 +23,7 @@ namespace wc {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 template <typename T> struct Mfma;
 template <> struct Mfma<half_t> {
@@ -40,12 +42,17 @@ template <> struct Mfma<bf16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
+// fp32: a lane reads four consecutive reduction elements with one 16-byte LDS access and feeds
+// them to four v_mfma_f32_32x32x2_f32, each of which pairs element e of the lower lanes' chunk
+// with element e of the upper lanes' chunk (4 elements further along the reduction axis).
 template <> struct Mfma<float> {
-  using Frag = float;
-  static constexpr int kpack = 1;
-  static constexpr int kstep = 2;
+  using Frag = floatx4;
+  static constexpr int kpack = 4;
+  static constexpr int kstep = 8;
   __device__ static __forceinline__ floatx16 run(Frag a, Frag b, floatx16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    return c;
   }
 };
 
@@ -61,6 +68,13 @@ struct GemmArgs {
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
 
+// Operand rows in LDS are 64 bytes (four 16-byte chunks) with no padding; chunk c of row r sits
+// at position c ^ swizzle(r).  A workgroup pass writes whole rows, so stores touch every bank
+// once.  Fragment reads take the same chunk of consecutive rows: the swizzle gives rows of equal
+// r mod 2 among 8 consecutive rows, and rows of equal r mod 4 among 16, distinct positions, which
+// is conflict-free for 128-byte and for 256-byte wide bank sets alike.
+__device__ __forceinline__ int swizzle(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
+
 template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2>
 __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
   using MF = Mfma<T>;
@@ -68,12 +82,13 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
   constexpr int EPC = 16 / sizeof(T);              // elements per 16-byte chunk
   constexpr int CPR = BK / EPC;                    // chunks per tile row
-  constexpr int LDS_STRIDE = BK + EPC;             // padded row, elements
+  constexpr int LDS_STRIDE = BK;                   // unpadded row; the chunks of a row are swizzled
   constexpr int ROWS = BM + BN;
   constexpr int RPP = NT / CPR;                    // rows covered by one pass of the workgroup
   constexpr int NLOAD = ROWS / RPP;
   constexpr int STAGE = ROWS * LDS_STRIDE;         // elements per LDS stage
   static_assert(ROWS % RPP == 0 && BM % RPP == 0, "tile rows must be a multiple of the load pass");
+  static_assert(CPR == 4 && RPP % 16 == 0, "the swizzle assumes 64-byte rows and passes of whole 16-row groups");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -102,7 +117,7 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
       const int k = min(k0 + row - BM, g.K - 1);
       gptr[i] = Ut + (long long)k * g.Cp + lpart * EPC;
     }
-    loff[i] = row * LDS_STRIDE + lpart * EPC;
+    loff[i] = row * LDS_STRIDE + (lpart ^ swizzle(row)) * EPC;
   }
 
   Chunk16 regs[NLOAD];
@@ -118,9 +133,14 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave / NWK, wk = wave % NWK;
   const int l32 = lane & 31, lhi = lane >> 5;
-  // fragment read offsets inside a stage (elements)
-  const int xoff = (wp * WM * 32 + l32) * LDS_STRIDE + lhi * MF::kpack;
-  const int woff = (BM + wk * WN * 32 + l32) * LDS_STRIDE + lhi * MF::kpack;
+  // fragment read offsets inside a stage (elements); all rows a lane reads share l32's swizzle
+  const int xoff = (wp * WM * 32 + l32) * LDS_STRIDE;
+  const int woff = (BM + wk * WN * 32 + l32) * LDS_STRIDE;
+  const int fz = swizzle(l32);
+  auto koff = [&](int kk) {                        // element kk*kstep + lhi*kpack of a swizzled row
+    const int e = kk * MF::kstep + lhi * MF::kpack;
+    return (((e / EPC) ^ fz) * EPC) + e % EPC;
+  };
 
   floatx16 acc[WM][WN];
 #pragma unroll
@@ -142,12 +162,13 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
     constexpr int KK = BK / MF::kstep;
     typename MF::Frag xf[2][WM], wf[2][WN];
     auto fload = [&](int kk, int b) {
+      const int ko = koff(kk);
 #pragma unroll
       for (int i = 0; i < WM; ++i)
-        xf[b][i] = *reinterpret_cast<const typename MF::Frag*>(st + xoff + i * 32 * LDS_STRIDE + kk * MF::kstep);
+        xf[b][i] = *reinterpret_cast<const typename MF::Frag*>(st + xoff + i * 32 * LDS_STRIDE + ko);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
-        wf[b][j] = *reinterpret_cast<const typename MF::Frag*>(st + woff + j * 32 * LDS_STRIDE + kk * MF::kstep);
+        wf[b][j] = *reinterpret_cast<const typename MF::Frag*>(st + woff + j * 32 * LDS_STRIDE + ko);
     };
     fload(0, 0);
 #pragma unroll
@@ -219,7 +240,7 @@ static GemmConfig make_config() {
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
   constexpr int EI = sizeof(T) == 4 ? 1 : (NWP * NWK == 4 ? WM : WM / 2);
-  constexpr size_t stages = (size_t)2 * (BM + BN) * (BK + EPC) * sizeof(T);
+  constexpr size_t stages = (size_t)2 * (BM + BN) * BK * sizeof(T);
   constexpr size_t out_tile = (size_t)32 * NWP * EI * (BN + EPC) * sizeof(T);
   return GemmConfig{&gemm_kernel<T, WM, WN, BK, NWP, NWK>, BM, BN, BK,
                     stages > out_tile ? stages : out_tile, 64 * NWP * NWK};
@@ -281,7 +302,12 @@ static GemmConfig choose(int T_, int P, int K, int Cp) {
     if (i >= 0 && i < Configs<T>::n) return Configs<T>::get(i);
   }
   constexpr int n_auto = 5;
-  // (a reduction of <= 64 channels is one or two stages: the same argument holds for fp16)
+  // fp32 is bound by the MFMA rate: the 64 x 64 tile fills the chip best, except for long
+  // reductions with thousands of tiles, where 128 x 128 halves the LDS traffic (measured 5-9 %
+  // faster at Cp >= 256).  A reduction of <= 64 channels is one or two stages: small tiles again.
+  if constexpr (sizeof(T) == 4) {
+    if (Cp >= 256 && K >= 128 && (long long)ceil_div(P, 128) * ceil_div(K, 128) * T_ >= 2048) return Configs<T>::get(1);
+  }
   if (sizeof(T) == 4 || Cp <= 64) return Configs<T>::get(n_auto - 1);
   // Long reductions over many output channels: the 128 x 256 tile of eight wavefronts reads V
   // once per 256 channels (measured 3-13 % faster than any four-wavefront tile for Cp >= 512).
