@@ -32,6 +32,7 @@ sys.path.insert(0, ROOT)
 
 N, C, K, H, W, R, PAD, M_TILE = 64, 256, 256, 56, 56, 3, 1, 4
 MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
+HBM_PEAK_GB_S = 8000.0              # MI355X published HBM3E bandwidth
 # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116734 KiB, x2.00 by the copy
 # probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
 # profiles/conv3x3_f16_n64_c256_56x56_all_kernels.md.
@@ -230,6 +231,11 @@ def main():
     gemm_flops = 2.0 * T * P * C * K
     gemm_tflops = gemm_flops / (stage_us["batched_gemm"] * 1e-6) / 1e12
     es = 2
+    # The GEMM's algorithmic bytes (V and U read once, M written once): at 127 flop/byte the
+    # kernel sits left of the ridge of the MI355X roofline (2500 TFLOP/s / 8 TB/s = 312 flop/byte),
+    # so the HBM view is reported beside the MFMA one.
+    gemm_bytes = (V.numel() + U.numel() + Mb.numel()) * es
+    gemm_gb_s = gemm_bytes / (stage_us["batched_gemm"] * 1e-6) / 1e9
     hbm = {
         "input_transform": (x.numel() + V.numel()) * es,
         "output_transform": (Mb.numel() + y.numel()) * es,
@@ -248,7 +254,9 @@ def main():
         "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": MFMA_FP16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP16_PEAK_TFLOPS,
                      "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "wc::gemm_kernel (batched_gemm)",
-                     "flops_per_launch": gemm_flops, "avg_us": stage_us["batched_gemm"]},
+                     "flops_per_launch": gemm_flops, "avg_us": stage_us["batched_gemm"],
+                     "hbm_view": {"bytes_per_launch": gemm_bytes, "achieved": gemm_gb_s, "peak": HBM_PEAK_GB_S,
+                                  "unit": "GB/s", "frac": gemm_gb_s / HBM_PEAK_GB_S}},
         "stage_us": stage_us,
         "stage_hbm_tb_s": {k: v / (stage_us[k] * 1e-6) / 1e12 for k, v in hbm.items()},
         "ms_per_layer_one_call": ms_one_call,
