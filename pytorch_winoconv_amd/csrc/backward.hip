@@ -9,9 +9,9 @@
 //
 // V is the forward input transform (same kernels).  dM comes from a small gather kernel, the
 // contraction over the tiles runs on the batched GEMM after both operands have been transposed to
-// tile-contiguous fp32 (the sum over up to millions of tiles is kept in fp32 from the first
-// product to the last addition, whatever the storage type), and a last kernel applies G^T . G and
-// accumulates over image chunks.  Plain design throughout: this path is not performance-critical.
+// tile-contiguous order (in their storage type; the products of 16-bit operands are exact in fp32
+// and the sum over up to millions of tiles is kept in fp32 from the first product to the last
+// addition), and a last kernel applies G^T . G and accumulates over image chunks.
 #include "wc_transform.h"
 #include <algorithm>
 
@@ -181,89 +181,20 @@ __global__ __launch_bounds__(256) void grad_output_pieces_kernel(const GradOutAr
   }
 }
 
-// src (T, P, ld) of type T -> dst (T, S, n, Pq) fp32: dst[t][s][j][q] = src[t][s Pq + q][j], zero
-// where s Pq + q >= P.  64 x 64 tiles through LDS; grid (ceil(n / 64), S * Pq / 64, T).
-template <typename T>
-__global__ __launch_bounds__(256) void transpose_to_f32_kernel(const T* __restrict__ src, float* __restrict__ dst,
-                                                               long long P, int ld, int n, int S, int Pq) {
-  __shared__ float tile[64][65];
-  const int j0 = blockIdx.x * 64;
-  const int qblocks = Pq / 64;
-  const int s = blockIdx.y / qblocks, q0 = (blockIdx.y % qblocks) * 64;
-  const int t = blockIdx.z;
-  const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
-  const T* st = src + (long long)t * P * ld;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int row = ly + 4 * i;                       // tile-local p
-    const long long p = (long long)s * Pq + q0 + row;
-    const int j = j0 + lx;
-    tile[row][lx] = (p < P && j < n) ? static_cast<float>(st[p * ld + j]) : 0.f;
-  }
-  __syncthreads();
-  float* dt = dst + (((long long)t * S + s) * n) * Pq;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int jrow = ly + 4 * i;
-    const int j = j0 + jrow;
-    if (j < n) dt[(long long)j * Pq + q0 + lx] = tile[lx][jrow];
-  }
-}
-
-struct GradFilterArgs {
-  const float* dU;           // (T, S, K, ldc)
-  float* acc;                // (taps, K, C) running sum over image chunks
-  int K, C, ldc, S;
-  int kernel[3];
-  int step;
-  int m[3];
-  int n_pieces;
-  int first;                 // 1: overwrite acc, 0: add to it
-  long long total;           // taps * K * C
-  wc_piece piece[WC_MAX_PIECES];
-};
-
-// acc[tap][k][c] (+)= sum_i G[i0][j0] G[i1][j1] G[i2][j2] sum_s dU[t_off + e(i)][s][k][c] for the piece owning the tap
-__global__ __launch_bounds__(256) void grad_filter_transform_kernel(const GradFilterArgs a) {
+// dU[t][0][i] = sum over s of dU[t][s][i], i in [0, n): the parts of the split reduction, added in
+// a fixed order.  4 elements per thread; n is a multiple of 4.
+__global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ dU, int S, long long n, long long total4) {
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= a.total) return;
-  const int c = (int)(idx % a.C);
-  long long q = idx / a.C;
-  const int k = (int)(q % a.K);
-  const int tap = (int)(q / a.K);
-  const int x2 = tap % a.kernel[2], x1 = (tap / a.kernel[2]) % a.kernel[1], x0 = tap / (a.kernel[2] * a.kernel[1]);
-  // the piece that owns this tap and the tap's index inside it
-  int s = -1, j0 = 0, j1 = 0, j2 = 0;
-  for (int i = 0; i < a.n_pieces && s < 0; ++i) {
-    const wc_piece& pc = a.piece[i];
-    const int d0 = x0 - pc.tap0[0], d1 = x1 - pc.tap0[1], d2 = x2 - pc.tap0[2];
-    if (d0 < 0 || d1 < 0 || d2 < 0 || d0 % a.step || d1 % a.step || d2 % a.step) continue;
-    j0 = d0 / a.step; j1 = d1 / a.step; j2 = d2 / a.step;
-    if (j0 < pc.r[0] && j1 < pc.r[1] && j2 < pc.r[2]) s = i;
+  if (idx >= total4) return;
+  const long long n4 = n / 4;
+  const long long t = idx / n4, i = (idx % n4) * 4;
+  float* base = dU + t * S * n + i;
+  float4 sum = *reinterpret_cast<const float4*>(base);
+  for (int sp = 1; sp < S; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(base + sp * n);
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
   }
-  float val = 0.f;
-  if (s >= 0) {
-    const wc_piece& pc = a.piece[s];
-    const int n0 = a.m[0] + pc.r[0] - 1, n1 = a.m[1] + pc.r[1] - 1, n2 = a.m[2] + pc.r[2] - 1;
-    const int k0 = dev_kind_of(a.m[0], pc.r[0]), k1 = dev_kind_of(a.m[1], pc.r[1]), k2 = dev_kind_of(a.m[2], pc.r[2]);
-    for (int i0 = 0; i0 < n0; ++i0) {
-      const float g0 = table_g(k0, i0, j0);
-      if (g0 == 0.f) continue;
-      for (int i1 = 0; i1 < n1; ++i1) {
-        const float g01 = g0 * table_g(k1, i1, j1);
-        if (g01 == 0.f) continue;
-        for (int i2 = 0; i2 < n2; ++i2) {
-          const float g = g01 * table_g(k2, i2, j2);
-          if (g == 0.f) continue;
-          const long long t = pc.t_offset + (i0 * n1 + i1) * n2 + i2;
-          float u = 0.f;
-          for (int sp = 0; sp < a.S; ++sp) u += a.dU[((t * a.S + sp) * a.K + k) * a.ldc + c];
-          val = __builtin_fmaf(g, u, val);
-        }
-      }
-    }
-  }
-  a.acc[idx] = a.first ? val : a.acc[idx] + val;
+  *reinterpret_cast<float4*>(base) = sum;
 }
 
 // dw[k][c][tap] through element strides <- acc (taps, K, C)
@@ -296,7 +227,7 @@ struct BwdLayout {
   int Cp, ldm, ldc, chunk, S, Pq;
   long long tiles_per_image;
   size_t es;
-  size_t v_bytes, dm_bytes, vt_bytes, dmt_bytes, du_bytes, acc_bytes;
+  size_t v_bytes, dm_bytes, du_bytes, acc_bytes;
 };
 
 int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
@@ -312,22 +243,21 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
   const long long T = L->plan.t_total;
   // images per pass: the four large buffers of one pass stay below about 2 GiB
-  const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * (L->es + 4.0) * 1.1;
+  const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es * 1.1;
   int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(2048.0 * 1024 * 1024 / per_image);
   chunk = std::max(1, std::min(chunk, d->N));
   L->chunk = chunk;
   const long long Pc = L->tiles_per_image * chunk;
   if (Pc >= (1ll << 31)) return fail(WC_ERR_UNSUPPORTED, "chunk of %d images has too many tiles", chunk);
-  // split of the tile axis: enough 64 x 64 output tiles for the whole chip, every part >= 64 tiles
-  const long long tiles = T * ((d->K + 63) / 64) * ((d->C + 63) / 64);
+  // split of the tile axis: about four workgroups of the product per CU, every part >= 256 tiles
+  const int bt = (d->K > 64 && d->C > 64) ? 128 : 64;
+  const long long tiles = T * ((d->K + bt - 1) / bt) * ((d->C + bt - 1) / bt);
   long long S = (1024 + tiles - 1) / tiles;
-  S = std::max(1ll, std::min(S, std::min(64ll, (Pc + 63) / 64)));
+  S = std::max(1ll, std::min(S, std::min(64ll, Pc / 256)));
   L->S = (int)S;
-  L->Pq = (int)(((Pc + S - 1) / S + 63) / 64 * 64);
+  L->Pq = (int)(((Pc + S - 1) / S + 31) / 32 * 32);
   L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
   L->dm_bytes = round256((size_t)T * Pc * L->ldm * L->es);
-  L->vt_bytes = round256((size_t)T * S * d->C * L->Pq * 4);
-  L->dmt_bytes = round256((size_t)T * S * d->K * L->Pq * 4);
   L->du_bytes = round256((size_t)T * S * d->K * L->ldc * 4);
   L->acc_bytes = round256((size_t)d->kernel[0] * d->kernel[1] * d->kernel[2] * d->K * d->C * 4);
   return WC_OK;
@@ -342,7 +272,7 @@ int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* d, size_t* bytes
   BwdLayout L;
   int rc = make_bwd_layout(d, &L);
   if (rc) return rc;
-  *bytes = L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes + L.acc_bytes;
+  *bytes = L.v_bytes + L.dm_bytes + L.du_bytes + L.acc_bytes;
   return WC_OK;
 }
 
@@ -353,7 +283,7 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
   if (rc) return rc;
   WC_CHECK_ARG(x && dy && dw && dw_strides, "wc_conv_backward_weight: null pointer");
   if (!workspace) return fail(WC_ERR_WORKSPACE, "wc_conv_backward_weight: null workspace");
-  const size_t need = L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes + L.acc_bytes;
+  const size_t need = L.v_bytes + L.dm_bytes + L.du_bytes + L.acc_bytes;
   if (workspace_bytes < need)
     return fail(WC_ERR_WORKSPACE, "wc_conv_backward_weight: workspace of %zu bytes, %zu needed", workspace_bytes, need);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
@@ -362,10 +292,8 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   void* V = ws;
   void* dM = ws + L.v_bytes;
-  float* Vt = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes);
-  float* dMt = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes);
-  float* dU = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes);
-  float* acc = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.vt_bytes + L.dmt_bytes + L.du_bytes);
+  float* dU = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes);
+  float* acc = reinterpret_cast<float*>(ws + L.v_bytes + L.dm_bytes + L.du_bytes);
   const int T = L.plan.t_total;
   const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L.es;
   const size_t y_image = (size_t)L.out[0] * L.out[1] * L.out[2] * d->K * L.es;
@@ -419,34 +347,18 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
       WC_CHECK_LAUNCH("grad_output_transform_kernel");
     }
     // the part length of this pass (the last pass may hold fewer images)
-    const int Pq = (int)(((P + L.S - 1) / L.S + 63) / 64 * 64);
-    dispatch_dtype(d->dtype, [&](auto t) {
-      using TT = decltype(t);
-      const dim3 gv((unsigned)ceil_div(d->C, 64), (unsigned)(L.S * (Pq / 64)), (unsigned)T);
-      hipLaunchKernelGGL(transpose_to_f32_kernel<TT>, gv, dim3(256), 0, s, static_cast<const TT*>(V), Vt, P, L.Cp,
-                         d->C, L.S, Pq);
-      const dim3 gm((unsigned)ceil_div(d->K, 64), (unsigned)(L.S * (Pq / 64)), (unsigned)T);
-      hipLaunchKernelGGL(transpose_to_f32_kernel<TT>, gm, dim3(256), 0, s, static_cast<const TT*>(dM), dMt, P, L.ldm,
-                         d->K, L.S, Pq);
-      return 0;
-    });
-    WC_CHECK_LAUNCH("transpose_to_f32_kernel");
-    // dU[(t, s)] (K x C) = dMt[(t, s)] (K x Pq) . Vt[(t, s)] (C x Pq)^T, fp32
-    rc = wc_batched_gemm(dMt, Vt, dU, T * L.S, d->K, Pq, d->C, L.ldc, WC_F32, stream);
+    const int Pq = (int)(((P + L.S - 1) / L.S + 31) / 32 * 32);
+    // dU[(t, s)] (K x C, fp32) = sum over the tiles of part s of dM[t][p][.] (x) V[t][p][.]: operands in
+    // the storage type (their values already are), products summed in fp32
+    rc = batched_gemm_tn(dM, V, dU, T, P, L.ldm, L.Cp, d->K, d->C, L.ldc, L.S, Pq, d->dtype, stream);
     if (rc) return rc;
-    {
-      GradFilterArgs g;
-      g.dU = dU; g.acc = acc;
-      g.K = d->K; g.C = d->C; g.ldc = L.ldc; g.S = L.S;
-      for (int i = 0; i < 3; ++i) { g.kernel[i] = d->kernel[i]; g.m[i] = L.plan.m[i]; }
-      g.step = L.plan.tap_step;
-      g.n_pieces = L.plan.n_pieces;
-      for (int i = 0; i < L.plan.n_pieces; ++i) g.piece[i] = L.plan.piece[i];
-      g.first = b0 == 0;
-      g.total = (long long)taps * d->K * d->C;
-      hipLaunchKernelGGL(grad_filter_transform_kernel, dim3((unsigned)ceil_div_ll(g.total, 256)), dim3(256), 0, s, g);
-      WC_CHECK_LAUNCH("grad_filter_transform_kernel");
+    if (L.S > 1) {
+      const long long n = (long long)d->K * L.ldc, total4 = (long long)T * n / 4;
+      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)ceil_div_ll(total4, 256)), dim3(256), 0, s, dU, L.S, n, total4);
+      WC_CHECK_LAUNCH("sum_parts_kernel");
     }
+    rc = grad_filter_transform(d, &L.plan, dU, acc, L.ldc, L.S, b0 == 0, stream);
+    if (rc) return rc;
   }
   const long long total = (long long)taps * d->K * d->C;
   dispatch_dtype(d->dtype, [&](auto t) {

@@ -70,4 +70,14 @@ __device__ __forceinline__ int xcd_remap(int hw_id, int per_xcd) {
   return (hw_id % kXcds) * per_xcd + hw_id / kXcds;
 }
 
+// acc (taps, K, C) (+)= G^T dU G per piece of the plan; dU (T, S, K, ldc) with the parts already
+// summed into part 0; `first` overwrites acc instead of adding (backward_filter.hip).
+int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const float* dU, float* acc, int ldc, int S,
+                          bool first, void* stream);
+
+// D[t][s] (na x nb, fp32, row stride ldd) = sum over rows p in [s Pq, (s + 1) Pq) of
+// A[t][p][.] (x) B[t][p][.], operands (T, P, ld) of storage type `dtype` (gemm_tn.hip).
+int batched_gemm_tn(const void* A, const void* B, float* D, int T, long long P, int lda, int ldb, int na, int nb,
+                    int ldd, int S, int Pq, int dtype, void* stream);
+
 }  // namespace wc

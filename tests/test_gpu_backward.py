@@ -25,6 +25,8 @@ CASES = [
     ((1, 4, 5, 7, 7), (4, 4, 2, 3, 1), 1, 0, 2),
     ((4, 64, 28, 28), (64, 64, 3, 3), 1, 1, 4),
     ((1, 3, 9, 9), (2, 3, 1, 1), 1, 0, 2),                # 1 x 1 kernel
+    ((6, 24, 40, 40), (40, 24, 3, 3), 1, 1, 2),           # tile sum split into 9 parts, the last one short
+    ((8, 72, 40, 40), (136, 72, 3, 3), 1, 1, 4),          # 128 x 128 product tiles with partial edges, 3 parts
 ]
 TOL = {torch.float32: (1e-3, 1e-3), torch.float16: (2e-2, 2e-2), torch.bfloat16: (2e-2, 2e-1)}
 
@@ -67,9 +69,9 @@ def test_weight_gradient_is_independent_of_the_image_chunking(dev):
     from pytorch_winoconv_amd import _lib
     lib = _lib.load()
     g = torch.Generator().manual_seed(3)
-    xs, ws = (5, 16, 18, 17), (24, 16, 3, 3)
+    xs, ws = (5, 16, 58, 57), (24, 16, 3, 3)   # 225 tiles per image: passes of 4 images split their sum
     x = torch.randn(*xs, generator=g).to(dev).contiguous(memory_format=torch.channels_last)
-    dy = torch.randn(5, 24, 18, 17, generator=g).to(dev).contiguous(memory_format=torch.channels_last)
+    dy = torch.randn(5, 24, 58, 57, generator=g).to(dev).contiguous(memory_format=torch.channels_last)
     ref = engine.conv_backward_weight(x, dy, ws, 1, 1, 4)
     for chunk in (1, 2, 4):
         desc = engine.make_desc(xs, ws, torch.float32, 1, 1, 4, chunk)
