@@ -142,6 +142,38 @@ def run_suite(steps=10):
     return out
 
 
+def run_backward(steps=20):
+    """us per call of the two gradients of the metric layer, next to the forward pass through the
+    same Python entry points."""
+    import torch
+    from pytorch_winoconv_amd import engine
+    dev = torch.device("cuda:0")
+    x, w = synthetic(N)
+    x = x.half().to(dev).contiguous(memory_format=torch.channels_last)
+    w = w.half().to(dev)
+    dy = torch.randn(N, K, H, W, generator=torch.Generator().manual_seed(1)).half().to(dev)
+    dy = dy.contiguous(memory_format=torch.channels_last)
+    calls = {
+        "forward": lambda: engine.conv_forward(x, w, None, 1, PAD, M_TILE),
+        "weight_gradient": lambda: engine.conv_backward_weight(x, dy, tuple(w.shape), 1, PAD, M_TILE),
+        "input_gradient": lambda: engine.conv_backward_input(dy, w, (H, W), 1, PAD, M_TILE),
+    }
+    out = {}
+    for name, fn in calls.items():
+        for _ in range(3):
+            fn()
+        best = float("inf")
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) / steps * 1e6)
+        out[name] = round(best, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,6 +182,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--suite", action="store_true",
                     help="also time every other benchmark configuration (adds a 'suite' list)")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the weight and input gradients of the metric layer")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -264,6 +298,8 @@ def main():
     }
     if args.suite:
         result["suite"] = run_suite()
+    if args.backward:
+        result["backward_us"] = run_backward()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
