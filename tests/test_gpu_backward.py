@@ -62,6 +62,23 @@ def test_gradients_against_fp64_autograd(dev, dtype, case):
     assert dx.dtype == dtype and tuple(dx.shape) == tuple(xs) and _rel(dx, gx) <= tol
 
 
+@pytest.mark.parametrize("k", [4, 5, 7])
+def test_weight_gradient_through_a_whole_kernel_tile(dev, k):
+    """One F(2,k) x F(2,k) tile instead of DWM pieces: the generic gradient kernels.  fp32; the
+    bound grows with k as the forward error of these tiles does (1e-3 is the fp32 bound up to
+    k = 5; F(2,7) loses another decimal digit)."""
+    g = torch.Generator().manual_seed(5)
+    xs, ws = (2, 6, 15, 14), (5, 6, k, k)
+    x = torch.randn(*xs, generator=g)
+    w = torch.randn(*ws, generator=g) * (2.0 / (6 * k * k)) ** 0.5
+    dy = torch.randn(*F.conv2d(x, w, padding=k // 2).shape, generator=g)
+    _, gw = _reference(x, w, dy, 1, k // 2)
+    dw = engine.conv_backward_weight(x.to(dev), dy.to(dev), ws, 1, k // 2, 2, whole_kernel=True)
+    assert _rel(dw, gw) <= (1e-3 if k <= 5 else 1e-2)
+    ref = engine.conv_backward_weight(x.to(dev), dy.to(dev), ws, 1, k // 2, 2)
+    assert _rel(ref, gw) <= 1e-3
+
+
 def test_weight_gradient_is_independent_of_the_image_chunking(dev):
     """The sum over tiles is split into parts and image chunks and added up in fp32: any chunking
     gives the same gradient up to fp32 summation order."""
