@@ -7,11 +7,12 @@
 //   dU[t][k][c] = sum over tiles p of dM[t][p][k] * V[t][p][c]     dM = A dy A^T per tile
 //   dg          = G^T dU G                                         per piece, onto its taps
 //
-// V is the forward input transform (same kernels).  dM comes from a small gather kernel, the
-// contraction over the tiles runs on the batched GEMM after both operands have been transposed to
-// tile-contiguous order (in their storage type; the products of 16-bit operands are exact in fp32
-// and the sum over up to millions of tiles is kept in fp32 from the first product to the last
-// addition), and a last kernel applies G^T . G and accumulates over image chunks.
+// V is the forward input transform (same kernels) and dM comes from a gather kernel of the same
+// shape; both keep the forward layout (rows = tiles, channels contiguous).  The contraction over
+// the tiles runs on MFMA straight from those layouts (gemm_tn.hip: operands in their storage type,
+// whose products are exact in fp32; the sum over up to millions of tiles is kept in fp32 from the
+// first product to the last addition), split into parts that are added here, and a last kernel
+// applies G^T . G and accumulates over image chunks (backward_filter.hip).
 #include "wc_transform.h"
 #include <algorithm>
 
@@ -242,7 +243,7 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
   const long long T = L->plan.t_total;
-  // images per pass: the four large buffers of one pass stay below about 2 GiB
+  // images per pass: the two large buffers of one pass stay below about 2 GiB
   const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es * 1.1;
   int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(2048.0 * 1024 * 1024 / per_image);
   chunk = std::max(1, std::min(chunk, d->N));
