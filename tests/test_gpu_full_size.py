@@ -119,3 +119,33 @@ def test_stage_calls_beyond_2g_elements(dev):
     ref = F.conv2d(x_nchw[N - 1:].double().cpu(), w.double().cpu(), padding=1)
     err = float((yc[N - 1:].double().cpu() - ref).abs().max() / ref.abs().max())
     assert err <= 2e-2, err
+
+
+GRAD_CONFIGS = [c for c in CONFIGS if c[0] in ("metric F(4,3)", "metric F(2,3)", "c2 vgg 64->64 @224 m4", "c4 5x5 s1 tile 4",
+                                               "c4 7x7 s2", "c5 3-D", "c5 3-D tile 2x4x4")]
+
+
+@pytest.mark.parametrize("cfg", GRAD_CONFIGS, ids=[c[0] for c in GRAD_CONFIGS])
+def test_full_size_gradients_are_the_adjoints_of_the_forward_pass(dev, cfg):
+    """The gradients are the adjoints of the two linear maps w -> conv(x, w) and x -> conv(x, w):
+    <dw(x, dy), w'> = <dy, conv(x, w')> and <dx(dy, w), x'> = <dy, conv(x', w)>.  With dy set to the
+    forward output itself the right-hand sides are squared norms, so the identity is checked to a
+    relative bound; the forward pass is the one the tests above check, and no full-size CPU
+    reference is needed.  Sums in fp64 on the device.  Measured: 5e-9 in fp32, <= 3e-5 in fp16 (rounding errors average out over the sum)."""
+    name, xs, ws, stride, pad, m, dtype = cfg
+    x, w = _data(xs, ws, dtype, dev)
+    xd, wd = x.to(dev), w.to(dev)
+    g = torch.Generator().manual_seed(9)
+    w2 = (torch.randn(*ws, generator=g) * float(w.float().std())).to(dtype).to(dev)
+    x2 = torch.randn(*xs, generator=g).to(dtype).to(dev)
+    tol = 1e-6 if dtype == F32 else 1e-3
+
+    dy = engine.conv_forward(xd, w2, None, stride, pad, m)
+    dw = engine.conv_backward_weight(xd, dy, ws, stride, pad, m)
+    lhs, rhs = float((dw.double() * w2.double()).sum()), float((dy.double() ** 2).sum())
+    assert abs(lhs - rhs) <= tol * rhs, (name, "weight gradient", lhs, rhs)
+
+    dy = engine.conv_forward(x2, wd, None, stride, pad, m)
+    dx = engine.conv_backward_input(dy, wd, xs[2:], stride, pad, m)
+    lhs, rhs = float((dx.double() * x2.double()).sum()), float((dy.double() ** 2).sum())
+    assert abs(lhs - rhs) <= tol * rhs, (name, "input gradient", lhs, rhs)
