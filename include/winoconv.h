@@ -74,6 +74,15 @@ typedef struct {
                     * 1: one F(2,k) x F(2,k) tile for the whole k x k kernel, k = 4..7, the arithmetic
                     *    of the reference's PyTorch path (matrix_conv.py:112-135, tables :31-35):
                     *    2-D, stride 1, m = 2 only; loses accuracy quickly with k, fp16 above all */
+  int stacked;     /* 0: every piece of a DWM plan has its own transform-domain elements and products, and
+                    *    the output transform adds the pieces (the reference's structure: outputAggregate,
+                    *    src/split_kernel.cu:184-203);
+                    * 1: all pieces share one tile F(m, r_max) per axis (r_max = most taps of any piece on
+                    *    that axis; shorter pieces count their missing taps as zero) and lie side by side
+                    *    along the reduction axis of U and V (row length n_pieces * Cp), so the batched
+                    *    GEMM adds them: M shrinks to one piece's size.  Same sum, other rounding.
+                    *    2-D only.  The plan then reports t_offset = 0 for every piece and
+                    *    t_total = prod(m + r_max - 1). */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */

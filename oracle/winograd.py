@@ -170,21 +170,64 @@ def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
                 odims=od, grid=grid, two_d=two_d, stride=stride)
 
 
+def stacked_pieces(pieces):
+    """The pieces of a plan re-tiled for summation in the transform domain: every piece gets the
+    tile F(m, r_max) per axis (r_max = most taps of any piece on that axis), element offset 0, and
+    remembers in "real" how many of those taps it has; the others count as zero.  The sum over
+    the pieces of U_s . V_s then has ONE output transform, i.e. the pieces can lie side by side
+    along the reduction axis of the batched product (linearity of A^T . A; nothing the reference
+    does - it adds the pieces after their output transforms, src/split_kernel.cu:184-203)."""
+    rp = [max(pc["axes"][ax][2] for pc in pieces) for ax in range(3)]
+    out = []
+    for pc in pieces:
+        axes = [(pc["axes"][ax][0], pc["axes"][ax][1], rp[ax]) for ax in range(3)]
+        out.append({"axes": axes, "ms": list(pc["ms"]), "alphas": [pc["ms"][ax] + rp[ax] - 1 for ax in range(3)],
+                    "t_offset": 0, "real": [pc["axes"][ax][2] for ax in range(3)]})
+    T = out[0]["alphas"][0] * out[0]["alphas"][1] * out[0]["alphas"][2]
+    return out, T
+
+
+def _own_taps(w, pc):
+    """A filter that holds the taps the piece owns (tap0 + j*step, j < real) at their places and
+    zero everywhere else, large enough for every tap index of the shared tile (j < r_max)."""
+    need = [pc["axes"][ax][0] + (pc["axes"][ax][2] - 1) * pc["axes"][ax][1] + 1 for ax in range(3)]
+    wz = torch.zeros(tuple(w.shape[:2]) + tuple(max(n, k) for n, k in zip(need, w.shape[2:])), dtype=w.dtype)
+    i0, i1, i2 = [torch.arange(pc["real"][ax]) * pc["axes"][ax][1] + pc["axes"][ax][0] for ax in range(3)]
+    sel = (slice(None), slice(None), i0[:, None, None], i1[None, :, None], i2[None, None, :])
+    wz[sel] = w[sel]
+    return wz
+
+
 def dwm_conv(x, w, bias=None, stride=1, padding=0, m=2, discipline="fp32", stages=None,
-             whole_kernel=False):
+             whole_kernel=False, stacked=False):
     """Native-layout Winograd/DWM convolution.  x NC[D]HW, w (K, C, [kD,] kH, kW).
     Returns y NC[D]HW in the storage type of `discipline`.  If `stages` is a dict the
     intermediate buffers U, V, M and the plan are stored in it.  `whole_kernel`: one F(m, k) tile
-    per axis instead of the DWM pieces (the reference's matrix_conv arithmetic)."""
+    per axis instead of the DWM pieces (the reference's matrix_conv arithmetic).  `stacked`: the
+    pieces are summed by the batched product (see stacked_pieces); U and V then are
+    (T, K, n_pieces * C) and (T, P, n_pieces * C)."""
     st = _STORE[discipline]
     plan = conv_plan(tuple(x.shape), tuple(w.shape), stride, padding, m, whole_kernel)
     x3, w3, two_d = _as_3d(x.to(st), w.to(st))
     xl = x3.permute(0, 2, 3, 4, 1).contiguous()                      # dwm.py:84, :132
-    U = filter_transform(w3, plan["pieces"], plan["T_total"], discipline)
-    V = input_transform(xl, plan["pieces"], plan["T_total"], plan["pads"], stride, plan["grid"], discipline)
-    M = batched_product(V, U, discipline)
-    y = output_transform(M, plan["pieces"], x.shape[0], plan["grid"], plan["odims"],
-                         None if bias is None else bias, discipline)
+    if stacked and len(plan["pieces"]) > 1:
+        pcs, T = stacked_pieces(plan["pieces"])
+        Us, Vs = [], []
+        for pc in pcs:
+            wz = _own_taps(w3, pc)
+            Us.append(filter_transform(wz, [pc], T, discipline))
+            Vs.append(input_transform(xl, [pc], T, plan["pads"], stride, plan["grid"], discipline))
+        U, V = torch.cat(Us, dim=2), torch.cat(Vs, dim=2)
+        plan = dict(plan, pieces=pcs, T_total=T)
+        M = batched_product(V, U, discipline)
+        y = output_transform(M, pcs[:1], x.shape[0], plan["grid"], plan["odims"],
+                             None if bias is None else bias, discipline)
+    else:
+        U = filter_transform(w3, plan["pieces"], plan["T_total"], discipline)
+        V = input_transform(xl, plan["pieces"], plan["T_total"], plan["pads"], stride, plan["grid"], discipline)
+        M = batched_product(V, U, discipline)
+        y = output_transform(M, plan["pieces"], x.shape[0], plan["grid"], plan["odims"],
+                             None if bias is None else bias, discipline)
     if stages is not None:
         stages.update(U=U, V=V, M=M, plan=plan, y_cl=y)
     y = y.permute(0, 4, 1, 2, 3)                                     # dwm.py:105, :144

@@ -15,7 +15,7 @@ import ctypes
 
 import torch
 
-from .. import _lib
+from .. import _lib, engine
 from ..engine import (_ptr, _stream, _require_gpu, _w_strides, make_desc, out_dims)
 
 
@@ -107,7 +107,7 @@ def split_and_concat(direction, in_a, out, *args):
 
 
 def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, algo="dwm", U=None,
-                  chunk_images=0):
+                  chunk_images=0, stacked=None):
     """Whole convolution on channel-last tensors, written into `Output`.
 
     Input (B, D, H, W, C) contiguous; Weight any strided view whose dims are (kD, kH, kW, C, K)
@@ -116,7 +116,8 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     tile (4 allowed for 2-D 3x3 stride 1); kernels larger than 3 or stride 2 are decomposed
     (algo "dwm"); algo "whole" keeps a square 2-D kernel of 4..7 taps as one F(2,k) x F(2,k) tile,
     the arithmetic of the reference's matrix_conv path (matrix_conv.py:112-135).  `U` is an
-    optional filter transformed earlier by engine.transform_filter."""
+    optional filter transformed earlier by engine.transform_filter with the same options;
+    `stacked` as in engine.conv_forward (None chooses)."""
     if algo not in ("dwm", "whole"):
         raise ValueError("winograd_conv: algo must be 'dwm' or 'whole', got %r" % (algo,))
     whole = algo == "whole"
@@ -136,10 +137,14 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     if isinstance(padding, int):
         padding = (0 if flat else padding, padding, padding)
     w_kc = Weight.permute(4, 3, 0, 1, 2)                 # (K, C, kD, kH, kW) view, no copy
+    stacked = engine._stack(stacked, Input.dtype, 2 if flat else 3, whole)
     if flat:
-        desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole)
+        desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole,
+                         stacked)
     else:
-        desc = make_desc((B, C, D, H, W), (K, C, kD, kH, kW), Input.dtype, stride, padding, m, chunk_images, whole)
+        desc = make_desc((B, C, D, H, W), (K, C, kD, kH, kW), Input.dtype, stride, padding, m, chunk_images, whole,
+                         stacked)
+    engine.check_u(desc, U)
     out, _ = out_dims(desc)
     _check_out(Output, (B, out[0], out[1], out[2], K), Input, "winograd_conv")
     nbytes = ctypes.c_size_t()

@@ -17,7 +17,7 @@ namespace {
 struct Layout {
   wc_plan plan;
   int out[3], grid[3];
-  int Cp, ldm, chunk;
+  int Cp, ldm, chunk;   // Cp: row length of U and V (pieces side by side in a stacked plan)
   long long tiles_per_image;
   size_t es;
   size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
@@ -30,7 +30,7 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   if (rc) return rc;
   rc = wc_conv_out_dims(d, L->out, L->grid);
   if (rc) return rc;
-  L->Cp = wc_padded_channels(d->C);
+  L->Cp = stacked_row(d, &L->plan);
   L->ldm = wc_padded_channels8(d->K);
   L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];

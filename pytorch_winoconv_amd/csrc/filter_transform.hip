@@ -39,10 +39,12 @@ struct FilterFastArgs {
 
 // One (k, c) of one piece with compile-time kinds: loads the taps once, transforms in registers
 // and writes the alpha^d elements (lanes along c: coalesced rows of U).
+// `taps`: how many of the tile's taps per axis the piece really has; the others count as zero (a
+// stacked plan transforms every piece with the tile of the longest one).
 template <typename T, int K0, int K1, int K2>
 __device__ __forceinline__ void transform_taps(const T* __restrict__ w, const long long (&s)[5], int k, int c,
                                                bool ok, const int (&tap0)[3], int step, T* __restrict__ U,
-                                               long long plane) {
+                                               long long plane, const int (&taps)[3]) {
   constexpr int R0 = Mats<K0>::r, R1 = Mats<K1>::r, R2 = Mats<K2>::r;
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
   float g[R0 * R1 * R2][1];
@@ -51,9 +53,11 @@ __device__ __forceinline__ void transform_taps(const T* __restrict__ w, const lo
     static_for<0, R1>([&](auto j1_) {
       static_for<0, R2>([&](auto j2_) {
         constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
-        const float v = static_cast<float>(wp[(tap0[0] + j0 * step) * s[2] + (tap0[1] + j1 * step) * s[3] +
-                                             (tap0[2] + j2 * step) * s[4]]);
-        g[(j0 * R1 + j1) * R2 + j2][0] = ok ? v : 0.f;
+        const bool real = j0 < taps[0] && j1 < taps[1] && j2 < taps[2];
+        const float v = static_cast<float>(wp[(tap0[0] + (real ? j0 : 0) * step) * s[2] +
+                                             (tap0[1] + (real ? j1 : 0) * step) * s[3] +
+                                             (tap0[2] + (real ? j2 : 0) * step) * s[4]]);
+        g[(j0 * R1 + j1) * R2 + j2][0] = (ok && real) ? v : 0.f;
       });
     });
   });
@@ -76,8 +80,9 @@ __global__ __launch_bounds__(256) void filter_transform_fast_kernel(const Filter
   if (idx >= a.K * a.Cp) return;
   const int c = idx % a.Cp, k = idx / a.Cp;
   T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + idx;
+  const int all[3] = {Mats<K0>::r, Mats<K1>::r, Mats<K2>::r};
   transform_taps<T, K0, K1, K2>(static_cast<const T*>(a.w), a.s, k, c, c < a.C, a.tap0, a.step, U,
-                                (long long)a.K * a.Cp);
+                                (long long)a.K * a.Cp, all);
 }
 
 using FilterFastKernel = void (*)(FilterFastArgs);
@@ -100,6 +105,8 @@ struct FilterArgs {
   int m[3];
   int n_pieces;
   long long total;    // T * K * Cp
+  int stacked;        // pieces side by side along the rows of U, all with the tile of rp taps
+  int rp[3];
   wc_piece piece[WC_MAX_PIECES];
 };
 
@@ -117,20 +124,23 @@ __global__ __launch_bounds__(256) void filter_transform_pieces_kernel(const Filt
   if (idx >= a.K * a.Cp) return;
   const wc_piece& pc = a.piece[blockIdx.y];
   const int c = idx % a.Cp, k = idx / a.Cp;
-  const long long plane = (long long)a.K * a.Cp;
-  T* U = static_cast<T*>(a.U) + (long long)pc.t_offset * plane + idx;
+  const int row = a.stacked ? a.Cp * a.n_pieces : a.Cp;          // row length of U
+  const long long plane = (long long)a.K * row;
+  T* U = static_cast<T*>(a.U) + (long long)pc.t_offset * plane + (long long)k * row +
+         (a.stacked ? (int)blockIdx.y * a.Cp : 0) + c;
   const T* w = static_cast<const T*>(a.w);
   const bool ok = c < a.C;
+  const int r0 = a.stacked ? a.rp[0] : pc.r[0], r1 = a.stacked ? a.rp[1] : pc.r[1], r2 = a.stacked ? a.rp[2] : pc.r[2];
   constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
-#define WC_BODY(K0, K1, K2) transform_taps<T, K0, K1, K2>(w, a.s, k, c, ok, pc.tap0, a.step, U, plane)
+#define WC_BODY(K0, K1, K2) transform_taps<T, K0, K1, K2>(w, a.s, k, c, ok, pc.tap0, a.step, U, plane, pc.r)
 #define WC_ROW(K0, K1) \
-  switch (pc.r[2]) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
+  switch (r2) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
 #define WC_PLANE(K0) \
-  switch (pc.r[1]) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
+  switch (r1) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
   if constexpr (FLAT) {
     WC_PLANE(KIND_11)
   } else {
-    switch (pc.r[0]) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
+    switch (r0) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
   }
 #undef WC_PLANE
 #undef WC_ROW
@@ -211,6 +221,8 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   a.n_pieces = plan->n_pieces;
   for (int i = 0; i < plan->n_pieces; ++i) a.piece[i] = plan->piece[i];
   a.total = (long long)plan->t_total * d->K * a.Cp;
+  a.stacked = d->stacked && plan->n_pieces > 1;
+  stacked_taps(plan, a.rp);
   bool small_taps = true;
   for (int i = 0; i < plan->n_pieces; ++i)
     for (int q = 0; q < 3; ++q) small_taps = small_taps && plan->piece[i].r[q] >= 1 && plan->piece[i].r[q] <= 3;
@@ -229,6 +241,7 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
     WC_CHECK_LAUNCH("filter_transform_pieces_kernel");
     return WC_OK;
   }
+  if (a.stacked) return fail(WC_ERR_UNSUPPORTED, "stacked filter transform needs output tile 2 or 4 in 2-D");
   const long long blocks = ceil_div_ll(a.total, 256);
   WC_CHECK_ARG(blocks < (1ll << 31), "wc_filter_transform: problem too large");
   void (*gen)(FilterArgs) = dispatch_dtype(d->dtype, [](auto t) -> void (*)(FilterArgs) {

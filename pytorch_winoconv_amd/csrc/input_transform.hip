@@ -15,6 +15,10 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   const int Cp = wc_padded_channels(d->C);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
   const bool flat = plan->m[0] == 1;
+  const bool stacked = d->stacked && plan->n_pieces > 1;
+  const int row = stacked_row(d, plan);              // row length of V
+  int rp[3];
+  stacked_taps(plan, rp);
   // Channels per thread.  Measured on MI355X at N=64, C=256, 56x56 fp16: F(4,3) tiles (36 live
   // elements per channel) run best with 2 channels per thread (more wavefronts in flight),
   // F(2,r) tiles with 16-byte accesses; 3-D tiles and whole-kernel tiles (up to 64 elements) use 2.
@@ -27,10 +31,10 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
     if (d->C % v == 0) { vec = v; break; }
   InArgs a;
   a.x = x; a.V = V;
-  a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = Cp;
+  a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = row;
   a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
   a.step = plan->tap_step;
-  a.t_stride = P * Cp;
+  a.t_stride = P * row;
   a.n_cvec = Cp / vec;
   a.total = P * a.n_cvec;
   const long long blocks = ceil_div_ll(a.total, 256);
@@ -53,15 +57,18 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       g.o = a;
       g.n_pieces = plan->n_pieces;
       g.pad1 = d->pad[1]; g.pad2 = d->pad[2];
+      g.col_step = stacked ? Cp : 0;
       for (int s = 0; s < plan->n_pieces; ++s) {
         const wc_piece& pc = plan->piece[s];
-        g.info[s] = pc.t_offset | (pc.tap0[1] << 16) | (pc.tap0[2] << 20) | (pc.r[1] << 24) | (pc.r[2] << 28);
+        const int r1 = stacked ? rp[1] : pc.r[1], r2 = stacked ? rp[2] : pc.r[2];
+        g.info[s] = pc.t_offset | (pc.tap0[1] << 16) | (pc.tap0[2] << 20) | (r1 << 24) | (r2 << 28);
       }
       hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), g);
       WC_CHECK_LAUNCH("input_transform_pieces_kernel");
       return WC_OK;
     }
   }
+  if (stacked) return fail(WC_ERR_UNSUPPORTED, "stacked input transform needs a 2-D plan with output tile 2 or 4");
   for (int s = 0; s < plan->n_pieces; ++s) {
     const wc_piece& pc = plan->piece[s];
     int k[3];

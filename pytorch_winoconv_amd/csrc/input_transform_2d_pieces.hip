@@ -14,7 +14,7 @@ __global__ __launch_bounds__(256) void input_transform_pieces_kernel(InPiecesArg
     const int t_offset = info & 0xffff;
     const int base1 = ((info >> 16) & 15) - g.pad1, base2 = ((info >> 20) & 15) - g.pad2;
     const int r1 = (info >> 24) & 15, r2 = (info >> 28) & 15;
-#define WC_BODY(K1, K2) transform_window<T, KIND_11, K1, K2, VEC>(a, w, 0, base1, base2, t_offset)
+#define WC_BODY(K1, K2) transform_window<T, KIND_11, K1, K2, VEC>(a, w, 0, base1, base2, t_offset, s * g.col_step)
 #define WC_ROW(K1) \
   switch (r2) { case 1: WC_BODY(K1, KA); break; case 2: WC_BODY(K1, KB); break; default: WC_BODY(K1, KC); }
     switch (r1) { case 1: WC_ROW(KA) break; case 2: WC_ROW(KB) break; default: WC_ROW(KC) }

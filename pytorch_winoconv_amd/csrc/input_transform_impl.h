@@ -56,7 +56,7 @@ __device__ __forceinline__ bool in_decode(const InArgs& a, int blk, int vec, InW
 // One window (tile x VEC channels) of one piece: load, transform, store.
 template <typename T, int K0, int K1, int K2, int VEC>
 __device__ __forceinline__ void transform_window(const InArgs& a, const InWhere& w, int base0, int base1,
-                                                 int base2, int t_offset) {
+                                                 int base2, int t_offset, int col0 = 0) {
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
   constexpr int m0 = Mats<K0>::m, m1 = Mats<K1>::m, m2 = Mats<K2>::m;
   const T* x = static_cast<const T*>(a.x);
@@ -97,7 +97,7 @@ __device__ __forceinline__ void transform_window(const InArgs& a, const InWhere&
   if constexpr (A0 > 1) {
     apply_axis<MatSel<K0, false>, 0, A0, A1, A2, VEC>(d, t2);
   }
-  T* V = static_cast<T*>(a.V) + (long long)t_offset * a.t_stride + w.p * a.Cp + w.c;
+  T* V = static_cast<T*>(a.V) + (long long)t_offset * a.t_stride + w.p * a.Cp + col0 + w.c;
   static_for<0, A0 * A1 * A2>([&](auto e_) {
     constexpr int e = decltype(e_)::value;
     if constexpr (A0 > 1) store_pack<T, VEC>(V + e * a.t_stride, t2[e]);
@@ -120,6 +120,7 @@ struct InPiecesArgs {
   InArgs o;                       // base0/1/2 and t_offset unused
   int n_pieces;
   int pad1, pad2;
+  int col_step;                   // columns of V between two pieces (stacked plans), else 0
   int info[WC_MAX_PIECES];        // t_offset | tap0_h << 16 | tap0_w << 20 | r_h << 24 | r_w << 28
 };
 using InPiecesKernel = void (*)(InPiecesArgs);

@@ -345,9 +345,20 @@ static OutMultiKernel pick_multi(bool flat, int m, int vec) {
 
 using namespace wc;
 
-extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan, const void* M,
+extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan_in, const void* M,
                                    const void* bias, int n_images, void* y, void* stream) {
-  WC_CHECK_ARG(d && plan && M && y, "wc_output_transform: null pointer");
+  WC_CHECK_ARG(d && plan_in && M && y, "wc_output_transform: null pointer");
+  // a stacked plan has one set of products (the batched GEMM has added the pieces): the output
+  // transform of a single piece with the shared tile
+  wc_plan one;
+  const wc_plan* plan = plan_in;
+  if (d->stacked && plan_in->n_pieces > 1 && plan_in->n_pieces <= WC_MAX_PIECES) {
+    one = *plan_in;
+    one.n_pieces = 1;
+    stacked_taps(plan_in, one.piece[0].r);
+    one.piece[0].t_offset = 0;
+    plan = &one;
+  }
   WC_CHECK_ARG(n_images > 0, "wc_output_transform: n_images %d", n_images);
   int out[3], grid[3];
   int rc = wc_conv_out_dims(d, out, grid);

@@ -126,6 +126,9 @@ static int check_desc(const wc_conv_desc* d) {
     return fail(WC_ERR_UNSUPPORTED, "output tile 4 in 3-D (2 x 4 x 4) is implemented for 3x3x3 kernels at stride 1");
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
+  WC_CHECK_ARG(d->stacked == 0 || d->stacked == 1, "stacked must be 0 or 1");
+  if (d->stacked && (d->ndim != 2 || d->whole_kernel))
+    return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for 2-D DWM plans");
   if (d->whole_kernel) {
     if (d->ndim != 2 || d->stride != 1 || d->m != 2)
       return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");
@@ -173,6 +176,17 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
       }
   plan->n_pieces = np;
   plan->t_total = t;
+  if (d->stacked) {
+    int rp[3];
+    stacked_taps(plan, rp);
+    t = 1;
+    for (int q = 0; q < 3; ++q) {
+      if (rp[q] > 3) return fail(WC_ERR_UNSUPPORTED, "stacked plans need pieces of at most 3 taps");
+      t *= plan->m[q] + rp[q] - 1;
+    }
+    for (int s = 0; s < np; ++s) plan->piece[s].t_offset = 0;
+    plan->t_total = t;
+  }
   return WC_OK;
 }
 

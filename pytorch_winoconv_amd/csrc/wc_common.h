@@ -60,6 +60,18 @@ inline auto dispatch_dtype(int dtype, F&& f) {
   }
 }
 
+// Taps per axis of the tile that the pieces of a stacked plan share.
+inline void stacked_taps(const wc_plan* plan, int rp[3]) {
+  rp[0] = rp[1] = rp[2] = 1;
+  for (int s = 0; s < plan->n_pieces; ++s)
+    for (int q = 0; q < 3; ++q)
+      if (plan->piece[s].r[q] > rp[q]) rp[q] = plan->piece[s].r[q];
+}
+// Row length of U and V in elements: the pieces of a stacked plan lie side by side.
+inline int stacked_row(const wc_conv_desc* d, const wc_plan* plan) {
+  return wc_padded_channels(d->C) * (d->stacked ? plan->n_pieces : 1);
+}
+
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;
 

@@ -40,9 +40,11 @@ def _triple(v, nd, fill):
     return ((fill,) if nd == 2 else ()) + v
 
 
-def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False):
+def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False, stacked=False):
     """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter.  `whole_kernel`: one
-    F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces."""
+    F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces.  `stacked`: the
+    DWM pieces share one tile and are added by the batched GEMM instead of by the output transform
+    (2-D; same sum, fewer bytes moved for kernels above 3 x 3)."""
     nd = len(x_shape) - 2
     if nd not in (2, 3) or len(w_shape) != nd + 2:
         raise ValueError("expected 4-D or 5-D input and matching filter, got %r and %r"
@@ -65,6 +67,7 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.dtype = _DTYPES[dtype]
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
+    d.stacked = int(bool(stacked))
     return d
 
 
@@ -115,10 +118,14 @@ def _w_strides(w):
 
 
 # ---------------------------------------------------------------- stages (used by the tests)
+def _row(desc, plan):
+    """Row length of U and V: the padded channel count, times the pieces of a stacked plan."""
+    return _lib.load().wc_padded_channels(desc.C) * (plan.n_pieces if desc.stacked else 1)
+
+
 def filter_transform(desc, plan, w):
     _require_gpu(w)
-    Cp = _lib.load().wc_padded_channels(desc.C)
-    U = torch.empty(plan.t_total, desc.K, Cp, dtype=w.dtype, device=w.device)
+    U = torch.empty(plan.t_total, desc.K, _row(desc, plan), dtype=w.dtype, device=w.device)
     check(_lib.load().wc_filter_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(w),
                                           _w_strides(w), _ptr(U), _stream(w)))
     return U
@@ -130,7 +137,7 @@ def input_transform(desc, plan, x_cl):
     _, grid = out_dims(desc)
     n = x_cl.shape[0]
     P = n * grid[0] * grid[1] * grid[2]
-    V = torch.empty(plan.t_total, P, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
+    V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
     check(lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(x_cl), n, _ptr(V), _stream(x_cl)))
     return V
 
@@ -159,27 +166,52 @@ def output_transform(desc, plan, M, bias, n_images):
 
 
 # ---------------------------------------------------------------- whole convolution
-def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False):
-    """Transformed filter U for later calls of conv_forward(..., U=U)."""
+def _stack(stacked, dtype, nd, whole_kernel):
+    """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
+    16-bit 2-D plans (1.15-1.3x for 5x5 and 7x7 kernels; fewer bytes moved), piece by piece for
+    fp32 (whose product is bound by the MFMA rate, and stacking adds zero taps to it)."""
+    if stacked is None:
+        return nd == 2 and dtype != torch.float32 and not whole_kernel
+    return bool(stacked)
+
+
+def check_u(desc, U):
+    """A transformed filter made with other options (tile, stacking) has another size: refuse it
+    rather than read it with the wrong layout."""
+    if U is None:
+        return
+    n = ctypes.c_size_t()
+    check(_lib.load().wc_conv_u_elems(ctypes.byref(desc), ctypes.byref(n)))
+    if not U.is_contiguous() or U.numel() != n.value:
+        raise ValueError("U has %d elements, this convolution needs a contiguous transformed filter of %d "
+                         "(transform_filter must be called with the same options)" % (U.numel(), n.value))
+
+
+def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
+    """Transformed filter U for later calls of conv_forward(..., U=U) with the same options."""
     _require_gpu(w)
-    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel)
+    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel)
+    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked)
     return filter_transform(desc, plan_conv(desc), w)
 
 
-def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False):
+def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False,
+                 stacked=None):
     """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
-    without a copy, any other layout is permuted once."""
+    without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses."""
     _require_gpu(x, w, bias, U)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
     if x.shape[0] == 0:
         # empty batch: the shape arithmetic is checked on one image, nothing is launched
-        out, _ = out_dims(make_desc((1,) + tuple(x.shape[1:]), w.shape, x.dtype, stride, padding, m, 0, whole_kernel))
+        out, _ = out_dims(make_desc((1,) + tuple(x.shape[1:]), w.shape, x.dtype, stride, padding, m, 0, whole_kernel,
+                                    stacked))
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
-    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images, whole_kernel)
+    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images, whole_kernel, stacked)
     out, _ = out_dims(desc)
     x_cl = channel_last(x)
     nbytes = ctypes.c_size_t()
@@ -189,8 +221,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     y = torch.empty([desc.N] + osp + [desc.K], dtype=x.dtype, device=x.device)
     if bias is not None:
         bias = bias.contiguous()
-    if U is not None and not U.is_contiguous():
-        raise ValueError("U must be contiguous")
+    check_u(desc, U)
     check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_cl), _ptr(w), _w_strides(w), _ptr(U),
                               _ptr(bias), _ptr(y), _ptr(ws), nbytes.value, _stream(x)))
     return channel_first_view(y)

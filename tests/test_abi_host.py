@@ -175,6 +175,36 @@ def test_whole_kernel_plans():
             engine.plan_conv(d)
 
 
+def test_stacked_plans():
+    """Pieces that share one tile: element offset 0 for every piece, T of the tile of the longest
+    piece per axis, U / V / workspace sized for the pieces side by side; 2-D DWM plans only."""
+    lib = _lib.load()
+    from oracle import winograd as ow
+    for ws, stride, m in (((4, 8, 5, 5), 1, 4), ((4, 8, 7, 7), 1, 2), ((4, 8, 7, 7), 2, 4), ((4, 8, 3, 3), 2, 2),
+                          ((4, 8, 4, 6), 1, 2), ((4, 8, 3, 3), 1, 4)):
+        xs = (2, 8, 20, 21)
+        plain = engine.plan_conv(engine.make_desc(xs, ws, torch.float16, stride, 1, m))
+        d = engine.make_desc(xs, ws, torch.float16, stride, 1, m, stacked=True)
+        plan = engine.plan_conv(d)
+        pcs, T = ow.stacked_pieces(ow.conv_plan(xs, ws, stride, 1, m)["pieces"])
+        assert plan.n_pieces == plain.n_pieces == len(pcs) and plan.t_total == T
+        for i in range(plan.n_pieces):
+            assert plan.piece[i].t_offset == 0
+            assert list(plan.piece[i].r) == list(plain.piece[i].r) == pcs[i]["real"]
+            assert list(plan.piece[i].tap0) == list(plain.piece[i].tap0)
+        ue, nbytes = ctypes.c_size_t(), ctypes.c_size_t()
+        assert lib.wc_conv_u_elems(ctypes.byref(d), ctypes.byref(ue)) == 0
+        assert ue.value == T * 4 * 32 * plan.n_pieces
+        assert lib.wc_conv_workspace_bytes(ctypes.byref(d), ctypes.byref(nbytes)) == 0
+        out, grid = engine.out_dims(d)
+        P = 2 * grid[1] * grid[2]
+        r256 = lambda v: (v + 255) // 256 * 256                       # each buffer starts on a 256-byte boundary
+        assert nbytes.value == r256(2 * ue.value) + r256(2 * T * P * 32 * plan.n_pieces) + r256(2 * T * P * 8)
+    for xs, ws, kw in (((2, 8, 9, 20, 20), (4, 8, 5, 5, 5), {}), ((2, 8, 20, 20), (4, 8, 5, 5), {"whole_kernel": True})):
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(engine.make_desc(xs, ws, torch.float32, 1, 0, 2, stacked=True, **kw))
+
+
 def test_product_generator_equals_oracle_generator():
     """pytorch_winoconv_amd.wincnn (Lagrange-basis form) against oracle.cook_toom (the
     reference generator's steps), exact rationals, and against the reference's F(2,9) literals."""

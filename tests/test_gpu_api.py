@@ -231,5 +231,5 @@ def test_forward_is_capturable_in_a_hip_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         got = y.clone()
-        want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, 2, 4)     # eager, own buffers
+        want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, 2, 4, stacked=False)     # eager, own buffers
         assert torch.equal(got.permute(0, 3, 1, 2), want), i

@@ -96,3 +96,38 @@ def test_fp16_discipline_is_within_the_stated_tolerance():
         y = ow.dwm_conv(x, w, None, 1, 1, m, "fp16")
         assert y.dtype == torch.float16
         assert float((y.double() - ref).abs().max() / ref.abs().max()) < 2e-2
+
+
+STACKED_CASES = [
+    ((2, 5, 13, 14), (6, 5, 5, 5), 1, 2, 4), ((1, 4, 15, 16), (3, 4, 7, 7), 1, 3, 2),
+    ((2, 3, 15, 14), (4, 3, 7, 7), 2, 3, 4), ((1, 4, 12, 12), (3, 4, 3, 3), 2, 1, 2),
+    ((1, 3, 10, 11), (2, 3, 4, 6), 1, (1, 2), 2), ((1, 3, 20, 21), (2, 3, 10, 9), 1, 4, 2),
+]
+
+
+@pytest.mark.parametrize("case", STACKED_CASES)
+def test_stacked_pieces_give_the_same_convolution(case):
+    """Pieces summed by the batched product instead of after their output transforms: the same
+    convolution in fp64, the integer-exact property of F(2,r) in fp32, and the buffer shapes
+    (T of ONE shared tile, the pieces side by side along the reduction axis)."""
+    xs, ws, s, p, m = case
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(*xs, dtype=torch.float64, generator=g)
+    w = torch.randn(*ws, dtype=torch.float64, generator=g)
+    b = torch.randn(ws[0], dtype=torch.float64, generator=g)
+    st = {}
+    y = ow.dwm_conv(x, w, b, s, p, m, "fp64", st, stacked=True)
+    ref = _conv(x, w, b, s, p)
+    assert y.shape == ref.shape and float((y - ref).abs().max() / ref.abs().max()) < 1e-12
+    plain = ow.conv_plan(xs, ws, s, p, m)
+    n = len(plain["pieces"])
+    rmax = [max(pc["axes"][ax][2] for pc in plain["pieces"]) for ax in (1, 2)]
+    T = (m + rmax[0] - 1) * (m + rmax[1] - 1)
+    P = st["V"].shape[1]
+    assert st["U"].shape == (T, ws[0], n * xs[1]) and st["V"].shape == (T, P, n * xs[1])
+    assert st["M"].shape == (T, P, ws[0]) and T <= plain["T_total"]
+    if m == 2:
+        xi = torch.randint(-3, 4, xs, generator=g).float()
+        wi = (torch.randint(-2, 3, ws, generator=g) * 4).float()
+        yi = ow.dwm_conv(xi, wi, None, s, p, m, "fp32", stacked=True)
+        assert torch.equal(yi.double(), _conv(xi.double(), wi.double(), None, s, p))
