@@ -72,7 +72,9 @@ def cpu_baseline(sample_images=32, repeats=3):
 
 
 SUITE = [
-    # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size)
+    # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size).
+    # c4: the 16-bit default adds the DWM pieces in the batched GEMM ("stacked"); two lines with the
+    # reference's structure (pieces added after their output transforms) stand beside them.
     ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(2,3) x13", "vgg", None, 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(4,3) x13", "vgg", None, 1, 1, 4, "f32"),
@@ -80,13 +82,15 @@ SUITE = [
     ("c3 fp16 N64 C128 28x28 F(4,3)", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)xF(4,3)^2", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, "f16"),
     ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
@@ -105,7 +109,8 @@ def run_suite(steps=10):
     out = []
 
     def one(xs, ws, stride, pad, m, dt):
-        dtype = torch.float16 if dt == "f16" else torch.float32
+        dtype = torch.float32 if dt == "f32" else torch.float16
+        stacked = False if dt.endswith("-pieces") else None        # None: the engine's default
         g = torch.Generator().manual_seed(0)
         fan = 1
         for v in ws[1:]:
@@ -114,7 +119,7 @@ def run_suite(steps=10):
         x = x.contiguous(memory_format=torch.channels_last if len(xs) == 4 else torch.channels_last_3d)
         w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype).to(dev)
         for _ in range(2):
-            y = engine.conv_forward(x, w, None, stride, pad, m)
+            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked)
         # best of three rounds: a single round now and then includes a stall of tens of milliseconds
         # (the caching allocator returning memory between configurations of very different sizes)
         ms = float("inf")
@@ -122,7 +127,7 @@ def run_suite(steps=10):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
-                engine.conv_forward(x, w, None, stride, pad, m)
+                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked)
             torch.cuda.synchronize()
             ms = min(ms, (time.perf_counter() - t0) / steps * 1e3)
         flops = 2.0 * xs[0] * ws[0] * ws[1]

@@ -37,6 +37,11 @@ CONFIGS = [
     ("c4 7x7 s2 tile 4", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, H16),
     ("c4 3x3 s2", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, H16),
     ("c4 7x7 s2", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, H16),
+    # the same plans with the reference's structure (pieces added after their output transforms); the
+    # lines above run the 16-bit default, which adds the pieces in the batched GEMM
+    ("c4 5x5 s1 tile 4 piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, H16),
+    ("c4 7x7 s1 piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, H16),
+    ("c4 7x7 s2 tile 4 piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, H16),
     ("c5 3-D", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, H16),
     ("c5 3-D tile 2x4x4", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, H16),
 ]
@@ -57,7 +62,12 @@ def test_full_size_config(dev, cfg):
     name, xs, ws, stride, pad, m, dtype = cfg
     x, w = _data(xs, ws, dtype, dev)
     xd, wd = x.to(dev), w.to(dev)
-    y = engine.conv_forward(xd, wd, None, stride, pad, m)
+    stacked = False if name.endswith("piece by piece") else None
+
+    def forward(a):
+        return engine.conv_forward(a, wd, None, stride, pad, m, stacked=stacked)
+
+    y = forward(xd)
     conv = F.conv2d if len(xs) == 4 else F.conv3d
     tol = 1e-3 if dtype == F32 else 2e-2
     # one image against fp64 on the CPU (the last one: it sits in the last, possibly partial, chunk)
@@ -68,20 +78,19 @@ def test_full_size_config(dev, cfg):
     assert err <= tol, (name, err)
     if xs[0] > 1:
         perm = torch.randperm(xs[0], generator=torch.Generator().manual_seed(1))
-        yp = engine.conv_forward(xd[perm.to(dev)].contiguous(), wd, None, stride, pad, m)
+        yp = forward(xd[perm.to(dev)].contiguous())
         assert torch.equal(yp, y[perm.to(dev)]), name
     # linearity on a second input (fp32 accumulate, one rounding of each result)
     x2 = torch.randn(xs, generator=torch.Generator().manual_seed(2)).to(dtype).to(dev)
     if dtype == H16:
         xs_sum = (xd.float() + x2.float()).half()          # what the engine really sees
-        lhs = engine.conv_forward(xs_sum, wd, None, stride, pad, m).float()
-        rhs = engine.conv_forward((xs_sum.float() - x2.float()).half(), wd, None, stride, pad, m).float() \
-            + engine.conv_forward(x2, wd, None, stride, pad, m).float()
+        lhs = forward(xs_sum).float()
+        rhs = forward((xs_sum.float() - x2.float()).half()).float() + forward(x2).float()
         scale = float(rhs.abs().max())
         assert float((lhs - rhs).abs().max()) / scale <= 3e-2, name
     else:
-        lhs = engine.conv_forward(xd + x2, wd, None, stride, pad, m)
-        rhs = y + engine.conv_forward(x2, wd, None, stride, pad, m)
+        lhs = forward(xd + x2)
+        rhs = y + forward(x2)
         assert float((lhs - rhs).abs().max() / rhs.abs().max()) <= 1e-4, name
 
 
