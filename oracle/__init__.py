@@ -30,7 +30,10 @@ in tests/test_oracle_*.py):
   split_plan.*         pinned: all 36 keys of the reference LUT (golden JSON).
   tiles.*              pinned: torch unfold / brute-force loops, odd edges.
   winograd.*           pinned: fp64 torch conv2d/conv3d, integer-exact KATs,
-                       the reference kernels' unrolled spot formulas.
+                       the reference kernels' unrolled spot formulas.  The stacked
+                       form of dwm_conv (pieces added by the batched product, which
+                       the reference does not do) is pinned by the same fp64
+                       convolution and integer-exact checks.
   Tables F(2,8..11) of the reference (matrix_conv.py:36-39) are not restated:
   nothing here uses them.
 """
