@@ -100,9 +100,10 @@ VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256
          (512, 512, 14)]
 
 
-def run_suite(steps=10):
+def run_suite(steps=10, only=None):
     """ms per layer (whole forward through the one-call entry point, filter transform included)
-    and direct-convolution-equivalent TFLOP/s for every other benchmark configuration."""
+    and direct-convolution-equivalent TFLOP/s for every other benchmark configuration (`only`:
+    just the configurations whose name contains that text)."""
     import torch
     from pytorch_winoconv_amd import engine
     dev = torch.device("cuda:0")
@@ -136,6 +137,8 @@ def run_suite(steps=10):
         return ms, flops
 
     for name, xs, ws, stride, pad, m, dt in SUITE:
+        if only and only not in name:
+            continue
         if xs == "vgg":
             ms = fl = 0.0
             for c, k, hw in VGG16:
@@ -187,6 +190,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--suite", action="store_true",
                     help="also time every other benchmark configuration (adds a 'suite' list)")
+    ap.add_argument("--suite-only", default=None, metavar="TEXT",
+                    help="with --suite: only the configurations whose name contains TEXT")
     ap.add_argument("--backward", action="store_true",
                     help="also time the weight and input gradients of the metric layer")
     ap.add_argument("--copy-probe", action="store_true",
@@ -302,7 +307,7 @@ def main():
         "one_call_matches_stages": same,
     }
     if args.suite:
-        result["suite"] = run_suite()
+        result["suite"] = run_suite(only=args.suite_only)
     if args.backward:
         result["backward_us"] = run_backward()
     if not args.no_cpu:

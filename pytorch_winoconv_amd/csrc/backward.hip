@@ -247,6 +247,10 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es * 1.1;
   int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(2048.0 * 1024 * 1024 / per_image);
   chunk = std::max(1, std::min(chunk, d->N));
+  if (d->chunk_images <= 0 && chunk < d->N) {   // equal passes rather than full ones and a short last one
+    const int passes = (d->N + chunk - 1) / chunk;
+    chunk = (d->N + passes - 1) / passes;
+  }
   L->chunk = chunk;
   const long long Pc = L->tiles_per_image * chunk;
   if (Pc >= (1ll << 31)) return fail(WC_ERR_UNSUPPORTED, "chunk of %d images has too many tiles", chunk);

@@ -43,6 +43,8 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
     const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es;
     chunk = (int)(2048.0 * 1024 * 1024 / per_image);
     if (chunk < 1) chunk = 1;
+    // equal passes rather than full ones and a short last one
+    if (chunk < d->N) chunk = (d->N + (d->N + chunk - 1) / chunk - 1) / ((d->N + chunk - 1) / chunk);
   }
   if (chunk > d->N) chunk = d->N;
   L->chunk = chunk;
