@@ -243,9 +243,9 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
   const long long T = L->plan.t_total;
-  // images per pass: the two large buffers of one pass stay below about 2 GiB
+  // images per pass: the two large buffers of one pass stay below about 8 GiB
   const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es * 1.1;
-  int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(2048.0 * 1024 * 1024 / per_image);
+  int chunk = d->chunk_images > 0 ? d->chunk_images : (int)(8192.0 * 1024 * 1024 / per_image);
   chunk = std::max(1, std::min(chunk, d->N));
   if (d->chunk_images <= 0 && chunk < d->N) {   // equal passes rather than full ones and a short last one
     const int passes = (d->N + chunk - 1) / chunk;

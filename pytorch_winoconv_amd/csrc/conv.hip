@@ -39,9 +39,9 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   if (chunk <= 0) {
     // Measured on MI355X (N=64, C=K=256, 56x56, fp16): one pass over the whole batch is fastest,
     // smaller chunks lose more to partially filled launches than they gain from cache residency.
-    // The chunk only bounds the scratch footprint: V + M of one chunk stay below 2 GiB.
+    // The chunk only bounds the scratch footprint: V + M of one chunk stay below 8 GiB.
     const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es;
-    chunk = (int)(2048.0 * 1024 * 1024 / per_image);
+    chunk = (int)(8192.0 * 1024 * 1024 / per_image);
     if (chunk < 1) chunk = 1;
     // equal passes rather than full ones and a short last one
     if (chunk < d->N) chunk = (d->N + (d->N + chunk - 1) / chunk - 1) / ((d->N + chunk - 1) / chunk);

@@ -123,10 +123,29 @@ def test_stage_calls_beyond_2g_elements(dev):
         assert torch.equal(y[b:b + 1], y1), ("output transform", b)
     del V, M
     x_nchw = x.permute(0, 3, 1, 2)                                         # channels_last view, no copy
-    yc = engine.conv_forward(x_nchw, w, None, 1, 1, 2)                     # chunked: V + M bounded at 2 GiB
+    yc = engine.conv_forward(x_nchw, w, None, 1, 1, 2)                     # chunked: V + M bounded at 8 GiB
     assert torch.equal(yc.permute(0, 2, 3, 1), y[:, 0])                    # stage output keeps a depth axis of 1
     ref = F.conv2d(x_nchw[N - 1:].double().cpu(), w.double().cpu(), padding=1)
     err = float((yc[N - 1:].double().cpu() - ref).abs().max() / ref.abs().max())
+    assert err <= 2e-2, err
+
+
+def test_stacked_plan_beyond_2g_elements_in_one_pass(dev):
+    """7x7 kernel, pieces stacked: V of one pass holds 16 x 125440 x 1152 = 2.3e9 elements.  Images are
+    independent, so every image of the batch must equal its own single-image convolution bit for
+    bit, and one of them is checked against fp64."""
+    N, C, K, H = 40, 128, 128, 112
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn(K, C, 7, 7, generator=g) * (2.0 / (C * 49)) ** 0.5).half().to(dev)
+    x = torch.randn(N, C, H, H, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    desc = engine.make_desc(x.shape, w.shape, H16, 1, 3, 2, stacked=True)
+    plan = engine.plan_conv(desc)
+    assert plan.t_total * (N * 56 * 56) * (plan.n_pieces * C) > 2 ** 31
+    y = engine.conv_forward(x, w, None, 1, 3, 2, stacked=True)
+    for b in (0, 17, N - 1):
+        assert torch.equal(y[b:b + 1], engine.conv_forward(x[b:b + 1], w, None, 1, 3, 2, stacked=True)), b
+    ref = F.conv2d(x[N - 1:].double().cpu(), w.double().cpu(), padding=3)
+    err = float((y[N - 1:].double().cpu() - ref).abs().max() / ref.abs().max())
     assert err <= 2e-2, err
 
 
