@@ -225,7 +225,9 @@ size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 struct BwdLayout {
   wc_plan plan;
   int out[3], grid[3];
-  int Cp, ldm, ldc, chunk, S, Pq;
+  int Cp, ldm, ldc, chunk, S, Pq;   // Cp: row length of V; ldc: row length of dU (both span the pieces of a stacked plan)
+  int ncol;                         // columns of dU that are computed
+  wc_plan dm_plan;                  // the plan dM follows: the plan itself, or its one shared tile when stacked
   long long tiles_per_image;
   size_t es;
   size_t v_bytes, dm_bytes, du_bytes, acc_bytes;
@@ -237,9 +239,18 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   rc = wc_conv_out_dims(d, L->out, L->grid);
   if (rc) return rc;
   if (L->plan.t_total > 0xffff) return fail(WC_ERR_UNSUPPORTED, "plan with %d transform elements is too large", L->plan.t_total);
-  L->Cp = wc_padded_channels(d->C);
+  const bool stacked = d->stacked && L->plan.n_pieces > 1;
+  L->Cp = stacked_row(d, &L->plan);
   L->ldm = wc_padded_channels8(d->K);
-  L->ldc = wc_padded_channels8(d->C);
+  L->ncol = stacked ? L->Cp : d->C;
+  L->ldc = wc_padded_channels8(L->ncol);
+  L->dm_plan = L->plan;
+  if (stacked) {
+    // one set of dM for all pieces: the adjoint of the single output transform of the stacked forward pass
+    L->dm_plan.n_pieces = 1;
+    stacked_taps(&L->plan, L->dm_plan.piece[0].r);
+    L->dm_plan.piece[0].t_offset = 0;
+  }
   L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
   const long long T = L->plan.t_total;
@@ -255,8 +266,8 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   const long long Pc = L->tiles_per_image * chunk;
   if (Pc >= (1ll << 31)) return fail(WC_ERR_UNSUPPORTED, "chunk of %d images has too many tiles", chunk);
   // split of the tile axis: about four workgroups of the product per CU, every part >= 256 tiles
-  const int bt = (d->K > 64 && d->C > 64) ? 128 : 64;
-  const long long tiles = T * ((d->K + bt - 1) / bt) * ((d->C + bt - 1) / bt);
+  const int bt = (d->K > 64 && L->ncol > 64) ? 128 : 64;
+  const long long tiles = T * ((d->K + bt - 1) / bt) * ((L->ncol + bt - 1) / bt);
   long long S = (1024 + tiles - 1) / tiles;
   S = std::max(1ll, std::min(S, std::min(64ll, Pc / 256)));
   L->S = (int)S;
@@ -316,15 +327,16 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
       a.oD = L.out[0]; a.oH = L.out[1]; a.oW = L.out[2]; a.K = d->K; a.ldm = L.ldm;
       a.nD = L.grid[0]; a.nH = L.grid[1]; a.nW = L.grid[2];
       a.P = P;
-      for (int i = 0; i < 3; ++i) a.m[i] = L.plan.m[i];
-      a.n_pieces = L.plan.n_pieces;
-      for (int i = 0; i < L.plan.n_pieces; ++i) a.piece[i] = L.plan.piece[i];
+      const wc_plan& gp = L.dm_plan;
+      for (int i = 0; i < 3; ++i) a.m[i] = gp.m[i];
+      a.n_pieces = gp.n_pieces;
+      for (int i = 0; i < gp.n_pieces; ++i) a.piece[i] = gp.piece[i];
       a.total = (long long)T * P * L.ldm;
       const long long blocks = ceil_div_ll(a.total, 256);
       WC_CHECK_ARG(blocks < (1ll << 31), "wc_conv_backward_weight: problem too large");
       bool small_taps = true;
-      for (int i = 0; i < L.plan.n_pieces; ++i)
-        for (int q = 0; q < 3; ++q) small_taps = small_taps && L.plan.piece[i].r[q] <= 3;
+      for (int i = 0; i < gp.n_pieces; ++i)
+        for (int q = 0; q < 3; ++q) small_taps = small_taps && gp.piece[i].r[q] <= 3;
       const int m0 = L.plan.m[0], mo = L.plan.m[1];
       void (*fn)(GradOutArgs) = nullptr;
       long long threads = a.total;
@@ -355,7 +367,7 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
     const int Pq = (int)(((P + L.S - 1) / L.S + 31) / 32 * 32);
     // dU[(t, s)] (K x C, fp32) = sum over the tiles of part s of dM[t][p][.] (x) V[t][p][.]: operands in
     // the storage type (their values already are), products summed in fp32
-    rc = batched_gemm_tn(dM, V, dU, T, P, L.ldm, L.Cp, d->K, d->C, L.ldc, L.S, Pq, d->dtype, stream);
+    rc = batched_gemm_tn(dM, V, dU, T, P, L.ldm, L.Cp, d->K, L.ncol, L.ldc, L.S, Pq, d->dtype, stream);
     if (rc) return rc;
     if (L.S > 1) {
       const long long n = (long long)d->K * L.ldc, total4 = (long long)T * n / 4;

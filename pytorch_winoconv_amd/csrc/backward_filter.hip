@@ -21,6 +21,9 @@ struct GradFilterArgs {
   int step;
   int m[3];
   int n_pieces;
+  int stacked;               // pieces side by side along the rows of dU, all with the tile of rp taps
+  int Cp;                    // columns of dU per piece of a stacked plan
+  int rp[3];
   int first;                 // 1: overwrite acc, 0: add to it
   long long total;           // taps * K * C
   wc_piece piece[WC_MAX_PIECES];
@@ -85,7 +88,8 @@ struct MatGT {
 // piece's taps.
 template <int K0, int K1, int K2>
 __device__ __forceinline__ void grad_taps(const float* __restrict__ src, long long t_stride, float* __restrict__ acc,
-                                          long long plane, const int (&tap0)[3], int step, int kH, int kW, bool first) {
+                                          long long plane, const int (&tap0)[3], int step, int kH, int kW, bool first,
+                                          const int (&taps)[3]) {
   constexpr int R0 = Mats<K0>::r, R1 = Mats<K1>::r, R2 = Mats<K2>::r;
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
   float u[A0 * A1 * A2][1];
@@ -103,10 +107,13 @@ __device__ __forceinline__ void grad_taps(const float* __restrict__ src, long lo
     static_for<0, R1>([&](auto j1_) {
       static_for<0, R2>([&](auto j2_) {
         constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
-        const int tap = ((tap0[0] + j0 * step) * kH + tap0[1] + j1 * step) * kW + tap0[2] + j2 * step;
-        float* dst = acc + tap * plane;
-        const float v = g0[(j0 * R1 + j1) * R2 + j2][0];
-        *dst = first ? v : *dst + v;
+        // (a stacked plan transforms with the tile of the longest piece: taps this piece lacks are dropped)
+        if (j0 < taps[0] && j1 < taps[1] && j2 < taps[2]) {
+          const int tap = ((tap0[0] + j0 * step) * kH + tap0[1] + j1 * step) * kW + tap0[2] + j2 * step;
+          float* dst = acc + tap * plane;
+          const float v = g0[(j0 * R1 + j1) * R2 + j2][0];
+          *dst = first ? v : *dst + v;
+        }
       });
     });
   });
@@ -122,20 +129,21 @@ __global__ __launch_bounds__(256) void grad_filter_pieces_kernel(const GradFilte
   const wc_piece& pc = a.piece[blockIdx.y];
   const int c = idx % a.C, k = idx / a.C;
   const long long t_stride = (long long)a.S * a.K * a.ldc;
-  const float* src = a.dU + pc.t_offset * t_stride + (long long)k * a.ldc + c;
+  const float* src = a.dU + pc.t_offset * t_stride + (long long)k * a.ldc + (a.stacked ? (int)blockIdx.y * a.Cp : 0) + c;
+  const int r0 = a.stacked ? a.rp[0] : pc.r[0], r1 = a.stacked ? a.rp[1] : pc.r[1], r2 = a.stacked ? a.rp[2] : pc.r[2];
   float* acc = a.acc + idx;
   const long long plane = (long long)a.K * a.C;
   const bool first = a.first != 0;
   constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
-#define WC_BODY(K0, K1, K2) grad_taps<K0, K1, K2>(src, t_stride, acc, plane, pc.tap0, a.step, a.kernel[1], a.kernel[2], first)
+#define WC_BODY(K0, K1, K2) grad_taps<K0, K1, K2>(src, t_stride, acc, plane, pc.tap0, a.step, a.kernel[1], a.kernel[2], first, pc.r)
 #define WC_ROW(K0, K1) \
-  switch (pc.r[2]) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
+  switch (r2) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
 #define WC_PLANE(K0) \
-  switch (pc.r[1]) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
+  switch (r1) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
   if constexpr (M0 == 1) {
     WC_PLANE(KIND_11)
   } else {
-    switch (pc.r[0]) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
+    switch (r0) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
   }
 #undef WC_PLANE
 #undef WC_ROW
@@ -155,6 +163,9 @@ int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const floa
   g.n_pieces = plan->n_pieces;
   for (int i = 0; i < plan->n_pieces; ++i) g.piece[i] = plan->piece[i];
   g.first = first;
+  g.stacked = d->stacked && plan->n_pieces > 1;
+  g.Cp = wc_padded_channels(d->C);
+  stacked_taps(plan, g.rp);
   g.total = (long long)d->kernel[0] * d->kernel[1] * d->kernel[2] * d->K * d->C;
   const int m0 = plan->m[0], mo = plan->m[1];
   bool small_taps = true;
@@ -167,6 +178,7 @@ int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const floa
     const dim3 grid((unsigned)ceil_div_ll((long long)d->K * d->C, 256), (unsigned)plan->n_pieces);
     hipLaunchKernelGGL(fn, grid, dim3(256), 0, s, g);
   } else {
+    if (g.stacked) return fail(WC_ERR_UNSUPPORTED, "stacked weight gradient needs a 2-D plan with output tile 2 or 4");
     hipLaunchKernelGGL(grad_filter_transform_kernel, dim3((unsigned)ceil_div_ll(g.total, 256)), dim3(256), 0, s, g);
   }
   WC_CHECK_LAUNCH("grad_filter_transform_kernel");

@@ -228,15 +228,16 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
 
 
 # ---------------------------------------------------------------- gradients
-def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
+def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
     """Gradient of sum(y * dy) with respect to the filter of conv_forward(x, w, ...): a tensor of
     shape `w_shape` (K, C, [kD,] kH, kW) in x's dtype.  The reference has no backward pass; this one
-    works in the transform domain (see include/winoconv.h)."""
+    works in the transform domain (see include/winoconv.h).  `stacked` as in conv_forward."""
     _require_gpu(x, dy)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel)
     if dy.dtype != x.dtype:
         raise TypeError("x and dy must share one dtype")
     lib = _lib.load()
-    desc = make_desc(x.shape, w_shape, x.dtype, stride, padding, m, 0, whole_kernel)
+    desc = make_desc(x.shape, w_shape, x.dtype, stride, padding, m, 0, whole_kernel, stacked)
     out, _ = out_dims(desc)
     osp = out[1:] if desc.ndim == 2 else out
     if tuple(dy.shape) != (x.shape[0], w_shape[0]) + tuple(osp):

@@ -130,3 +130,33 @@ def test_random_shapes_stacked(dev, case):
     y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), stride, pad, m, stacked=True)
     assert tuple(y.shape) == tuple(ref.shape), case
     assert _rel(y, ref) <= _tol(dtype, m), case
+
+
+GRAD_CASES = CASES[:7] + [((6, 24, 40, 40), (40, 24, 5, 5), 1, 2, 2),      # tile sum split into parts
+                          ((8, 72, 40, 40), (136, 72, 5, 5), 1, 2, 4)]     # 128 x 128 product tiles, partial edges
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", GRAD_CASES)
+def test_stacked_weight_gradient(dev, dtype, case):
+    """The weight gradient of a stacked plan (one dM for all pieces, V with the pieces side by side,
+    taps a piece lacks dropped at the end) against fp64 autograd, and against the piece-by-piece
+    gradient: taps of pieces that already have the longest tile come out bit-identical."""
+    xs, ws, stride, pad, m = case
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / (ws[1] * ws[2] * ws[3])) ** 0.5).to(dtype)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    y = F.conv2d(xr, wr, stride=stride, padding=pad)
+    dy = torch.randn(*y.shape, generator=g).to(dtype)
+    gw, = torch.autograd.grad(y, (wr,), dy.double())
+    dw = engine.conv_backward_weight(x.to(dev), dy.to(dev), ws, stride, pad, m, stacked=True)
+    assert dw.dtype == dtype and tuple(dw.shape) == tuple(ws) and _rel(dw, gw) <= _tol(dtype, m)
+    dw_pieces = engine.conv_backward_weight(x.to(dev), dy.to(dev), ws, stride, pad, m, stacked=False)
+    plan = ow.conv_plan(xs, ws, stride, pad, m)
+    rmax = [max(pc["axes"][ax][2] for pc in plan["pieces"]) for ax in (1, 2)]
+    for pc in plan["pieces"]:
+        (h0, hs, hr), (w0, wsx, wr_) = pc["axes"][1], pc["axes"][2]
+        if [hr, wr_] == rmax:
+            sel = (slice(None), slice(None), slice(h0, h0 + hr * hs, hs), slice(w0, w0 + wr_ * wsx, wsx))
+            assert torch.equal(dw[sel], dw_pieces[sel])
