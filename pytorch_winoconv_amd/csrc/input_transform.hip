@@ -50,10 +50,23 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
     small_taps = pc.r[1] >= 1 && pc.r[1] <= 3 && pc.r[2] >= 1 && pc.r[2] <= 3 && pc.tap0[1] < 16 && pc.tap0[2] < 16;
   }
   if (small_taps && plan->m[1] == plan->m[2]) {
-    InPiecesKernel fn = pick_in_2d_pieces(d->dtype, plan->m[1], vec);
+    // Stacked plans of small problems give every piece its own threads (one thread per tile and
+    // channel group, looping over the pieces, then leaves most of the chip idle: 2.2x faster at
+    // N=8, C=24, 56x56, 7x7); large ones keep the loop, which reads each window from cache once per
+    // piece and measured 7-30 % faster there.
+    const bool per_piece_threads = stacked && a.total < 512 * 1024;
+    InPiecesKernel fn = per_piece_threads ? pick_in_2d_stacked(d->dtype, plan->m[1], vec)
+                                          : pick_in_2d_pieces(d->dtype, plan->m[1], vec);
     if (fn) {
       InPiecesArgs g;
       a.base0 = a.base1 = a.base2 = 0; a.t_offset = 0;
+      dim3 launch = launch_grid;
+      if (per_piece_threads) {
+        a.total = P * a.n_cvec * plan->n_pieces;
+        a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);
+        WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
+        launch = dim3((unsigned)(a.per_xcd * kXcds));
+      }
       g.o = a;
       g.n_pieces = plan->n_pieces;
       g.pad1 = d->pad[1]; g.pad2 = d->pad[2];
@@ -63,7 +76,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
         const int r1 = stacked ? rp[1] : pc.r[1], r2 = stacked ? rp[2] : pc.r[2];
         g.info[s] = pc.t_offset | (pc.tap0[1] << 16) | (pc.tap0[2] << 20) | (r1 << 24) | (r2 << 28);
       }
-      hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), g);
+      hipLaunchKernelGGL(fn, launch, dim3(256), 0, as_stream(stream), g);
       WC_CHECK_LAUNCH("input_transform_pieces_kernel");
       return WC_OK;
     }

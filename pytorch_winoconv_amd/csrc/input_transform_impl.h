@@ -125,6 +125,7 @@ struct InPiecesArgs {
 };
 using InPiecesKernel = void (*)(InPiecesArgs);
 InPiecesKernel pick_in_2d_pieces(int dtype, int m, int vec);     // nullptr if the combination is not built
+InPiecesKernel pick_in_2d_stacked(int dtype, int m, int vec);    // stacked plans: one thread per (tile, piece, channels)
 
 using InKernel = void (*)(InArgs);
 
