@@ -166,13 +166,26 @@ def output_transform(desc, plan, M, bias, n_images):
 
 
 # ---------------------------------------------------------------- whole convolution
-def _stack(stacked, dtype, nd, whole_kernel):
+def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1):
     """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
-    16-bit 2-D plans (1.15-1.3x for 5x5 and 7x7 kernels; fewer bytes moved), piece by piece for
-    fp32 (whose product is bound by the MFMA rate, and stacking adds zero taps to it)."""
-    if stacked is None:
-        return nd == 2 and dtype != torch.float32 and not whole_kernel
-    return bool(stacked)
+    16-bit 2-D plans (1.15-1.3x for 5x5 and 7x7 kernels; fewer bytes moved); for fp32, whose
+    product is bound by the MFMA rate and to which stacking adds zero taps, only plans of up to
+    four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x)."""
+    if stacked is not None:
+        return bool(stacked)
+    if nd != 2 or whole_kernel:
+        return False
+    if dtype != torch.float32:
+        return True
+    if w_shape is None:
+        return False
+    if isinstance(stride, (tuple, list)):
+        stride = stride[0]
+    n = 1
+    for k in w_shape[2:]:
+        taps = [(int(k) + 1 - q) // 2 for q in range(2)] if stride == 2 else [int(k)]
+        n *= sum((t + 2) // 3 if t != 4 else 2 for t in taps if t > 0)
+    return 1 < n <= 4
 
 
 def check_u(desc, U):
@@ -190,7 +203,7 @@ def check_u(desc, U):
 def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
     """Transformed filter U for later calls of conv_forward(..., U=U) with the same options."""
     _require_gpu(w)
-    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel)
+    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel, w.shape, stride)
     desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked)
     return filter_transform(desc, plan_conv(desc), w)
 
@@ -201,7 +214,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
     without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses."""
     _require_gpu(x, w, bias, U)
-    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
@@ -233,7 +246,7 @@ def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=
     shape `w_shape` (K, C, [kD,] kH, kW) in x's dtype.  The reference has no backward pass; this one
     works in the transform domain (see include/winoconv.h).  `stacked` as in conv_forward."""
     _require_gpu(x, dy)
-    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w_shape, stride)
     if dy.dtype != x.dtype:
         raise TypeError("x and dy must share one dtype")
     lib = _lib.load()

@@ -97,9 +97,11 @@ def test_cached_filter_chunks_and_size_check(dev):
     U_pieces = engine.transform_filter(w, xs, 1, 2, 4, stacked=False)
     with pytest.raises(ValueError):
         engine.conv_forward(x, w, None, 1, 2, 4, U=U_pieces, stacked=True)
-    # fp32 keeps the piece-by-piece form unless asked
+    # fp32: stacked by default up to four pieces (5x5), piece by piece beyond (7x7: nine)
     xf, wf = x.float(), w.float()
-    assert torch.equal(engine.conv_forward(xf, wf, None, 1, 2, 4), engine.conv_forward(xf, wf, None, 1, 2, 4, stacked=False))
+    assert torch.equal(engine.conv_forward(xf, wf, None, 1, 2, 4), engine.conv_forward(xf, wf, None, 1, 2, 4, stacked=True))
+    w7 = torch.randn(16, 24, 7, 7, generator=g).to(dev) * 0.05
+    assert torch.equal(engine.conv_forward(xf, w7, None, 1, 3, 4), engine.conv_forward(xf, w7, None, 1, 3, 4, stacked=False))
 
 
 def _random_cases(seed, n):
