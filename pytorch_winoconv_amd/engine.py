@@ -293,10 +293,12 @@ def conv_backward_input(dy, w, x_spatial, stride=1, padding=0, m=2):
     elif stride != 1:
         raise NotImplementedError("stride must be 1 or 2")
     w_rot = w.flip(tuple(range(2, 2 + nd))).transpose(0, 1)
-    # output tile: the caller's, except where the 3-D tile 4 does not exist and for stride 2, where
+    # output tile: the caller's, except where the 3-D tile 4 does not exist, for stride 2, where
     # three quarters of the zero-filled dy are zeros and the F(4,r) rounding error is not averaged
-    # down (fp16: 2.6e-2 of the gradient's range against 2e-3 with tile 2)
-    mm = m if (stride == 1 and (m == 2 or nd == 2 or ks == (3, 3, 3))) else 2
+    # down (fp16: 2.6e-2 of the gradient's range against 2e-3 with tile 2), and for fewer than 8
+    # output channels, where the sum is too short to average it down either (fp16, K = 1: up to
+    # 3e-2 with tile 4, 1e-3 with tile 2)
+    mm = m if (stride == 1 and w.shape[0] >= 8 and (m == 2 or nd == 2 or ks == (3, 3, 3))) else 2
     dx = conv_forward(dy, w_rot, None, 1, tuple(k - 1 - p for k, p in zip(ks, pads)), mm)
     if tuple(dx.shape[2:]) != want:
         raise ValueError("dy of shape %r does not belong to an input of extent %r" % (tuple(dy.shape), want))

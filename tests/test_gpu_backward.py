@@ -79,6 +79,21 @@ def test_weight_gradient_through_a_whole_kernel_tile(dev, k):
     assert _rel(ref, gw) <= 1e-3
 
 
+def test_input_gradient_of_few_output_channels_uses_tile_2(dev):
+    """With fewer than 8 output channels the sum behind each input-gradient element is too short to
+    average the F(4,r) rounding error down (fp16, K = 1: up to 3e-2 of the range), so the engine
+    computes it with tile 2 whatever tile the forward pass uses: 2e-3 here."""
+    for seed in range(4):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(1, 32, 19, 9, generator=g).half()
+        w = (torch.randn(1, 32, 5, 3, generator=g) * (2.0 / (32 * 15)) ** 0.5).half()
+        dy = torch.randn(1, 1, 23, 9, generator=g).half()
+        gx, _ = _reference(x, w, dy, 1, (4, 1))
+        dx = engine.conv_backward_input(dy.to(dev), w.to(dev), (19, 9), 1, (4, 1), 4)
+        assert _rel(dx, gx) <= 2e-3
+        assert torch.equal(dx, engine.conv_backward_input(dy.to(dev), w.to(dev), (19, 9), 1, (4, 1), 2))
+
+
 def test_weight_gradient_is_independent_of_the_image_chunking(dev):
     """The sum over tiles is split into parts and image chunks and added up in fp32: any chunking
     gives the same gradient up to fp32 summation order."""
