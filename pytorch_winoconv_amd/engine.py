@@ -224,20 +224,42 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
                                     stacked))
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
-    desc = make_desc(x.shape, w.shape, x.dtype, stride, padding, m, chunk_images, whole_kernel, stacked)
-    out, _ = out_dims(desc)
+    desc, y_shape, nbytes, u_elems = _forward_setup(tuple(x.shape), tuple(w.shape), x.dtype, stride, padding, m,
+                                                    chunk_images, whole_kernel, stacked)
     x_cl = channel_last(x)
-    nbytes = ctypes.c_size_t()
-    check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
-    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
-    osp = out[1:] if desc.ndim == 2 else out
-    y = torch.empty([desc.N] + osp + [desc.K], dtype=x.dtype, device=x.device)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
     if bias is not None:
         bias = bias.contiguous()
-    check_u(desc, U)
+    if U is not None and (not U.is_contiguous() or U.numel() != u_elems):
+        check_u(desc, U)                                  # raises with the sizes in the message
     check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_cl), _ptr(w), _w_strides(w), _ptr(U),
-                              _ptr(bias), _ptr(y), _ptr(ws), nbytes.value, _stream(x)))
+                              _ptr(bias), _ptr(y), _ptr(ws), nbytes, _stream(x)))
     return channel_first_view(y)
+
+
+_SETUPS = {}
+
+
+def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked):
+    """Descriptor, output shape (channel-last), workspace bytes and size of U for one problem.  Kept
+    per problem: for small layers (a few tens of microseconds on the GPU) rebuilding them on every
+    call costs as much host time as the launches themselves."""
+    key = (x_shape, w_shape, dtype, stride if isinstance(stride, int) else tuple(stride),
+           padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked)
+    hit = _SETUPS.get(key)
+    if hit is None:
+        lib = _lib.load()
+        desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked)
+        out, _ = out_dims(desc)
+        nbytes, ue = ctypes.c_size_t(), ctypes.c_size_t()
+        check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+        check(lib.wc_conv_u_elems(ctypes.byref(desc), ctypes.byref(ue)))
+        osp = out[1:] if desc.ndim == 2 else out
+        if len(_SETUPS) >= 4096:
+            _SETUPS.clear()
+        hit = _SETUPS[key] = (desc, [desc.N] + osp + [desc.K], nbytes.value, ue.value)
+    return hit
 
 
 # ---------------------------------------------------------------- gradients
