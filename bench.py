@@ -194,6 +194,42 @@ def run_backward(steps=20):
     return out
 
 
+def run_split_concat(steps=20):
+    """Tile split / concat (bit-exact copies) at the metric layer's shape: us per call and HBM GB/s
+    of the algorithmic bytes (input once + tiles once; tiles once + output once)."""
+    import torch
+    from pytorch_winoconv_amd import backend
+    dev = torch.device("cuda:0")
+    out = {}
+    for name, dtype in (("f32", torch.float32), ("f16", torch.float16)):
+        for alpha, m in ((4, 2), (6, 4)):
+            x = torch.randn(N, H + 2, W + 2, C, device=dev).to(dtype)            # padded by one, channel-last
+            nH, nW = (H + m - 1) // m, (W + m - 1) // m
+            tiles = torch.empty(N * nH * nW, C, alpha, alpha, dtype=dtype, device=dev)
+            yt = torch.randn(N * nH * nW, K, m, m, device=dev).to(dtype)
+            y = torch.empty(N, H, W, K, dtype=dtype, device=dev)
+            calls = {
+                "split": (lambda: backend.WinoSplit(x, tiles, 1, alpha, alpha, m, 1, nH, nW, True),
+                          (x.numel() + tiles.numel()) * x.element_size()),
+                "concat": (lambda: backend.WinoConcat(yt, y, m, True), (yt.numel() + y.numel()) * y.element_size()),
+            }
+            for what, (fn, nbytes) in calls.items():
+                for _ in range(3):
+                    fn()
+                best = float("inf")
+                for _ in range(3):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(steps):
+                        fn()
+                    torch.cuda.synchronize()
+                    best = min(best, (time.perf_counter() - t0) / steps)
+                out["%s %s %dx%d tiles, step %d" % (what, name, alpha if what == "split" else m,
+                                                    alpha if what == "split" else m, m)] = {
+                    "us": round(best * 1e6, 1), "MB": round(nbytes / 1e6, 1), "GB_s": round(nbytes / best / 1e9, 0)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -208,6 +244,8 @@ def main():
                     help="with --suite: only the configurations whose name contains TEXT")
     ap.add_argument("--backward", action="store_true",
                     help="also time the weight and input gradients of the metric layer")
+    ap.add_argument("--split-concat", action="store_true",
+                    help="also time the tile split / concat kernels at the metric layer's shape")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -344,6 +382,8 @@ def main():
         result["suite"] = run_suite(only=args.suite_only)
     if args.backward:
         result["backward_us"] = run_backward()
+    if args.split_concat:
+        result["split_concat"] = run_split_concat()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

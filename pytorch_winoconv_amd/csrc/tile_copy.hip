@@ -5,10 +5,14 @@
 //   split : tiles[((b*nD+d)*nH+h)*nW+w][c][k][i][j] = x[b][m*d+k][m*h+i][m*w+j][c], 0 outside
 //   concat: y[b][m*d+k][m*h+i][m*w+j][c] = tiles[((b*nD+d)*nH+h)*nW+w][c][k][i][j] if inside
 //
-// Both are pure HBM-bound copies.  One workgroup moves one tile x 64 channels through LDS so
-// that the channel-last side is accessed with lanes along C and the tile side as one
-// contiguous run of 64*E elements (the reference writes E scalars per lane with stride E).
+// Both are pure HBM-bound copies.  A workgroup moves a row of up to 8 neighbouring tiles x 64
+// channels through LDS: the channel-last side is accessed in 16-byte vectors along C (the
+// overlapping window columns of neighbouring tiles are read once), the tile side as contiguous
+// runs of 64*E elements per tile in 16-byte vectors (the reference writes E scalars per lane with
+// stride E).  Channel counts that are not a multiple of the vector length take the scalar
+// kernels below, one tile per workgroup.
 #include "wc_common.h"
+#include <algorithm>
 
 namespace wc {
 
@@ -91,6 +95,131 @@ __global__ __launch_bounds__(256) void wino_concat_kernel(TileArgs a) {
   }
 }
 
+
+typedef uint32_t Vec16 __attribute__((ext_vector_type(4)));   // one 16-byte access
+
+struct RowArgs {
+  TileArgs t;
+  int TW;                 // tiles along W per workgroup
+  int w_groups;           // ceil(nW / TW)
+  int cols;               // window columns of the workgroup's tiles together: m (TW - 1) + bW
+};
+
+// pixel (k, i, col) of the staged region -> offset of its first channel in LDS
+template <typename U>
+__device__ __forceinline__ int pix_off(int pixel) {
+  constexpr int V = 16 / sizeof(U);
+  return pixel * (kCC + V);                      // rows stay 16-byte aligned; the pad spreads the banks
+}
+
+// e -> pixel of tile 0 of the row: the table all threads use instead of dividing by runtime extents
+__device__ __forceinline__ void fill_table(int* table, int E, int bH, int bW, int cols) {
+  for (int e = threadIdx.x; e < E; e += 256) {
+    const int j = e % bW; const int r = e / bW;
+    table[e] = ((r / bH) * bH + r % bH) * cols + j;
+  }
+}
+
+template <typename U>
+__global__ __launch_bounds__(256) void wino_split_row_kernel(RowArgs g) {
+  constexpr int V = 16 / sizeof(U);              // elements per vector
+  constexpr int VPC = kCC / V;                   // vectors per pixel
+  const TileArgs& a = g.t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int E = a.bD * a.bH * a.bW;
+  int* table = reinterpret_cast<int*>(lds_raw);
+  U* lds = reinterpret_cast<U*>(lds_raw + (E * 4 + 15) / 16 * 16);
+  int blk = blockIdx.x;
+  const int cc = blk % a.c_chunks; blk /= a.c_chunks;
+  const int wg = blk % g.w_groups; int q = blk / g.w_groups;
+  const int th = q % a.nH; q /= a.nH;
+  const int td = q % a.nD;
+  const int b = q / a.nD;
+  const int tw0 = wg * g.TW;
+  const int ntw = min(g.TW, a.nW - tw0);
+  const int c0 = cc * kCC;
+  const int cn = min(kCC, a.C - c0);
+  fill_table(table, E, a.bH, a.bW, g.cols);
+  // gather the window of the tile row: 16-byte vectors along the channels
+  const U* x = static_cast<const U*>(a.src);
+  const int cols = a.m * (ntw - 1) + a.bW;
+  const int pixels = a.bD * a.bH * cols;
+  for (int idx = threadIdx.x; idx < pixels * VPC; idx += 256) {
+    const int cv = idx % VPC, px = idx / VPC;
+    const int col = px % cols; const int r = px / cols;
+    const int i = r % a.bH, k = r / a.bH;
+    const int z = a.m * td + k, yy = a.m * th + i, xx = a.m * tw0 + col;
+    Vec16 v = {0u, 0u, 0u, 0u};
+    if (cv * V < cn && z < a.D && yy < a.H && xx < a.W)
+      v = *reinterpret_cast<const Vec16*>(x + ((((long long)b * a.D + z) * a.H + yy) * a.W + xx) * a.C + c0 + cv * V);
+    *reinterpret_cast<Vec16*>(lds + pix_off<U>((k * a.bH + i) * g.cols + col) + cv * V) = v;
+  }
+  __syncthreads();
+  // tiles[p][c0 + c][e], c < cn: one contiguous run of cn * E elements per tile
+  const long long p0 = (((long long)b * a.nD + td) * a.nH + th) * a.nW + tw0;
+  const int run = cn * E;                        // a multiple of V
+  for (int o = threadIdx.x * V; o < ntw * run; o += 256 * V) {
+    const int t = o / run; const int w = o % run;
+    int c = w / E, e = w % E;
+    alignas(16) U out[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      out[v] = lds[pix_off<U>(table[e] + a.m * t) + c];
+      if (++e == E) { e = 0; ++c; }
+    }
+    *reinterpret_cast<Vec16*>(static_cast<U*>(a.dst) + ((p0 + t) * a.C + c0) * E + w) = *reinterpret_cast<const Vec16*>(out);
+  }
+}
+
+template <typename U>
+__global__ __launch_bounds__(256) void wino_concat_row_kernel(RowArgs g) {
+  constexpr int V = 16 / sizeof(U);
+  constexpr int VPC = kCC / V;
+  const TileArgs& a = g.t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int E = a.bD * a.bH * a.bW;
+  int* table = reinterpret_cast<int*>(lds_raw);
+  U* lds = reinterpret_cast<U*>(lds_raw + (E * 4 + 15) / 16 * 16);
+  int blk = blockIdx.x;
+  const int cc = blk % a.c_chunks; blk /= a.c_chunks;
+  const int wg = blk % g.w_groups; int q = blk / g.w_groups;
+  const int th = q % a.nH; q /= a.nH;
+  const int td = q % a.nD;
+  const int b = q / a.nD;
+  const int tw0 = wg * g.TW;
+  const int ntw = min(g.TW, a.nW - tw0);
+  const int c0 = cc * kCC;
+  const int cn = min(kCC, a.C - c0);
+  fill_table(table, E, a.bH, a.bW, g.cols);
+  __syncthreads();
+  const long long p0 = (((long long)b * a.nD + td) * a.nH + th) * a.nW + tw0;
+  const int run = cn * E;
+  for (int o = threadIdx.x * V; o < ntw * run; o += 256 * V) {
+    const int t = o / run; const int w = o % run;
+    int c = w / E, e = w % E;
+    alignas(16) U in[V];
+    *reinterpret_cast<Vec16*>(in) = *reinterpret_cast<const Vec16*>(static_cast<const U*>(a.src) + ((p0 + t) * a.C + c0) * E + w);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      lds[pix_off<U>(table[e] + a.m * t) + c] = in[v];
+      if (++e == E) { e = 0; ++c; }
+    }
+  }
+  __syncthreads();
+  U* y = static_cast<U*>(a.dst);
+  const int cols = a.m * ntw;                    // tiles do not overlap: bW == m
+  const int pixels = a.bD * a.bH * cols;
+  for (int idx = threadIdx.x; idx < pixels * VPC; idx += 256) {
+    const int cv = idx % VPC, px = idx / VPC;
+    const int col = px % cols; const int r = px / cols;
+    const int i = r % a.bH, k = r / a.bH;
+    const int z = a.m * td + k, yy = a.m * th + i, xx = a.m * tw0 + col;
+    if (cv * V < cn && z < a.D && yy < a.H && xx < a.W)
+      *reinterpret_cast<Vec16*>(y + ((((long long)b * a.D + z) * a.H + yy) * a.W + xx) * a.C + c0 + cv * V) =
+          *reinterpret_cast<const Vec16*>(lds + pix_off<U>((k * a.bH + i) * g.cols + col) + cv * V);
+  }
+}
+
 static int launch_tiles(bool split, const void* src, void* dst, int B, int D, int H, int W, int C,
                         int bD, int bH, int bW, int m, int nD, int nH, int nW, int elem_size,
                         void* stream) {
@@ -106,6 +235,37 @@ static int launch_tiles(bool split, const void* src, void* dst, int B, int D, in
   WC_CHECK_ARG(blocks < (1ll << 31), "%s: too many tiles", name);
   TileArgs a{src, dst, B, D, H, W, C, bD, bH, bW, m, nD, nH, nW, ceil_div(C, kCC)};
   hipStream_t s = as_stream(stream);
+  const int V = 16 / elem_size;
+  const bool aligned = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (reinterpret_cast<uintptr_t>(dst) % 16 == 0);
+  if (C % V == 0 && aligned && (split || bW == m)) {
+    // a row of tiles per workgroup: at most 8, fewer for large tiles (LDS)
+    const int E = bD * bH * bW;
+    RowArgs g;
+    g.t = a;
+    int tw = std::min(8, nW);
+    auto lds_bytes = [&](int t) {
+      return (size_t)(E * 4 + 15) / 16 * 16 + (size_t)bD * bH * (m * (t - 1) + bW) * (kCC + V) * elem_size;
+    };
+    while (tw > 2 && lds_bytes(tw) > 36 * 1024) --tw;       // four workgroups per CU when the tile allows
+    while (tw > 1 && lds_bytes(tw) > 56 * 1024) --tw;
+    if (lds_bytes(tw) <= 56 * 1024) {
+      g.TW = tw;
+      g.w_groups = ceil_div(nW, tw);
+      g.cols = m * (tw - 1) + bW;
+      const long long rows = (long long)B * nD * nH * g.w_groups * a.c_chunks;
+      WC_CHECK_ARG(rows < (1ll << 31), "%s: too many tiles", name);
+      const size_t lb = lds_bytes(tw);
+      if (split) {
+        if (elem_size == 4) wino_split_row_kernel<uint32_t><<<(unsigned)rows, 256, lb, s>>>(g);
+        else wino_split_row_kernel<uint16_t><<<(unsigned)rows, 256, lb, s>>>(g);
+      } else {
+        if (elem_size == 4) wino_concat_row_kernel<uint32_t><<<(unsigned)rows, 256, lb, s>>>(g);
+        else wino_concat_row_kernel<uint16_t><<<(unsigned)rows, 256, lb, s>>>(g);
+      }
+      WC_CHECK_LAUNCH(name);
+      return WC_OK;
+    }
+  }
   const size_t lds = (size_t)bD * bH * bW * (kCC + 1) * elem_size;   // <= 56 KB
   if (split) {
     if (elem_size == 4) wino_split_kernel<uint32_t><<<(unsigned)blocks, 256, lds, s>>>(a);

@@ -25,6 +25,13 @@ def _rel(a, b):
     ((1, 3, 12, 7), (3, 3, 5, 5), 2),
     ((2, 6, 6, 7, 9), (3, 6, 3, 3, 3), 2),
     ((1, 130, 5, 6, 6), (3, 130, 2, 3, 2), 2),
+    # channel counts that take the vectorised kernels (a row of up to 8 tiles per workgroup):
+    ((2, 64, 37, 41), (3, 64, 3, 3), 2),             # 20 tiles per row: full and partial groups
+    ((1, 72, 30, 19), (3, 72, 3, 3), 4),             # a partial channel chunk (72 = 64 + 8), 6 x 6 tiles
+    ((2, 8, 21, 23), (3, 8, 5, 5), 2),               # 6 x 6 tiles with step 2
+    ((1, 136, 9, 11, 13), (3, 136, 3, 3, 3), 2),     # 4 x 4 x 4 tiles
+    ((1, 16, 7, 20, 22), (3, 16, 3, 3, 3), 4),       # 6 x 6 x 6 tiles: few tiles fit the staging buffer
+    ((3, 256, 14, 14), (3, 256, 1, 1), 2),           # 2 x 2 tiles without overlap
 ])
 def test_wino_split_bit_exact(dev, dtype, shape, wshape, m):
     torch.manual_seed(1)
@@ -38,6 +45,8 @@ def test_wino_split_bit_exact(dev, dtype, shape, wshape, m):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("osize,K,B,m", [
     ((7, 9), 5, 2, 2), ((8, 8), 70, 1, 2), ((13, 10), 64, 2, 4), ((5, 7, 6), 6, 2, 2), ((4, 4, 5), 130, 1, 2),
+    ((37, 41), 64, 2, 2), ((30, 19), 72, 1, 4), ((21, 23), 8, 2, 2), ((9, 11, 13), 136, 1, 2), ((7, 20, 22), 16, 1, 4),
+    ((56, 56), 256, 2, 4),
 ])
 def test_wino_concat_bit_exact(dev, dtype, osize, K, B, m):
     torch.manual_seed(2)
