@@ -95,8 +95,11 @@ class _WinoConvNd(nn.Module):
         return 4 if self.nd == 2 else 2
 
     def _tile_for(self, dtype):
-        # F(4,r) tiles lose about 1e-1 of the output range in bfloat16 (8 mantissa bits): tile 2 there
-        if self.output_block is None and dtype == torch.bfloat16:
+        # F(4,r) tiles lose about 1e-1 of the output range in bfloat16 (8 mantissa bits): tile 2 there.
+        # In float16 their rounding error averages down over the input channels (1e-2 of the range
+        # at worst for 8 and more); with fewer it does not (3e-2 seen with one channel): tile 2 too.
+        if self.output_block is None and (dtype == torch.bfloat16 or
+                                          (dtype == torch.float16 and self.in_channels < 8)):
             return 2
         return self._tile()
 

@@ -205,6 +205,17 @@ def test_stacked_plans():
             engine.plan_conv(engine.make_desc(xs, ws, torch.float32, 1, 0, 2, stacked=True, **kw))
 
 
+def test_modules_pick_tile_2_where_tile_4_loses_accuracy():
+    import pytorch_winoconv_amd as pkg
+    wide, thin = pkg.WinoConv2d(64, 64, 3, padding=1), pkg.WinoConv2d(3, 64, 3, padding=1)
+    assert wide._tile_for(torch.float16) == 4 and wide._tile_for(torch.float32) == 4
+    assert wide._tile_for(torch.bfloat16) == 2          # 8 mantissa bits
+    assert thin._tile_for(torch.float16) == 2            # too few channels to average the rounding error down
+    assert thin._tile_for(torch.float32) == 4
+    assert pkg.WinoConv2d(3, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4   # an explicit choice stands
+    assert pkg.WinoConv3d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
+
+
 def test_product_generator_equals_oracle_generator():
     """pytorch_winoconv_amd.wincnn (Lagrange-basis form) against oracle.cook_toom (the
     reference generator's steps), exact rationals, and against the reference's F(2,9) literals."""

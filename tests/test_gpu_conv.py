@@ -3,7 +3,9 @@ against the CPU oracle run in the same arithmetic discipline.
 
 Tolerances (max |y - y64| / max |y64|, fp64 conv fed the same already-rounded inputs):
   fp32 F(2x2,3x3) and every fp32 F(2,r) plan: 1e-3 (measured ~1e-6),
-  fp16 (any plan, F(4x4,3x3) included):       2e-2.
+  fp16 (any plan, F(4x4,3x3) included):       2e-2 (F(4,r) tiles: with 8 or more input channels; the
+      rounding error of a tile-4 transform averages down over the channels, and with one or two
+      channels unlucky data reach 3e-2 - the modules use tile 2 there).
 """
 import pytest
 import torch
