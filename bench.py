@@ -271,9 +271,15 @@ def main():
     x_cl = engine.channel_last(x)
     T, P = plan.t_total, N * grid[1] * grid[2]
     Cp, ldm = lib.wc_padded_channels(C), lib.wc_padded_channels8(K)
-    U = torch.empty(T, K, Cp, dtype=dtype, device=dev)
-    V = torch.empty(T, P, Cp, dtype=dtype, device=dev)
-    Mb = torch.empty(T, P, ldm, dtype=dtype, device=dev)
+    # U, V and M laid out as wc_conv_forward lays them out in its workspace (each 256-byte aligned)
+    nb = ctypes.c_size_t()
+    _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nb)))
+    wsbuf = torch.empty(nb.value, dtype=torch.uint8, device=dev)
+    r256 = lambda v: (v + 255) // 256 * 256
+    ub, vb = r256(T * K * Cp * 2), r256(T * P * Cp * 2)
+    U = wsbuf[:T * K * Cp * 2].view(dtype).view(T, K, Cp)
+    V = wsbuf[ub:ub + T * P * Cp * 2].view(dtype).view(T, P, Cp)
+    Mb = wsbuf[ub + vb:ub + vb + T * P * ldm * 2].view(dtype).view(T, P, ldm)
     y = torch.empty(N, out[1], out[2], K, dtype=dtype, device=dev)
     st = engine._stream(x)
     d_, p_ = ctypes.byref(desc), ctypes.byref(plan)
