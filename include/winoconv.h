@@ -81,7 +81,7 @@ typedef struct {
                     *    that axis; shorter pieces count their missing taps as zero) and lie side by side
                     *    along the reduction axis of U and V (row length n_pieces * Cp), so the batched
                     *    GEMM adds them: M shrinks to one piece's size.  Same sum, other rounding.
-                    *    2-D only.  The plan then reports t_offset = 0 for every piece and
+                    *    Output tile 2, or 4 in 2-D.  The plan then reports t_offset = 0 for every piece and
                     *    t_total = prod(m + r_max - 1). */
 } wc_conv_desc;
 

@@ -137,7 +137,7 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     if isinstance(padding, int):
         padding = (0 if flat else padding, padding, padding)
     w_kc = Weight.permute(4, 3, 0, 1, 2)                 # (K, C, kD, kH, kW) view, no copy
-    stacked = engine._stack(stacked, Input.dtype, 2 if flat else 3, whole, (K, C, kH, kW), stride)
+    stacked = engine._stack(stacked, Input.dtype, 2 if flat else 3, whole, (K, C, kH, kW), stride, m)
     if flat:
         desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole,
                          stacked)

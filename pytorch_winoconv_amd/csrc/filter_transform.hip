@@ -241,7 +241,7 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
     WC_CHECK_LAUNCH("filter_transform_pieces_kernel");
     return WC_OK;
   }
-  if (a.stacked) return fail(WC_ERR_UNSUPPORTED, "stacked filter transform needs output tile 2 or 4 in 2-D");
+  if (a.stacked) return fail(WC_ERR_UNSUPPORTED, "stacked filter transform needs output tile 2 or 4 in 2-D, 2 in 3-D");
   const long long blocks = ceil_div_ll(a.total, 256);
   WC_CHECK_ARG(blocks < (1ll << 31), "wc_filter_transform: problem too large");
   void (*gen)(FilterArgs) = dispatch_dtype(d->dtype, [](auto t) -> void (*)(FilterArgs) {

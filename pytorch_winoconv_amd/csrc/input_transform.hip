@@ -81,12 +81,15 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       return WC_OK;
     }
   }
-  if (stacked) return fail(WC_ERR_UNSUPPORTED, "stacked input transform needs a 2-D plan with output tile 2 or 4");
+  if (stacked && (flat || plan->m[1] != 2))
+    return fail(WC_ERR_UNSUPPORTED, "stacked input transform needs output tile 2 or 4 in 2-D, 2 in 3-D");
+  // one launch per piece (3-D plans); the pieces of a stacked plan all use the shared tile and
+  // write their own columns of V
   for (int s = 0; s < plan->n_pieces; ++s) {
     const wc_piece& pc = plan->piece[s];
     int k[3];
     for (int q = 0; q < 3; ++q) {
-      k[q] = kind_of(plan->m[q], pc.r[q]);
+      k[q] = kind_of(plan->m[q], stacked ? rp[q] : pc.r[q]);
       if (k[q] < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[q], pc.r[q]);
     }
     InKernel fn = nullptr;
@@ -131,6 +134,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
     if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for kinds (%d,%d,%d) not built", k[0], k[1], k[2]);
     a.base0 = pc.tap0[0] - d->pad[0]; a.base1 = pc.tap0[1] - d->pad[1]; a.base2 = pc.tap0[2] - d->pad[2];
     a.t_offset = pc.t_offset;
+    a.V = static_cast<char*>(V) + (stacked ? (long long)s * Cp * (d->dtype == WC_F32 ? 4 : 2) : 0);
     hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("input_transform_kernel");
   }

@@ -127,8 +127,8 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
   WC_CHECK_ARG(d->stacked == 0 || d->stacked == 1, "stacked must be 0 or 1");
-  if (d->stacked && (d->ndim != 2 || d->whole_kernel))
-    return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for 2-D DWM plans");
+  if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
+    return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
   if (d->whole_kernel) {
     if (d->ndim != 2 || d->stride != 1 || d->m != 2)
       return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");

@@ -166,18 +166,18 @@ def output_transform(desc, plan, M, bias, n_images):
 
 
 # ---------------------------------------------------------------- whole convolution
-def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1):
+def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
-    16-bit 2-D plans (1.15-1.3x for 5x5 and 7x7 kernels; fewer bytes moved); for fp32, whose
-    product is bound by the MFMA rate and to which stacking adds zero taps, only plans of up to
-    four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x)."""
+    16-bit plans (2-D: 1.15-1.3x for 5x5 and 7x7 kernels; 3-D: 1.05-1.4x; fewer bytes moved); for
+    fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
+    plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x)."""
     if stacked is not None:
         return bool(stacked)
-    if nd != 2 or whole_kernel:
+    if whole_kernel or (nd == 3 and m != 2):
         return False
     if dtype != torch.float32:
         return True
-    if w_shape is None:
+    if w_shape is None or nd != 2:
         return False
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
@@ -203,7 +203,7 @@ def check_u(desc, U):
 def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
     """Transformed filter U for later calls of conv_forward(..., U=U) with the same options."""
     _require_gpu(w)
-    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel, w.shape, stride)
+    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel, w.shape, stride, m)
     desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked)
     return filter_transform(desc, plan_conv(desc), w)
 
@@ -214,7 +214,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
     without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses."""
     _require_gpu(x, w, bias, U)
-    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
@@ -268,7 +268,7 @@ def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=
     shape `w_shape` (K, C, [kD,] kH, kW) in x's dtype.  The reference has no backward pass; this one
     works in the transform domain (see include/winoconv.h).  `stacked` as in conv_forward."""
     _require_gpu(x, dy)
-    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w_shape, stride)
+    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w_shape, stride, m)
     if dy.dtype != x.dtype:
         raise TypeError("x and dy must share one dtype")
     lib = _lib.load()

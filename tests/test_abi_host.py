@@ -200,9 +200,12 @@ def test_stacked_plans():
         P = 2 * grid[1] * grid[2]
         r256 = lambda v: (v + 255) // 256 * 256                       # each buffer starts on a 256-byte boundary
         assert nbytes.value == r256(2 * ue.value) + r256(2 * T * P * 32 * plan.n_pieces) + r256(2 * T * P * 8)
-    for xs, ws, kw in (((2, 8, 9, 20, 20), (4, 8, 5, 5, 5), {}), ((2, 8, 20, 20), (4, 8, 5, 5), {"whole_kernel": True})):
-        with pytest.raises(NotImplementedError):
-            engine.plan_conv(engine.make_desc(xs, ws, torch.float32, 1, 0, 2, stacked=True, **kw))
+    d3 = engine.make_desc((2, 8, 9, 20, 20), (4, 8, 5, 5, 5), torch.float32, 1, 0, 2, stacked=True)
+    p3 = engine.plan_conv(d3)
+    assert p3.n_pieces == 8 and p3.t_total == 64 and all(p3.piece[i].t_offset == 0 for i in range(8))
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(engine.make_desc((2, 8, 20, 20), (4, 8, 5, 5), torch.float32, 1, 0, 2, stacked=True,
+                                          whole_kernel=True))
 
 
 def test_modules_pick_tile_2_where_tile_4_loses_accuracy():

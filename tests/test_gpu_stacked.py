@@ -162,3 +162,48 @@ def test_stacked_weight_gradient(dev, dtype, case):
         if [hr, wr_] == rmax:
             sel = (slice(None), slice(None), slice(h0, h0 + hr * hs, hs), slice(w0, w0 + wr_ * wsx, wsx))
             assert torch.equal(dw[sel], dw_pieces[sel])
+
+
+CASES_3D = [
+    ((1, 6, 7, 9, 8), (5, 6, 5, 5, 5), 1, 2),             # 8 pieces, all padded to F(2,3)^3
+    ((2, 3, 6, 10, 9), (4, 3, 4, 5, 3), 1, (1, 2, 1)),    # 2+2, 3+2 and 3 taps: shared tile F(2,2) x F(2,3) x F(2,3)
+    ((1, 8, 9, 9, 9), (6, 8, 3, 3, 3), 2, 1),             # stride 2: parity pieces of 2 and 1 taps
+    ((1, 40, 6, 12, 12), (33, 40, 7, 3, 5), 1, (3, 1, 2)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("case", CASES_3D)
+def test_stacked_3d(dev, dtype, case):
+    """3-D DWM plans (output tile 2) stacked: forward against the oracle and fp64 convolution, the
+    weight gradient against fp64 autograd."""
+    xs, ws, stride, pad = case
+    g = torch.Generator().manual_seed(31)
+    fan = ws[1] * ws[2] * ws[3] * ws[4]
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    ref = F.conv3d(xr, wr, b.double(), stride=stride, padding=pad)
+    st = {}
+    yo = ow.dwm_conv(x, w, b, stride, pad, 2, DISC[dtype], st, stacked=True)
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), stride, pad, 2, stacked=True)
+    assert tuple(y.shape) == tuple(ref.shape) and _rel(y, ref.detach()) <= _tol(dtype, 2)
+    assert _rel(y, yo) <= 4 * STAGE_TOL[dtype]
+    desc = engine.make_desc(xs, ws, dtype, stride, pad, 2, stacked=True)
+    plan = engine.plan_conv(desc)
+    assert plan.t_total == st["plan"]["T_total"] and plan.n_pieces == len(st["plan"]["pieces"])
+    n, C = plan.n_pieces, xs[1]
+    Cp = _lib.load().wc_padded_channels(C)
+    V = engine.input_transform(desc, plan, engine.channel_last(x.to(dev)))
+    U = engine.filter_transform(desc, plan, w.to(dev))
+    for i in range(n):
+        assert _rel(V[:, :, i * Cp:i * Cp + C], st["V"][:, :, i * C:(i + 1) * C]) <= STAGE_TOL[dtype]
+        assert _rel(U[:, :, i * Cp:i * Cp + C], st["U"][:, :, i * C:(i + 1) * C]) <= STAGE_TOL[dtype]
+    dy = torch.randn(*ref.shape, generator=g).to(dtype)
+    gw, = torch.autograd.grad(ref, (wr,), dy.double())
+    dw = engine.conv_backward_weight(x.to(dev), dy.to(dev), ws, stride, pad, 2, stacked=True)
+    assert _rel(dw, gw) <= _tol(dtype, 2)
+    # tile 4 does not exist for 3-D DWM plans, stacked or not
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(engine.make_desc(xs, ws, dtype, stride, pad, 4, stacked=True))
