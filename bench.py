@@ -73,12 +73,14 @@ def cpu_baseline(sample_images=32, repeats=3):
 
 SUITE = [
     # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size).
+    # c3, 64 channels: the default is the fused F(2,3) kernel; the three-kernel F(4,3) line stands beside it.
     # c4: the 16-bit default adds the DWM pieces in the batched GEMM ("stacked"); two lines with the
     # reference's structure (pieces added after their output transforms) stand beside them.
     ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(2,3) x13", "vgg", None, 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(4,3) x13", "vgg", None, 1, 1, 4, "f32"),
-    ("c3 fp16 N64 C64 56x56 F(4,3)", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 4, "f16"),
+    ("c3 fp16 N64 C64 56x56 F(2,3) one kernel", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f16"),
+    ("c3 fp16 N64 C64 56x56 F(4,3) three kernels", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 4, "f16-unfused"),
     ("c3 fp16 N64 C128 28x28 F(4,3)", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, "f16"),
@@ -113,6 +115,7 @@ def run_suite(steps=10, only=None):
     def one(xs, ws, stride, pad, m, dt):
         dtype = torch.float32 if dt == "f32" else torch.float16
         stacked = False if dt.endswith("-pieces") else None        # None: the engine's default
+        unfused = dt.endswith("-unfused")                          # thin layers: keep the three-kernel path
         g = torch.Generator().manual_seed(0)
         fan = 1
         for v in ws[1:]:
@@ -121,7 +124,7 @@ def run_suite(steps=10, only=None):
         x = x.contiguous(memory_format=torch.channels_last if len(xs) == 4 else torch.channels_last_3d)
         w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype).to(dev)
         for _ in range(2):
-            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked)
+            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused)
         # best of three rounds: a single round now and then includes a stall of tens of milliseconds
         # (the caching allocator returning memory between configurations of very different sizes)
         ms = float("inf")
@@ -129,17 +132,17 @@ def run_suite(steps=10, only=None):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
-                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked)
+                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused)
             torch.cuda.synchronize()
             ms = min(ms, (time.perf_counter() - t0) / steps * 1e3)
         U = engine.transform_filter(w, xs, stride, pad, m, stacked=stacked)
-        engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked)
+        engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused)
         msc = float("inf")
         for _ in range(3):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
-                engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked)
+                engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused)
             torch.cuda.synchronize()
             msc = min(msc, (time.perf_counter() - t0) / steps * 1e3)
         flops = 2.0 * xs[0] * ws[0] * ws[1]

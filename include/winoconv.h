@@ -83,6 +83,11 @@ typedef struct {
                     *    GEMM adds them: M shrinks to one piece's size.  Same sum, other rounding.
                     *    Output tile 2, or 4 in 2-D.  The plan then reports t_offset = 0 for every piece and
                     *    t_total = prod(m + r_max - 1). */
+  int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2, at most 64 input
+                    *    channels (an even number up to 32, a multiple of 4 above) and at most 128 output
+                    *    channels run as one kernel: input transform, products and output transform of
+                    *    F(2x2, 3x3) without V and M in memory, the product kept in fp32 (x below 1 GiB);
+                    * 1: always filter transform -> input transform -> batched GEMM -> output transform. */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */
@@ -158,7 +163,8 @@ int wc_output_transform(const wc_conv_desc* desc, const wc_plan* plan,
  * The workspace holds U, V and M (the reference's tmp_weight_buffer, tmp_input_buffer,
  * tmp_product_buffer: dwm.py:122-125); images are processed in chunks that bound the size
  * of V and M.  `U_cached` (may be NULL) is a filter already transformed
- * by wc_filter_transform; `w` may then be NULL. */
+ * by wc_filter_transform; `w` may then be NULL.  Thin 16-bit 3x3 layers take one fused kernel
+ * instead (see wc_conv_desc.unfused); the workspace requirement is the same either way. */
 int wc_conv_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
 int wc_conv_u_elems(const wc_conv_desc* desc, size_t* elems);
 int wc_conv_forward(const wc_conv_desc* desc, const void* x,

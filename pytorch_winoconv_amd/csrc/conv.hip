@@ -99,6 +99,15 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   void* V = ws + L.u_bytes;
   void* M = ws + L.u_bytes + L.v_bytes;
   const void* U = U_cached;
+  if (!d->unfused && thin_conv_fits(d, &L.plan)) {
+    // thin 16-bit F(2x2, 3x3) layers: one kernel, no V and M
+    if (!U) {
+      rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
+      if (rc) return rc;
+      U = Uws;
+    }
+    return thin_conv_forward(d, &L.plan, x, U, bias, y, stream);
+  }
   if (!U) {
     rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
     if (rc) return rc;

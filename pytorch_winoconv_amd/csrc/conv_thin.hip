@@ -1,0 +1,334 @@
+// One-kernel F(2x2, 3x3) convolution for thin 16-bit layers (at most 64 input channels).
+//
+// Same arithmetic as the three-kernel path (input transform of src/split_kernel.cu:60-120, the
+// batched product of src/base_conv_launchers.cu:353-367, output transform of
+// src/split_kernel.cu:126-203), without V and M in HBM.  With few channels the product has so
+// little arithmetic per byte that the transform-domain buffers (4x the input and 4x the output
+// for this tile) are all the cost; here x is read once and y written once.
+//
+// What makes it fit: U of one wavefront's 16 output channels (16 elements x 16 x Cp) stays in
+// registers for the life of the workgroup, so LDS only carries the transformed input of the
+// 16 tiles in flight.  A workgroup (4 wavefronts, 16 output channels each) walks over blocks of
+// 16 tiles: every thread loads the 4 x 4 window of one tile for Cp / 16 channels, transforms it in
+// fp32 and stores the 16 elements to LDS in the storage type; after one barrier every wavefront
+// multiplies all 16 elements by its part of U on v_mfma_f32_16x16x32 (U as the row operand, so
+// a lane ends up with 4 consecutive output channels of one tile).  The width half of the output
+// transform happens in the MFMA accumulators (A^T has only 0 and +-1: elements are added into the
+// accumulators they belong to, with the sign applied to the operand), the height half in fp32
+// registers.  The window of the next block is loaded before the products of this one, and LDS is
+// double-buffered, so there is one barrier per block.
+#include "wc_transform.h"
+#include <algorithm>
+
+namespace wc {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+namespace {
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<half_t> {
+  using Frag = half8;
+  __device__ static __forceinline__ floatx4 run(Frag a, Frag b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<bf16_t> {
+  using Frag = bf16x8;
+  __device__ static __forceinline__ floatx4 run(Frag a, Frag b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// The accumulator scheme below is written for these matrices.
+static_assert(Mats<KIND_23>::at(0, 0) == 1 && Mats<KIND_23>::at(0, 1) == 1 && Mats<KIND_23>::at(0, 2) == 1 &&
+              Mats<KIND_23>::at(0, 3) == 0 && Mats<KIND_23>::at(1, 0) == 0 && Mats<KIND_23>::at(1, 1) == 1 &&
+              Mats<KIND_23>::at(1, 2) == -1 && Mats<KIND_23>::at(1, 3) == -1, "A^T of F(2,3)");
+
+constexpr int kThinTiles = 16;      // tiles per block
+constexpr int kThinK = 64;          // output channels per workgroup
+
+struct ThinArgs {
+  const void* x;
+  const void* U;
+  const void* bias;
+  void* y;
+  int H, W, C, K;
+  int oH, oW, nH, nW;
+  int pad1, pad2;
+  int P;          // tiles of the whole batch
+  int n_blocks;   // ceil(P / 16)
+  int per_xcd;    // gridDim.x / 8
+  int x_bytes;    // size of x, below 1 GiB
+  int y_bytes;    // size of y, below 2 GiB
+  int row_bytes;  // W * C * sizeof(T)
+  int k_whole;    // K is a multiple of 4: a lane's 4 output channels go out in one store
+  FastDiv div_nW, div_nH;
+};
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// B^T of F(2,3) along one axis of a 4 x 4 block (STRIDE: distance between the four elements,
+// OTHER: distance between the four lines).
+template <int STRIDE, int OTHER, typename V>
+__device__ __forceinline__ void bt23(const V (&in)[16], V (&out)[16]) {
+#pragma unroll
+  for (int l = 0; l < 4; ++l) {
+    const V d0 = in[l * OTHER], d1 = in[l * OTHER + STRIDE], d2 = in[l * OTHER + 2 * STRIDE], d3 = in[l * OTHER + 3 * STRIDE];
+    out[l * OTHER] = d0 - d2;
+    out[l * OTHER + STRIDE] = d1 + d2;
+    out[l * OTHER + 2 * STRIDE] = d2 - d1;
+    out[l * OTHER + 3 * STRIDE] = d1 - d3;
+  }
+}
+static_assert(Mats<KIND_23>::bt(0, 0) == 1 && Mats<KIND_23>::bt(0, 2) == -1 && Mats<KIND_23>::bt(1, 1) == 1 &&
+              Mats<KIND_23>::bt(1, 2) == 1 && Mats<KIND_23>::bt(2, 1) == -1 && Mats<KIND_23>::bt(2, 2) == 1 &&
+              Mats<KIND_23>::bt(3, 1) == 1 && Mats<KIND_23>::bt(3, 3) == -1, "B^T of F(2,3)");
+
+template <typename T, int CP>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
+  constexpr int VEC = CP / 16;            // channels per thread in the transform
+  constexpr int KS = CP / 32;             // MFMA steps along the channels
+  constexpr int PITCH = CP * 2 + 16;      // bytes per (element, tile) row in LDS; the pad spreads 16 rows over all banks
+  constexpr int BUF = 16 * kThinTiles * PITCH;
+  using MF = Mfma16<T>;
+  using Frag = typename MF::Frag;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kbase = blockIdx.y * kThinK + wave * 16;
+
+  // transform role: tile pl of the block, channels c .. c + VEC.  x is read through a buffer descriptor:
+  // one 32-bit offset per load, and a window element outside the image is an offset beyond the
+  // buffer, which reads as zero.
+  const int pl = tid >> 4;
+  const int c = (tid & 15) * VEC;
+  const bool c_ok = c < a.C;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.x), 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ydesc = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+  Pack<T, VEC> raw[16];
+
+  // Offset of a window element = row part + column part.  A row outside the image contributes
+  // 2^31 and a column outside 2^30: with x below 1 GiB every sum that contains one of them lies
+  // beyond the buffer, so no per-element select is needed.
+  auto load_window = [&](int blk) {
+    const int p = blk * kThinTiles + pl;
+    const bool valid = p < a.P && c_ok;
+    const int q = fast_div(p, a.div_nW);
+    const int tw = p - q * a.nW;
+    const int b = fast_div(q, a.div_nH);
+    const int th = q - b * a.nH;
+    const int y0 = 2 * th - a.pad1, x0 = 2 * tw - a.pad2;
+    const unsigned row0 = (unsigned)(b * a.H + y0) * (unsigned)a.row_bytes;
+    const unsigned col0 = (unsigned)(x0 * a.C + c) * (unsigned)sizeof(T);
+    unsigned rowoff[4], coloff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      rowoff[i] = valid && (unsigned)(y0 + i) < (unsigned)a.H ? row0 + i * a.row_bytes : 0x80000000u;
+      coloff[i] = (unsigned)(x0 + i) < (unsigned)a.W ? col0 + i * a.C * (unsigned)sizeof(T) : 0x40000000u;
+    }
+#pragma unroll
+    for (int i1 = 0; i1 < 4; ++i1)
+#pragma unroll
+      for (int i2 = 0; i2 < 4; ++i2) raw[i1 * 4 + i2] = buffer_load_pack<T, VEC>(rsrc, rowoff[i1] + coloff[i2]);
+  };
+
+  const int nwg = gridDim.x;
+  int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  if (blk < a.n_blocks) load_window(blk);   // in flight while U arrives
+
+  // this wavefront's part of U: row operand, lane = output channel kbase + lane % 16, 8 channels
+  // from 8 * (lane / 16).  Rows beyond K repeat row K - 1: a row of U only reaches the same row of the
+  // product, and those rows are never stored.
+  Frag u[16][KS];
+  {
+    const int ko = kbase + (lane & 15);
+    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + 8 * (lane >> 4);
+    static_for<0, 16>([&](auto t_) {
+      constexpr int t = decltype(t_)::value;
+      static_for<0, KS>([&](auto s_) {
+        constexpr int s = decltype(s_)::value;
+        u[t][s] = *reinterpret_cast<const Frag*>(U + (long long)t * a.K * CP + s * 32);
+      });
+    });
+  }
+
+  for (int it = 0; blk < a.n_blocks; blk += nwg, ++it) {
+    unsigned char* buf = lds + (it & 1) * BUF;
+    // Input transform, two channels at a time.  fp16 adds pairs of channels
+    // in fp16 like the reference's kernels (calculation_kernels.cu:786-806 computes in T); bf16,
+    // which has no packed add, goes through fp32.
+    T* vdst = reinterpret_cast<T*>(buf + pl * PITCH) + c;
+    static_for<0, VEC / 2>([&](auto h_) {
+      constexpr int h = decltype(h_)::value;
+      if constexpr (std::is_same<T, half_t>::value) {
+        half2v d[16], t2[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) d[e] = half2v{raw[e].v[2 * h], raw[e].v[2 * h + 1]};
+        bt23<1, 4>(d, t2);
+        bt23<4, 1>(t2, d);
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          *reinterpret_cast<half2v*>(vdst + e * (kThinTiles * PITCH / 2) + 2 * h) = d[e];
+      } else {
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        float2v d[16], t2[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          d[e] = float2v{static_cast<float>(raw[e].v[2 * h]), static_cast<float>(raw[e].v[2 * h + 1])};
+        bt23<1, 4>(d, t2);
+        bt23<4, 1>(t2, d);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float o[2] = {d[e][0], d[e][1]};
+          store_pack<T, 2>(vdst + e * (kThinTiles * PITCH / 2) + 2 * h, o);
+        }
+      }
+    });
+    __syncthreads();
+    if (blk + nwg < a.n_blocks) load_window(blk + nwg);
+
+    // Width half of the output transform in the accumulators, M[i][j] = U[i][j] V[i][j] over the channels:
+    // z0[i] = M[i][0] + M[i][1] + M[i][2], and M[i][1] - (M[i][2] + M[i][3]) as zp[i] - zn[i] (no operand
+    // needs its sign changed).  Consecutive MFMAs write different accumulators.
+    floatx4 z0[4], zp[4], zn[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const unsigned char* vrow = buf + (lane & 15) * PITCH + 16 * (lane >> 4);
+    static_for<0, KS>([&](auto s_) {
+      constexpr int s = decltype(s_)::value;
+      static_for<0, 4>([&](auto j_) {
+        constexpr int j = decltype(j_)::value;
+        Frag v[4];
+        static_for<0, 4>([&](auto i_) {
+          constexpr int i = decltype(i_)::value;
+          v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + s * 64);
+        });
+        static_for<0, 4>([&](auto i_) {
+          constexpr int i = decltype(i_)::value;
+          if constexpr (j <= 2) z0[i] = MF::run(u[i * 4 + j][s], v[i], z0[i]);
+        });
+        static_for<0, 4>([&](auto i_) {
+          constexpr int i = decltype(i_)::value;
+          if constexpr (j == 1) zp[i] = MF::run(u[i * 4 + j][s], v[i], zp[i]);
+          if constexpr (j >= 2) zn[i] = MF::run(u[i * 4 + j][s], v[i], zn[i]);
+        });
+      });
+    });
+
+    // height half of the output transform, bias, store: lane = tile lane % 16, output channels
+    // ko .. ko + 4.  Stores go through a buffer descriptor: an output position outside (oH, oW) gets
+    // an offset beyond the buffer and is dropped.
+    const int p = blk * kThinTiles + (lane & 15);
+    const int ko = kbase + 4 * (lane >> 4);
+    if (p < a.P && ko < a.K) {
+      const int q = fast_div(p, a.div_nW);
+      const int tw = p - q * a.nW;
+      const int b = fast_div(q, a.div_nH);
+      const int th = q - b * a.nH;
+      const T* bias = static_cast<const T*>(a.bias);
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (ko + r < a.K) bv[r] = static_cast<float>(bias[ko + r]);
+      }
+      floatx4 zw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) zw[i] = zp[i] - zn[i];
+      const unsigned o00 = (((unsigned)b * a.oH + 2 * th) * a.oW + 2 * tw) * a.K + ko;   // in elements
+      const bool h1 = 2 * th + 1 < a.oH, w1 = 2 * tw + 1 < a.oW;
+#pragma unroll
+      for (int oa = 0; oa < 2; ++oa) {
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob) {
+          floatx4 s4;
+          if (ob == 0) s4 = oa == 0 ? z0[0] + z0[1] + z0[2] : z0[1] - z0[2] - z0[3];
+          else s4 = oa == 0 ? zw[0] + zw[1] + zw[2] : zw[1] - zw[2] - zw[3];
+          const bool inside = (oa == 0 || h1) && (ob == 0 || w1);
+          const unsigned off = o00 + (oa * a.oW + ob) * a.K;
+          Pack<T, 4> o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o.v[r] = static_cast<T>(s4[r] + bv[r]);
+          if (a.k_whole) {
+            typedef unsigned u2 __attribute__((ext_vector_type(2)));
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, o), ydesc,
+                                                  inside ? off * (unsigned)sizeof(T) : kOutside, 0, 0);
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, o.v[r]), ydesc,
+                                                    inside && ko + r < a.K ? (off + r) * (unsigned)sizeof(T) : kOutside, 0, 0);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int CP>
+int launch_thin(ThinArgs a, int k_groups, void* stream) {
+  constexpr int lds = 2 * 16 * kThinTiles * (CP * 2 + 16);
+  // two workgroups per CU stay resident (registers and LDS); fewer when the output channels are split
+  int wgs = std::min(a.n_blocks, std::max(8, 512 / k_groups));
+  a.per_xcd = ceil_div(wgs, kXcds);
+  WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipLaunchKernelGGL((thin_conv3x3_kernel<T, CP>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256),
+                     lds, as_stream(stream), a);
+  WC_CHECK_LAUNCH("thin_conv3x3_kernel");
+  return WC_OK;
+}
+
+}  // namespace
+
+bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan) {
+  if (d->ndim != 2 || d->dtype == WC_F32 || d->whole_kernel) return false;
+  if (plan->n_pieces != 1 || plan->tap_step != 1 || plan->m[0] != 1 || plan->m[1] != 2 || plan->m[2] != 2) return false;
+  const wc_piece& pc = plan->piece[0];
+  if (pc.r[0] != 1 || pc.r[1] != 3 || pc.r[2] != 3) return false;
+  const int Cp = wc_padded_channels(d->C);
+  if (Cp > 64 || d->C % (Cp / 16) != 0) return false;
+  if ((long long)d->N * d->in[1] * d->in[2] * d->C * 2 >= (1ll << 30)) return false;   // 32-bit offsets into x, two spare bits
+  int out[3], grid[3];
+  if (wc_conv_out_dims(d, out, grid) != WC_OK) return false;
+  if ((long long)d->N * out[1] * out[2] * d->K * 2 >= (1ll << 31)) return false;      // and into y
+  return d->K <= 2 * kThinK;
+}
+
+int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x, const void* U, const void* bias,
+                      void* y, void* stream) {
+  WC_CHECK_ARG(thin_conv_fits(d, plan), "thin_conv_forward: problem outside the kernel's range");
+  int out[3], grid[3];
+  int rc = wc_conv_out_dims(d, out, grid);
+  if (rc) return rc;
+  const int Cp = wc_padded_channels(d->C);
+  const long long P = (long long)d->N * grid[1] * grid[2];
+  WC_CHECK_ARG(P < (1ll << 31) - kThinTiles, "thin_conv_forward: too many tiles");
+  WC_CHECK_ARG((reinterpret_cast<uintptr_t>(x) & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 7) == 0 &&
+                   (reinterpret_cast<uintptr_t>(U) & 15) == 0,
+               "thin_conv_forward: x and y must be 8-byte aligned, U 16-byte aligned");
+  ThinArgs a;
+  a.x = x; a.U = U; a.bias = bias; a.y = y;
+  a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.K = d->K;
+  a.oH = out[1]; a.oW = out[2]; a.nH = grid[1]; a.nW = grid[2];
+  a.pad1 = d->pad[1]; a.pad2 = d->pad[2];
+  a.P = (int)P;
+  a.n_blocks = (int)ceil_div_ll(P, kThinTiles);
+  a.per_xcd = 0;
+  a.x_bytes = (int)((long long)d->N * d->in[1] * d->in[2] * d->C * 2);
+  a.y_bytes = (int)((long long)d->N * out[1] * out[2] * d->K * 2);
+  a.k_whole = d->K % 4 == 0;
+  a.row_bytes = d->in[2] * d->C * 2;
+  a.div_nW = make_fast_div(a.nW);
+  a.div_nH = make_fast_div(a.nH);
+  const int k_groups = ceil_div(d->K, kThinK);
+  if (d->dtype == WC_F16) return Cp == 64 ? launch_thin<half_t, 64>(a, k_groups, stream) : launch_thin<half_t, 32>(a, k_groups, stream);
+  return Cp == 64 ? launch_thin<bf16_t, 64>(a, k_groups, stream) : launch_thin<bf16_t, 32>(a, k_groups, stream);
+}
+
+}  // namespace wc

@@ -92,4 +92,10 @@ int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const floa
 int batched_gemm_tn(const void* A, const void* B, float* D, int T, long long P, int lda, int ldb, int na, int nb,
                     int ldd, int S, int Pq, int dtype, void* stream);
 
+// One-kernel F(2x2, 3x3) forward pass for thin 16-bit layers (conv_thin.hip): whether the problem
+// with this single-piece plan is in its range, and the launch.  U (16, K, Cp) from wc_filter_transform.
+bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan);
+int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x, const void* U, const void* bias,
+                      void* y, void* stream);
+
 }  // namespace wc

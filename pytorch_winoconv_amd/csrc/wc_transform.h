@@ -72,4 +72,41 @@ __device__ __forceinline__ void store_pack(T* p, const float (&src)[VEC]) {
   *reinterpret_cast<Pack<T, VEC>*>(p) = v;
 }
 
+// VEC consecutive elements through one buffer load: the buffer descriptor carries the base and
+// the size of the input, the per-lane address is one 32-bit offset (half the registers of a 64-bit
+// pointer per load), and an offset beyond the size - which is how a window element outside the
+// image is encoded - reads as zero in hardware, so no select is needed afterwards.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> buffer_load_pack(__amdgpu_buffer_rsrc_t rsrc, unsigned off) {
+  if constexpr (sizeof(T) * VEC == 2) {
+    const unsigned short raw = __builtin_amdgcn_raw_buffer_load_b16(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  } else if constexpr (sizeof(T) * VEC == 4) {
+    const unsigned raw = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  } else {
+    static_assert(sizeof(T) * VEC == 8, "buffer_load_pack: 2, 4 or 8 bytes per lane");
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  }
+}
+
+constexpr unsigned kOutside = 0x80000000u;   // >= the descriptor's size (the host keeps it below 2 GiB)
+
+// Division of 0 <= n < 2^31 by a divisor fixed on the host: q = (n * mul) >> (31 + shift) with
+// shift = ceil(log2 d) and mul = floor(2^(31 + shift) / d) + 1 (exact: the excess of mul * d over
+// 2^(31 + shift) is at most d <= 2^shift, so n times it stays below 2^(31 + shift)).
+struct FastDiv {
+  unsigned mul, shift;
+};
+inline FastDiv make_fast_div(int d) {
+  unsigned s = 0;
+  while ((1ll << s) < d) ++s;
+  return FastDiv{(unsigned)((1ull << (31 + s)) / (unsigned)d + 1), s};
+}
+__device__ __forceinline__ int fast_div(int n, FastDiv f) {
+  return (int)(((unsigned long long)(unsigned)n * f.mul) >> (31 + f.shift));
+}
+
 }  // namespace wc

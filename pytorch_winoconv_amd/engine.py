@@ -40,7 +40,8 @@ def _triple(v, nd, fill):
     return ((fill,) if nd == 2 else ()) + v
 
 
-def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False, stacked=False):
+def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False, stacked=False,
+              unfused=False):
     """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter.  `whole_kernel`: one
     F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces.  `stacked`: the
     DWM pieces share one tile and are added by the batched GEMM instead of by the output transform
@@ -68,6 +69,7 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
     d.stacked = int(bool(stacked))
+    d.unfused = int(bool(unfused))
     return d
 
 
@@ -188,6 +190,18 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     return 1 < n <= 4
 
 
+def thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
+    """True for the layers wc_conv_forward runs as one fused F(2x2, 3x3) kernel (wc_conv_desc.unfused):
+    fp16 / bf16, 2-D, 3x3, stride 1, at most 64 input channels (padded to 32 or 64, so a multiple of 2 or
+    4) and 128 output channels.  Callers that cache U use it to transform the filter with tile 2."""
+    if dtype == torch.float32 or nd != 2 or tuple(kernel) != (3, 3):
+        return False
+    if (stride if isinstance(stride, int) else max(stride)) != 1:
+        return False
+    cp = (in_channels + 31) // 32 * 32
+    return cp <= 64 and in_channels % (cp // 16) == 0 and out_channels <= 128
+
+
 def check_u(desc, U):
     """A transformed filter made with other options (tile, stacking) has another size: refuse it
     rather than read it with the wrong layout."""
@@ -209,10 +223,11 @@ def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, s
 
 
 def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False,
-                 stacked=None):
+                 stacked=None, unfused=False):
     """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
-    without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses."""
+    without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses.
+    `unfused=True` keeps thin 16-bit 3x3 layers on the three-kernel path (wc_conv_desc.unfused)."""
     _require_gpu(x, w, bias, U)
     stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
@@ -225,7 +240,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
     desc, y_shape, nbytes, u_elems = _forward_setup(tuple(x.shape), tuple(w.shape), x.dtype, stride, padding, m,
-                                                    chunk_images, whole_kernel, stacked)
+                                                    chunk_images, whole_kernel, stacked, unfused)
     x_cl = channel_last(x)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
@@ -241,16 +256,16 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
 _SETUPS = {}
 
 
-def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked):
+def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused=False):
     """Descriptor, output shape (channel-last), workspace bytes and size of U for one problem.  Kept
     per problem: for small layers (a few tens of microseconds on the GPU) rebuilding them on every
     call costs as much host time as the launches themselves."""
     key = (x_shape, w_shape, dtype, stride if isinstance(stride, int) else tuple(stride),
-           padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked)
+           padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked, unfused)
     hit = _SETUPS.get(key)
     if hit is None:
         lib = _lib.load()
-        desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked)
+        desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused)
         out, _ = out_dims(desc)
         nbytes, ue = ctypes.c_size_t(), ctypes.c_size_t()
         check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))

@@ -210,13 +210,31 @@ def test_stacked_plans():
 
 def test_modules_pick_tile_2_where_tile_4_loses_accuracy():
     import pytorch_winoconv_amd as pkg
-    wide, thin = pkg.WinoConv2d(64, 64, 3, padding=1), pkg.WinoConv2d(3, 64, 3, padding=1)
+    wide, thin = pkg.WinoConv2d(256, 256, 3, padding=1), pkg.WinoConv2d(3, 64, 3, padding=1)
     assert wide._tile_for(torch.float16) == 4 and wide._tile_for(torch.float32) == 4
     assert wide._tile_for(torch.bfloat16) == 2          # 8 mantissa bits
     assert thin._tile_for(torch.float16) == 2            # too few channels to average the rounding error down
     assert thin._tile_for(torch.float32) == 4
     assert pkg.WinoConv2d(3, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4   # an explicit choice stands
     assert pkg.WinoConv3d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
+
+
+def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
+    """The cached U of a module must be the F(2,3) one wherever wc_conv_forward runs its fused kernel."""
+    import pytorch_winoconv_amd as pkg
+    from pytorch_winoconv_amd import engine
+    assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
+    assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float32) == 4
+    assert pkg.WinoConv2d(64, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4
+    assert pkg.WinoConv2d(64, 256, 3, padding=1)._tile_for(torch.float16) == 4      # too many output channels
+    assert pkg.WinoConv2d(96, 64, 3, padding=1)._tile_for(torch.float16) == 4       # too many input channels
+    assert pkg.WinoConv2d(64, 64, 5, padding=2)._tile_for(torch.float16) == 4
+    assert pkg.WinoConv2d(64, 64, 3, stride=2, padding=1)._tile_for(torch.float16) == 4
+    t = engine.thin_layer
+    assert t(torch.float16, 2, 64, 128, (3, 3), 1) and t(torch.bfloat16, 2, 16, 8, (3, 3), (1, 1))
+    assert t(torch.float16, 2, 40, 8, (3, 3), 1) and not t(torch.float16, 2, 42, 8, (3, 3), 1)   # 4 channels per thread
+    assert t(torch.float16, 2, 30, 8, (3, 3), 1) and not t(torch.float16, 2, 3, 8, (3, 3), 1)    # 2 channels per thread
+    assert not t(torch.float16, 3, 64, 64, (3, 3), 1) and not t(torch.float32, 2, 64, 64, (3, 3), 1)
 
 
 def test_product_generator_equals_oracle_generator():

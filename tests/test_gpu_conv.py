@@ -92,12 +92,13 @@ def test_conv_vs_oracle_same_discipline(dev, dtype, case):
     """HIP result against the CPU restatement with the same storage/rounding points: only the
     summation order differs.  fp32: <= 1e-5.  fp16: a different order flips single fp16
     roundings of M by one ulp (4.9e-4 relative), which A^T x A^T of F(4,3) amplifies by up to
-    64: <= 1e-2 of the output range."""
+    64: <= 1e-2 of the output range.  `unfused`: thin 16-bit 3x3 layers otherwise take the
+    one-kernel path, which keeps the product in fp32 (test_gpu_thin.py)."""
     xs, ws, stride, pad, m = case
     x, w, _ = _data(xs, ws, dtype, seed=5)
     om = (2, 4, 4) if (m == 4 and len(xs) == 5) else m        # the engine's 3-D "tile 4" is 2 x 4 x 4
     want = ow.dwm_conv(x, w, None, stride, pad, om, DISC[dtype])
-    y = engine.conv_forward(x.to(dev), w.to(dev), None, stride, pad, m)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, stride, pad, m, unfused=True)
     assert _nerr(y, want.double()) <= (1e-5 if dtype == torch.float32 else 1e-2)
 
 

@@ -1,0 +1,140 @@
+"""The one-kernel F(2x2, 3x3) path that wc_conv_forward takes for thin fp16 / bf16 3x3 stride-1 layers
+(at most 64 input channels; conv_thin.hip).  It computes what the three-kernel path computes
+(input transform of src/split_kernel.cu:60-120, batched product of
+src/base_conv_launchers.cu:353-367, output transform of src/split_kernel.cu:126-203) without V and M
+in memory, so the product is not rounded to the storage type before the output transform.
+
+Pinned three ways: bit-exact against an integer convolution on inputs for which every intermediate
+is exactly representable (any wrong index, sign or dropped term changes an integer); against fp64
+convolution and the CPU oracle on normal inputs (fp16 and bf16 2e-2 of the output range, the bound
+of the three-kernel path with this tile); and against the three-kernel path itself."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import winograd as ow
+from pytorch_winoconv_amd import engine
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    # N, C, K, H, W, pad
+    (2, 64, 64, 8, 8, 1),
+    (1, 64, 64, 7, 9, 1),        # odd output sizes: half-used tiles on both edges
+    (3, 32, 64, 13, 11, 0),
+    (2, 16, 48, 9, 9, 1),        # channels padded to 32, two per thread
+    (2, 64, 128, 12, 12, 1),     # two groups of output channels
+    (2, 40, 20, 10, 10, 1),      # channels padded to 64; K no multiple of 16
+    (1, 64, 6, 5, 5, 1),         # K no multiple of 4: element-wise stores
+    (1, 8, 7, 4, 4, 1),
+    (2, 64, 64, 3, 3, 0),        # one output pixel
+    (1, 24, 32, 6, 20, 2),       # padding wider than the kernel needs
+    (5, 64, 64, 30, 30, 1),      # more tiles than one round of workgroups' first blocks
+]
+
+
+def _rel(a, r):
+    r = r.double()
+    return float((a.double().cpu() - r).abs().max() / r.abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_exact_on_small_integers(dev, dtype, shape):
+    """x in -3..3, filter taps multiples of 4 (so G g G^T holds integers), integer bias: every
+    transformed value, product and sum is an integer below 2^24, exact in both storage types and
+    in the fp32 accumulators; the only rounding is the final one, of the exact result."""
+    N, C, K, H, W, pad = shape
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(-3, 4, (N, C, H, W), generator=g).double()
+    w = 4.0 * torch.randint(-2, 3, (K, C, 3, 3), generator=g).double()
+    b = torch.randint(-8, 9, (K,), generator=g).double()
+    ref = F.conv2d(x, w, b, padding=pad).float().to(dtype)
+    y = engine.conv_forward(x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev), 1, pad, 2)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert torch.equal(y.cpu(), ref), float((y.cpu().double() - ref.double()).abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_against_fp64_oracle_and_three_kernel_path(dev, dtype, shape):
+    N, C, K, H, W, pad = shape
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(N, C, H, W, generator=g).to(dtype)
+    w = (torch.randn(K, C, 3, 3, generator=g) * (2.0 / (9 * C)) ** 0.5).to(dtype)
+    b = torch.randn(K, generator=g).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=pad)
+    y_oracle = ow.dwm_conv(x, w, b, 1, pad, 2, "fp16" if dtype == torch.float16 else "bf16")
+    xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
+    y = engine.conv_forward(xd, wd, bd, 1, pad, 2)
+    y3 = engine.conv_forward(xd, wd, bd, 1, pad, 2, unfused=True)
+    tol = 2e-2                                   # of the output range, both types, tile 2
+    assert _rel(y, ref) <= tol and _rel(y3, ref) <= tol
+    assert _rel(y, y_oracle) <= tol and _rel(y, y3.cpu()) <= tol
+    # the product stays in fp32 here: no further from fp64 than the three-kernel path, rounding noise aside
+    assert _rel(y, ref) <= 1.5 * _rel(y3, ref) + 1e-4
+    no_bias = engine.conv_forward(xd, wd, None, 1, pad, 2)
+    assert _rel(no_bias, F.conv2d(x.double(), w.double(), None, padding=pad)) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_tile_request_and_cached_filter(dev, dtype):
+    """The fused kernel is the F(2,3) one: it runs for tile 2, with or without a cached U, and
+    never for tile 4."""
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(3, 48, 17, 15, generator=g).to(dtype).to(dev)
+    w = (torch.randn(40, 48, 3, 3, generator=g) * 0.05).to(dtype).to(dev)
+    b = torch.randn(40, generator=g).to(dtype).to(dev)
+    y2 = engine.conv_forward(x, w, b, 1, 1, 2)
+    U2 = engine.transform_filter(w, x.shape, 1, 1, 2)
+    assert torch.equal(engine.conv_forward(x, w, b, 1, 1, 2, U=U2), y2)
+    U4 = engine.transform_filter(w, x.shape, 1, 1, 4)
+    y4 = engine.conv_forward(x, w, b, 1, 1, 4, unfused=True)
+    assert torch.equal(engine.conv_forward(x, w, b, 1, 1, 4, U=U4), y4)
+    assert torch.equal(engine.conv_forward(x, w, b, 1, 1, 4), y4)
+    # unfused = stage by stage
+    desc = engine.make_desc(x.shape, w.shape, dtype, 1, 1, 2)
+    plan = engine.plan_conv(desc)
+    V = engine.input_transform(desc, plan, engine.channel_last(x))
+    M = engine.batched_gemm(V, engine.filter_transform(desc, plan, w))
+    y_st = engine.output_transform(desc, plan, M, b, x.shape[0])
+    y3 = engine.conv_forward(x, w, b, 1, 1, 2, unfused=True)
+    assert torch.equal(y3.permute(0, 2, 3, 1), y_st[:, 0])
+    assert not torch.equal(y3, y2)               # other roundings: the fused kernel did run above
+
+
+@pytest.mark.parametrize("case", [
+    # x shape, w shape, stride, dtype: outside the fused kernel's range, same result with and without `unfused`
+    ((2, 3, 9, 9), (8, 3, 3, 3), 1, torch.float16),          # odd channel count
+    ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float16),        # more than 64 input channels
+    ((2, 64, 9, 9), (136, 64, 3, 3), 1, torch.float16),      # more than 128 output channels
+    ((2, 64, 12, 12), (8, 64, 3, 3), 2, torch.float16),      # stride 2
+    ((2, 64, 12, 12), (8, 64, 5, 5), 1, torch.float16),      # DWM plan
+    ((2, 64, 9, 9), (8, 64, 3, 3), 1, torch.float32),
+    ((2, 64, 5, 9, 9), (8, 64, 3, 3, 3), 1, torch.float16),  # 3-D
+])
+def test_outside_the_range_nothing_changes(dev, case):
+    xs, ws, stride, dtype = case
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(*xs, generator=g).to(dtype).to(dev)
+    w = (torch.randn(*ws, generator=g) * 0.05).to(dtype).to(dev)
+    assert torch.equal(engine.conv_forward(x, w, None, stride, 1, 2),
+                       engine.conv_forward(x, w, None, stride, 1, 2, unfused=True))
+
+
+def test_resnet_layer_at_full_size(dev):
+    """N=64, C=K=64, 56x56 fp16 (the first ResNet-50 3x3 shape): fused against three kernels, and
+    linearity in the filter (conv(x, w1 + w2) = conv(x, w1) + conv(x, w2) up to rounding)."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(64, 64, 56, 56, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    w1 = (torch.randn(64, 64, 3, 3, generator=g) * (2.0 / 576) ** 0.5).half().to(dev)
+    w2 = (torch.randn(64, 64, 3, 3, generator=g) * (2.0 / 576) ** 0.5).half().to(dev)
+    y1 = engine.conv_forward(x, w1, None, 1, 1, 2)
+    y3 = engine.conv_forward(x, w1, None, 1, 1, 2, unfused=True)
+    scale = float(y3.float().abs().max())
+    assert float((y1.float() - y3.float()).abs().max()) <= 4e-3 * scale
+    y2 = engine.conv_forward(x, w2, None, 1, 1, 2)
+    y12 = engine.conv_forward(x, (w1.float() + w2.float()).half(), None, 1, 1, 2)
+    assert float((y12.float() - y1.float() - y2.float()).abs().max()) <= 6e-3 * scale
+    sample = F.conv2d(x[:2].double().cpu(), w1.double().cpu(), padding=1)
+    assert _rel(y1[:2], sample) <= 2e-3
