@@ -164,7 +164,7 @@ int wc_output_transform(const wc_conv_desc* desc, const wc_plan* plan,
  * tmp_product_buffer: dwm.py:122-125); images are processed in chunks that bound the size
  * of V and M.  `U_cached` (may be NULL) is a filter already transformed
  * by wc_filter_transform; `w` may then be NULL.  Thin 16-bit 3x3 layers take one fused kernel
- * instead (see wc_conv_desc.unfused); the workspace requirement is the same either way. */
+ * instead (see wc_conv_desc.unfused); the workspace then only holds U. */
 int wc_conv_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
 int wc_conv_u_elems(const wc_conv_desc* desc, size_t* elems);
 int wc_conv_forward(const wc_conv_desc* desc, const void* x,

@@ -21,6 +21,8 @@ struct Layout {
   long long tiles_per_image;
   size_t es;
   size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
+  bool thin;                          // the one-kernel path runs: V and M are not needed
+  size_t need() const { return thin ? u_bytes : u_bytes + v_bytes + m_bytes; }
 };
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -54,6 +56,7 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   L->u_bytes = round256((size_t)T * d->K * L->Cp * L->es);
   L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
+  L->thin = !d->unfused && thin_conv_fits(d, &L->plan);
   return WC_OK;
 }
 
@@ -66,7 +69,7 @@ int wc_conv_workspace_bytes(const wc_conv_desc* d, size_t* bytes) {
   Layout L;
   int rc = make_layout(d, &L);
   if (rc) return rc;
-  *bytes = L.u_bytes + L.v_bytes + L.m_bytes;
+  *bytes = L.need();
   return WC_OK;
 }
 
@@ -88,7 +91,7 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   WC_CHECK_ARG(x && y, "wc_conv_forward: null input or output");
   WC_CHECK_ARG(U_cached || (w && w_strides), "wc_conv_forward: neither a filter nor a transformed filter");
   if (!workspace) return fail(WC_ERR_WORKSPACE, "wc_conv_forward: null workspace");
-  const size_t need = L.u_bytes + L.v_bytes + L.m_bytes;
+  const size_t need = L.need();
   if (workspace_bytes < need)
     return fail(WC_ERR_WORKSPACE, "wc_conv_forward: workspace of %zu bytes, %zu needed", workspace_bytes, need);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
@@ -99,7 +102,7 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   void* V = ws + L.u_bytes;
   void* M = ws + L.u_bytes + L.v_bytes;
   const void* U = U_cached;
-  if (!d->unfused && thin_conv_fits(d, &L.plan)) {
+  if (L.thin) {
     // thin 16-bit F(2x2, 3x3) layers: one kernel, no V and M
     if (!U) {
       rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);

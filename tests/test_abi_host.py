@@ -115,6 +115,13 @@ def test_workspace_size_is_u_plus_v_plus_m():
     desc.chunk_images = 8
     assert lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0
     assert nbytes.value == 2 * (T * 256 * 256 + 2 * T * (P // 8) * 256)
+    # a layer the one-kernel path takes needs U only; with `unfused` all three buffers again
+    thin = engine.make_desc((64, 64, 56, 56), (64, 64, 3, 3), torch.float16, 1, 1, 2)
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(thin), ctypes.byref(nbytes)) == 0
+    assert nbytes.value == 2 * 16 * 64 * 64
+    thin.unfused = 1
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(thin), ctypes.byref(nbytes)) == 0
+    assert nbytes.value == 2 * (16 * 64 * 64 + 2 * 16 * 64 * 28 * 28 * 64)
 
 
 def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
