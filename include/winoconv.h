@@ -84,7 +84,7 @@ typedef struct {
                     *    Output tile 2, or 4 in 2-D.  The plan then reports t_offset = 0 for every piece and
                     *    t_total = prod(m + r_max - 1). */
   int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2, at most 64 input
-                    *    channels (an even number up to 32, a multiple of 4 above) and at most 128 output
+                    *    channels (an even number up to 32, a multiple of 4 above) and at most 512 output
                     *    channels run as one kernel: input transform, products and output transform of
                     *    F(2x2, 3x3) without V and M in memory, the product kept in fp32 (x below 1 GiB);
                     * 1: always filter transform -> input transform -> batched GEMM -> output transform. */

@@ -273,8 +273,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <typename T, int CP>
 int launch_thin(ThinArgs a, int k_groups, void* stream) {
   constexpr int lds = 2 * 16 * kThinTiles * (CP * 2 + 16);
-  // two workgroups per CU stay resident (registers and LDS); fewer when the output channels are split
-  int wgs = std::min(a.n_blocks, std::max(8, 512 / k_groups));
+  // two workgroups per CU stay resident (registers and LDS): 512 in all, shared among the groups
+  // of output channels, in whole multiples of the 8 XCDs
+  int wgs = std::min(a.n_blocks, std::max(kXcds, 512 / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
   WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -297,7 +298,7 @@ bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan) {
   int out[3], grid[3];
   if (wc_conv_out_dims(d, out, grid) != WC_OK) return false;
   if ((long long)d->N * out[1] * out[2] * d->K * 2 >= (1ll << 31)) return false;      // and into y
-  return d->K <= 2 * kThinK;
+  return d->K <= 8 * kThinK;
 }
 
 int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x, const void* U, const void* bias,

@@ -24,6 +24,7 @@ SHAPES = [
     (3, 32, 64, 13, 11, 0),
     (2, 16, 48, 9, 9, 1),        # channels padded to 32, two per thread
     (2, 64, 128, 12, 12, 1),     # two groups of output channels
+    (3, 32, 300, 20, 20, 1),     # five groups, the last one partly filled
     (2, 40, 20, 10, 10, 1),      # channels padded to 64; K no multiple of 16
     (1, 64, 6, 5, 5, 1),         # K no multiple of 4: element-wise stores
     (1, 8, 7, 4, 4, 1),
@@ -107,7 +108,7 @@ def test_tile_request_and_cached_filter(dev, dtype):
     # x shape, w shape, stride, dtype: outside the fused kernel's range, same result with and without `unfused`
     ((2, 3, 9, 9), (8, 3, 3, 3), 1, torch.float16),          # odd channel count
     ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float16),        # more than 64 input channels
-    ((2, 64, 9, 9), (136, 64, 3, 3), 1, torch.float16),      # more than 128 output channels
+    ((2, 64, 9, 9), (520, 64, 3, 3), 1, torch.float16),      # more than 512 output channels
     ((2, 64, 12, 12), (8, 64, 3, 3), 2, torch.float16),      # stride 2
     ((2, 64, 12, 12), (8, 64, 5, 5), 1, torch.float16),      # DWM plan
     ((2, 64, 9, 9), (8, 64, 3, 3), 1, torch.float32),
