@@ -65,7 +65,14 @@ def split_plan(kD, kH, kW):
     return plan
 
 
-def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=False):
+def axis_pairs(k):
+    """Chunks of two taps, the remainder last: [(first_tap, 1, n_taps), ...].  Not a split of the
+    reference (its rule is chunks of three, base_conv_launchers.h:58-388): pieces that start at
+    even taps see, with output tile 2, the same transformed input moved by whole tiles."""
+    return [(s, 1, min(2, k - s)) for s in range(0, k, 2)]
+
+
+def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=False, pairs=False):
     """General plan for a (kD, kH, kW) kernel with one stride for all axes.
 
     Each piece is one stride-1 sub-convolution: per axis (first_tap, tap_step,
@@ -80,6 +87,9 @@ def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=Fals
     if whole_kernel:
         assert stride == 1
         per_axis = [[(0, 1, k)] for k in kernel]
+    elif pairs:
+        assert stride == 1
+        per_axis = [axis_pairs(k) for k in kernel]
     else:
         per_axis = [axis_pieces(k, stride) for k in kernel]
     # m: one output tile extent for all axes, or one per axis (depth, height, width)

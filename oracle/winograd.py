@@ -155,7 +155,7 @@ def _as_3d(x, w):
     return x, w, two_d
 
 
-def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
+def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2, whole_kernel=False, pairs=False):
     """Shapes and pieces for an NC[D]HW x (K, C, [kD,] kH, kW) convolution."""
     two_d = len(x_shape) == 4
     sp = ([1] if two_d else []) + list(x_shape[2:])
@@ -163,7 +163,7 @@ def conv_plan(x_shape, w_shape, stride=1, padding=0, m=2, whole_kernel=False):
     if isinstance(padding, int):
         padding = [padding] * (len(x_shape) - 2)
     pads = ([0] if two_d else []) + list(padding)
-    pieces, T_total = conv_pieces(ks, stride, m, degenerate_depth=two_d, whole_kernel=whole_kernel)
+    pieces, T_total = conv_pieces(ks, stride, m, degenerate_depth=two_d, whole_kernel=whole_kernel, pairs=pairs)
     od = out_dims(sp, ks, pads, stride)
     grid = tile_grid(od, pieces[0]["ms"])
     return dict(spatial=sp, kernel=ks, pads=pads, pieces=pieces, T_total=T_total,
@@ -205,9 +205,11 @@ def dwm_conv(x, w, bias=None, stride=1, padding=0, m=2, discipline="fp32", stage
     intermediate buffers U, V, M and the plan are stored in it.  `whole_kernel`: one F(m, k) tile
     per axis instead of the DWM pieces (the reference's matrix_conv arithmetic).  `stacked`: the
     pieces are summed by the batched product (see stacked_pieces); U and V then are
-    (T, K, n_pieces * C) and (T, P, n_pieces * C)."""
+    (T, K, n_pieces * C) and (T, P, n_pieces * C).  `stacked=2`: the same with pieces of two taps
+    (split_plan.axis_pairs; 2-D, stride 1, m = 2), the decomposition whose pieces share one
+    transformed input in the product path."""
     st = _STORE[discipline]
-    plan = conv_plan(tuple(x.shape), tuple(w.shape), stride, padding, m, whole_kernel)
+    plan = conv_plan(tuple(x.shape), tuple(w.shape), stride, padding, m, whole_kernel, pairs=(stacked == 2))
     x3, w3, two_d = _as_3d(x.to(st), w.to(st))
     xl = x3.permute(0, 2, 3, 4, 1).contiguous()                      # dwm.py:84, :132
     if stacked and len(plan["pieces"]) > 1:

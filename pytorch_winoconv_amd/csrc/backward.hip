@@ -234,6 +234,8 @@ struct BwdLayout {
 };
 
 int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
+  if (d && d->stacked == 2)
+    return fail(WC_ERR_UNSUPPORTED, "the weight gradient is not built for plans with a shared transformed input (stacked = 2)");
   int rc = wc_plan_conv(d, &L->plan);
   if (rc) return rc;
   rc = wc_conv_out_dims(d, L->out, L->grid);

@@ -17,7 +17,10 @@ namespace {
 struct Layout {
   wc_plan plan;
   int out[3], grid[3];
-  int Cp, ldm, chunk;   // Cp: row length of U and V (pieces side by side in a stacked plan)
+  int Cp, ldm, chunk;   // Cp: row length of U, and of V unless the pieces share one transformed input
+  int vrow;             // row length of V
+  bool shared;
+  SharedShift shift;
   long long tiles_per_image;
   size_t es;
   size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
@@ -33,6 +36,9 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   rc = wc_conv_out_dims(d, L->out, L->grid);
   if (rc) return rc;
   L->Cp = stacked_row(d, &L->plan);
+  L->vrow = v_row(d, &L->plan);
+  L->shared = shared_input(d, &L->plan);
+  L->shift = shared_shift(d, L->grid);
   L->ldm = wc_padded_channels8(d->K);
   L->es = d->dtype == WC_F32 ? 4 : 2;
   L->tiles_per_image = (long long)L->grid[0] * L->grid[1] * L->grid[2];
@@ -42,7 +48,7 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
     // Measured on MI355X (N=64, C=K=256, 56x56, fp16): one pass over the whole batch is fastest,
     // smaller chunks lose more to partially filled launches than they gain from cache residency.
     // The chunk only bounds the scratch footprint: V + M of one chunk stay below 8 GiB.
-    const double per_image = (double)T * L->tiles_per_image * (L->Cp + L->ldm) * L->es;
+    const double per_image = (double)T * L->tiles_per_image * (L->vrow + L->ldm) * L->es;
     chunk = (int)(8192.0 * 1024 * 1024 / per_image);
     if (chunk < 1) chunk = 1;
     // equal passes rather than full ones and a short last one
@@ -54,7 +60,7 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   if (T * Pc * (long long)(L->Cp > L->ldm ? L->Cp : L->ldm) >= (1ll << 40))
     return fail(WC_ERR_UNSUPPORTED, "chunk of %d images is too large", chunk);
   L->u_bytes = round256((size_t)T * d->K * L->Cp * L->es);
-  L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
+  L->v_bytes = round256((size_t)T * (Pc + (L->shared ? L->shift.tail : 0)) * L->vrow * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
   L->thin = !d->unfused && thin_conv_fits(d, &L->plan);
   return WC_OK;
@@ -124,7 +130,8 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
     WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
     rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);
     if (rc) return rc;
-    rc = wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+    rc = L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
+                  : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
     if (rc) return rc;
     rc = wc_output_transform(d, &L.plan, M, bias, n, static_cast<unsigned char*>(y) + b0 * y_image, stream);
     if (rc) return rc;

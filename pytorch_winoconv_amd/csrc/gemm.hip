@@ -64,6 +64,10 @@ struct GemmArgs {
   long long sV, sU, sM;     // batch strides in elements
   int tiles_p, tiles_k, T;
   int n_blocks, per_xcd;
+  // shifted operand (plans whose pieces share one transformed input): rows of V are ldv apart, and
+  // after every run_blocks reduction blocks the V operand jumps on by `jump` elements
+  int ldv, run_blocks;
+  long long jump;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -75,7 +79,7 @@ typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte g
 // is conflict-free for 128-byte and for 256-byte wide bank sets alike.
 __device__ __forceinline__ int swizzle(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
 
-template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2>
+template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false>
 __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
   using MF = Mfma<T>;
   constexpr int NT = 64 * NWP * NWK;               // threads: NWP x NWK wavefronts
@@ -112,7 +116,7 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
     const int row = lrow + i * RPP;                // row of the stacked [X ; W] tile
     if (row < BM) {
       const int p = min(p0 + row, g.P - 1);
-      gptr[i] = Vt + (long long)p * g.Cp + lpart * EPC;
+      gptr[i] = Vt + (long long)p * (SHIFT ? g.ldv : g.Cp) + lpart * EPC;
     } else {
       const int k = min(k0 + row - BM, g.K - 1);
       gptr[i] = Ut + (long long)k * g.Cp + lpart * EPC;
@@ -121,9 +125,11 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   }
 
   Chunk16 regs[NLOAD];
-  auto gload = [&](int kt) {
+  // `vshift`: what the V operand has jumped by at reduction block kt (rows i < BM / RPP are V's)
+  auto gload = [&](int kt, long long vshift) {
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) regs[i] = *reinterpret_cast<const Chunk16*>(gptr[i] + kt * BK);
+    for (int i = 0; i < NLOAD; ++i)
+      regs[i] = *reinterpret_cast<const Chunk16*>(gptr[i] + kt * BK + (SHIFT && i < BM / RPP ? vshift : 0));
   };
   auto lstore = [&](int buf) {
 #pragma unroll
@@ -151,12 +157,17 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int nk = g.Cp / BK;
-  gload(0);
+  long long vshift = 0;
+  int run_left = SHIFT ? g.run_blocks : 0;
+  gload(0, 0);
   lstore(0);
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
-    if (kt + 1 < nk) gload(kt + 1);
+    if constexpr (SHIFT) {
+      if (--run_left == 0) { vshift += g.jump; run_left = g.run_blocks; }
+    }
+    if (kt + 1 < nk) gload(kt + 1, vshift);
     const T* st = lds + cur * STAGE;
     // fragments of step kk+1 are read from LDS while the MFMAs of step kk run
     constexpr int KK = BK / MF::kstep;
@@ -235,14 +246,14 @@ struct GemmConfig {
   int threads;
 };
 
-template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2>
+template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false>
 static GemmConfig make_config() {
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
   constexpr int EI = sizeof(T) == 4 ? 1 : (NWP * NWK == 4 ? WM : WM / 2);
   constexpr size_t stages = (size_t)2 * (BM + BN) * BK * sizeof(T);
   constexpr size_t out_tile = (size_t)32 * NWP * EI * (BN + EPC) * sizeof(T);
-  return GemmConfig{&gemm_kernel<T, WM, WN, BK, NWP, NWK>, BM, BN, BK,
+  return GemmConfig{&gemm_kernel<T, WM, WN, BK, NWP, NWK, SHIFT>, BM, BN, BK,
                     stages > out_tile ? stages : out_tile, 64 * NWP * NWK};
 }
 
@@ -324,6 +335,48 @@ static GemmConfig choose(int T_, int P, int K, int Cp) {
   return best;
 }
 
+// Tiles for the shifted operand (16-bit types): 256 x 128, 128 x 128, 64 x 64, largest that fills the chip.
+template <typename T>
+static GemmConfig choose_shifted(int T_, int P, int K) {
+  GemmConfig c[3] = {make_config<T, 4, 2, 32, 2, 2, true>(), make_config<T, 2, 2, 32, 2, 2, true>(),
+                     make_config<T, 1, 1, 32, 2, 2, true>()};
+  for (int i = 0; i < 2; ++i) {
+    if (c[i].bn / 2 >= K) continue;
+    if ((long long)ceil_div(P, c[i].bm) * ceil_div(K, c[i].bn) * T_ >= 512) return c[i];
+  }
+  return c[2];
+}
+
+int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, int Cp, SharedShift sh, int K, int ldm,
+                         int dtype, void* stream) {
+  WC_CHECK_ARG(V && U && M, "batched_gemm_shifted: null pointer");
+  WC_CHECK_ARG(T_ > 0 && P > 0 && K > 0 && Cp > 0 && Cp % 32 == 0, "batched_gemm_shifted: T %d, P %d, K %d, Cp %d", T_, P, K, Cp);
+  WC_CHECK_ARG(sh.n_run > 0 && sh.n_runs > 0 && sh.run_rows >= sh.n_run && sh.tail == (sh.n_runs - 1) * sh.run_rows + sh.n_run - 1,
+               "batched_gemm_shifted: bad shift description");
+  WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "batched_gemm_shifted: row stride %d", ldm);
+  if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_shifted: 16-bit types only");
+  GemmConfig c = dtype == WC_F16 ? choose_shifted<half_t>(T_, P, K) : choose_shifted<bf16_t>(T_, P, K);
+  GemmArgs g;
+  g.V = V; g.U = U; g.M = M;
+  g.P = P; g.K = K; g.ldm = ldm;
+  g.Cp = sh.n_runs * sh.n_run * Cp;                      // reduction length = row length of U
+  g.ldv = Cp;
+  g.run_blocks = sh.n_run * Cp / c.bk;                   // one run: the pieces of one piece row, contiguous rows of V
+  g.jump = (long long)(sh.run_rows - sh.n_run) * Cp;     // on to the same tile one grid row further
+  g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
+  g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
+  const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
+  WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_shifted: problem too large");
+  g.n_blocks = (int)blocks;
+  g.per_xcd = ceil_div((int)blocks, kXcds);
+  if (c.lds > 64 * 1024)
+    WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+  hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
+  WC_CHECK_LAUNCH("gemm_kernel (shifted operand)");
+  return WC_OK;
+}
+
 }  // namespace wc
 
 using namespace wc;
@@ -340,6 +393,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;
   g.sV = (long long)P * Cp; g.sU = (long long)K * Cp; g.sM = (long long)P * ldm;
+  g.ldv = Cp; g.run_blocks = 0; g.jump = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

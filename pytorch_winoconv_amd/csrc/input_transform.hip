@@ -15,8 +15,9 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   const int Cp = wc_padded_channels(d->C);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
   const bool flat = plan->m[0] == 1;
-  const bool stacked = d->stacked && plan->n_pieces > 1;
-  const int row = stacked_row(d, plan);              // row length of V
+  const bool shared = shared_input(d, plan);         // one piece's transform serves all pieces (see wc_common.h)
+  const bool stacked = d->stacked && plan->n_pieces > 1 && !shared;
+  const int row = v_row(d, plan);                    // row length of V
   int rp[3];
   stacked_taps(plan, rp);
   // Channels per thread.  Measured on MI355X at N=64, C=256, 56x56 fp16: F(4,3) tiles (36 live
@@ -34,7 +35,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = row;
   a.nD = grid[0]; a.nH = grid[1]; a.nW = grid[2];
   a.step = plan->tap_step;
-  a.t_stride = P * row;
+  a.t_stride = (P + (shared ? shared_shift(d, grid).tail : 0)) * row;
   a.n_cvec = Cp / vec;
   a.total = P * a.n_cvec;
   const long long blocks = ceil_div_ll(a.total, 256);
@@ -43,6 +44,17 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
   const dim3 launch_grid((unsigned)(a.per_xcd * kXcds));
 
+  if (shared) {
+    // the first piece with the tile all pieces share, over the extended tile grid
+    WC_CHECK_ARG(flat && plan->m[1] == 2 && plan->m[2] == 2, "wc_input_transform: shared input needs a 2-D plan with output tile 2");
+    InKernel fn = pick_in_2d(d->dtype, kind_of(2, rp[1]), kind_of(2, rp[2]), vec);
+    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform F(2,%d) x F(2,%d) not built", rp[1], rp[2]);
+    a.base0 = 0; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
+    a.t_offset = 0;
+    hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
+    WC_CHECK_LAUNCH("input_transform_kernel");
+    return WC_OK;
+  }
   // 2-D DWM plans: all pieces in one launch
   bool small_taps = plan->n_pieces > 1 && flat && plan->t_total <= 0xffff;
   for (int s = 0; s < plan->n_pieces && small_taps; ++s) {

@@ -50,6 +50,13 @@ static int axis_chunks(int k, int* start, int* size) {
   return n;
 }
 
+// chunks of two taps, the remainder last (plans whose pieces share one transformed input)
+static int axis_pairs(int k, AxisPiece* out) {
+  int n = 0;
+  for (int s = 0; s < k; s += 2) { out[n].tap0 = s; out[n].r = k - s >= 2 ? 2 : 1; ++n; }
+  return n;
+}
+
 static int axis_pieces(int k, int stride, AxisPiece* out) {
   int n = 0;
   int start[8], size[8];
@@ -126,9 +133,11 @@ static int check_desc(const wc_conv_desc* d) {
     return fail(WC_ERR_UNSUPPORTED, "output tile 4 in 3-D (2 x 4 x 4) is implemented for 3x3x3 kernels at stride 1");
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
-  WC_CHECK_ARG(d->stacked == 0 || d->stacked == 1, "stacked must be 0 or 1");
+  WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
     return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
+  if (d->stacked == 2 && (d->ndim != 2 || d->stride != 1 || d->m != 2))
+    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need a 2-D problem, stride 1 and output tile 2");
   if (d->whole_kernel) {
     if (d->ndim != 2 || d->stride != 1 || d->m != 2)
       return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");
@@ -147,6 +156,7 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   int n[3];
   for (int a = 0; a < 3; ++a) {
     if (d->whole_kernel) { ax[a][0].tap0 = 0; ax[a][0].r = d->kernel[a]; n[a] = 1; }
+    else if (d->stacked == 2) n[a] = axis_pairs(d->kernel[a], ax[a]);
     else n[a] = axis_pieces(d->kernel[a], d->stride, ax[a]);
   }
   if (n[0] * n[1] * n[2] > WC_MAX_PIECES)
@@ -199,6 +209,8 @@ int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
     out[a] = (d->in[a] + 2 * d->pad[a] - d->kernel[a]) / d->stride + 1;
     int m = a == 0 ? (flat_depth ? 1 : (d->m == 4 ? 2 : d->m)) : d->m;
     grid[a] = (out[a] + m - 1) / m;
+    // a shared transformed input covers the tiles that the pieces reach beyond the output's own
+    if (d->stacked == 2) grid[a] += (d->kernel[a] + 1) / 2 - 1;
   }
   return WC_OK;
 }

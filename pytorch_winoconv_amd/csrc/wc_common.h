@@ -72,6 +72,30 @@ inline int stacked_row(const wc_conv_desc* d, const wc_plan* plan) {
   return wc_padded_channels(d->C) * (d->stacked ? plan->n_pieces : 1);
 }
 
+// Plans with stacked == 2: the pieces start at even taps and use one tile F(2, 2 or 1) per axis, so
+// the transformed input of the piece that starts at tap (2 a, 2 b) is that of the first piece
+// a tile rows and b tiles further on.  V then holds one piece (row length Cp) over a tile grid
+// extended by the largest shifts (wc_conv_out_dims reports that grid), followed by `tail` rows that
+// only the products of the extension tiles read; the batched GEMM reads piece (a, b) of tile row p
+// at row p + a * grid_w + b.
+inline bool shared_input(const wc_conv_desc* d, const wc_plan* plan) { return d->stacked == 2 && plan->n_pieces > 1; }
+inline int v_row(const wc_conv_desc* d, const wc_plan* plan) {
+  return shared_input(d, plan) ? wc_padded_channels(d->C) : stacked_row(d, plan);
+}
+struct SharedShift { int n_run, n_runs, run_rows, tail; };   // pieces per tile row, piece rows, tiles per grid row
+inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
+  SharedShift s;
+  s.n_run = (d->kernel[2] + 1) / 2;
+  s.n_runs = (d->kernel[1] + 1) / 2;
+  s.run_rows = grid[2];
+  s.tail = (s.n_runs - 1) * s.run_rows + s.n_run - 1;
+  return s;
+}
+// M[t] (P x K, row stride ldm) = sum over pieces (a, b) of V[t][p + a run_rows + b][.] U[t][k][(a n_run + b) Cp + .];
+// V (T, P + tail, Cp), U (T, K, n_runs n_run Cp); 16-bit types (gemm.hip)
+int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
+                         int dtype, void* stream);
+
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;
 

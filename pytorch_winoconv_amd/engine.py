@@ -68,7 +68,9 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.dtype = _DTYPES[dtype]
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
-    d.stacked = int(bool(stacked))
+    d.stacked = 2 if stacked == 2 else int(bool(stacked))
+    if d.stacked == 2:
+        d.m = 2                      # the shared-input plan exists for output tile 2 only
     d.unfused = int(bool(unfused))
     return d
 
@@ -139,7 +141,12 @@ def input_transform(desc, plan, x_cl):
     _, grid = out_dims(desc)
     n = x_cl.shape[0]
     P = n * grid[0] * grid[1] * grid[2]
-    V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
+    if desc.stacked == 2 and plan.n_pieces > 1:
+        # one piece over the extended tile grid, plus the rows the shifted reads of the last tiles reach
+        tail = ((desc.kernel[1] + 1) // 2 - 1) * grid[2] + (desc.kernel[2] + 1) // 2 - 1
+        V = torch.zeros(plan.t_total, P + tail, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
+    else:
+        V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
     check(lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(x_cl), n, _ptr(V), _stream(x_cl)))
     return V
 
@@ -172,17 +179,24 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
     16-bit plans (2-D: 1.15-1.3x for 5x5 and 7x7 kernels; 3-D: 1.05-1.4x; fewer bytes moved); for
     fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
-    plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x)."""
+    plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit 2-D stride-1
+    kernels of 4 to 8 taps over at most 128 input channels get the plan whose two-tap pieces share
+    one transformed input (2; make_desc then uses output tile 2): 1.1x (5x5), 1.4x (4x4), 1.5x (7x7)
+    faster than stacked F(4,r) pieces at N=32, 128 channels, 112x112; with 256 channels or 9 taps the
+    larger product costs more than the smaller V saves."""
     if stacked is not None:
-        return bool(stacked)
+        return 2 if stacked == 2 else bool(stacked)
     if whole_kernel or (nd == 3 and m != 2):
-        return False
-    if dtype != torch.float32:
-        return True
-    if w_shape is None or nd != 2:
         return False
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
+    if dtype != torch.float32:
+        if (nd == 2 and stride == 1 and w_shape is not None and 4 <= max(w_shape[2:]) <= 8
+                and (int(w_shape[1]) + 31) // 32 * 32 <= 128):
+            return 2
+        return True
+    if w_shape is None or nd != 2:
+        return False
     n = 1
     for k in w_shape[2:]:
         taps = [(int(k) + 1 - q) // 2 for q in range(2)] if stride == 2 else [int(k)]
@@ -284,6 +298,8 @@ def conv_backward_weight(x, dy, w_shape, stride=1, padding=0, m=2, whole_kernel=
     works in the transform domain (see include/winoconv.h).  `stacked` as in conv_forward."""
     _require_gpu(x, dy)
     stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w_shape, stride, m)
+    if stacked == 2:
+        stacked = True               # the weight gradient has no shared-input form: pieces stacked with their own V
     if dy.dtype != x.dtype:
         raise TypeError("x and dy must share one dtype")
     lib = _lib.load()

@@ -1,0 +1,157 @@
+"""Plans whose pieces share one transformed input (`wc_conv_desc.stacked = 2`): the kernel is cut
+into pieces of two taps per axis on the tile F(2,2); a piece that starts at tap (2a, 2b) sees the
+transformed input of the first piece a tile rows and b tiles further on, so V holds one piece over
+an extended tile grid and the batched GEMM reads every piece's rows at that piece's tile offset.
+Nothing the reference does (it splits into pieces of three taps, each with its own transforms:
+src/base_conv_launchers.h:58-388); the sum over the pieces is the same convolution.
+
+Pinned by: U and every shifted view of V bit-equal to the CPU oracle's per-piece transforms;
+bit-exact integer convolution in fp16 on inputs whose every intermediate is an exactly
+representable integer; fp64 convolution (fp16, bf16 2e-2 of the output range) on random shapes."""
+import random
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import winograd as ow
+from pytorch_winoconv_amd import _lib, engine
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # x shape, w shape, pad
+    ((2, 32, 12, 12), (8, 32, 5, 5), 2),
+    ((1, 64, 20, 17), (40, 64, 7, 7), 3),
+    ((2, 16, 9, 14), (8, 16, 4, 6), (1, 2)),
+    ((2, 5, 13, 11), (6, 5, 5, 3), (2, 0)),
+    ((1, 40, 30, 30), (33, 40, 7, 7), 3),
+    ((2, 32, 10, 10), (8, 32, 3, 3), 1),         # 2 x 2 pieces of a 3 x 3 kernel
+    ((2, 24, 10, 10), (8, 24, 10, 9), 4),        # 25 pieces
+    ((2, 24, 10, 10), (8, 24, 2, 1), 0),         # one piece: an ordinary plan
+    ((3, 128, 28, 28), (128, 128, 5, 5), 2),
+]
+
+
+def _rel(a, r):
+    r = r.double()
+    return float((a.double().cpu() - r).abs().max() / r.abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES)
+def test_stages_against_the_oracle(dev, dtype, case):
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / (ws[1] * ws[2] * ws[3])) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    st = {}
+    y_oracle = ow.dwm_conv(x, w, b, 1, pad, 2, "fp16" if dtype == torch.float16 else "bf16", st, stacked=2)
+    desc = engine.make_desc(xs, ws, dtype, 1, pad, 2, stacked=2)
+    plan = engine.plan_conv(desc)
+    n_h, n_w = (ws[2] + 1) // 2, (ws[3] + 1) // 2
+    assert plan.n_pieces == n_h * n_w == len(st["plan"]["pieces"])
+    for i, pc in enumerate(st["plan"]["pieces"]):
+        assert list(plan.piece[i].tap0) == [a[0] for a in pc["axes"]] and plan.piece[i].t_offset == 0
+    C, N = xs[1], xs[0]
+    Cp = _lib.load().wc_padded_channels(C)
+    U = engine.filter_transform(desc, plan, w.to(dev))
+    assert U.shape == (plan.t_total, ws[0], plan.n_pieces * Cp)
+    for i in range(plan.n_pieces):
+        assert torch.equal(U[:, :, i * Cp:i * Cp + C].cpu(), st["U"][:, :, i * C:(i + 1) * C])
+    # the grid the library reports covers the tiles the pieces reach: (n_h - 1, n_w - 1) more than the output's
+    (_, oH, oW), (_, gH, gW) = engine.out_dims(desc)
+    nH, nW = (oH + 1) // 2, (oW + 1) // 2
+    assert (gH, gW) == (nH + n_h - 1, nW + n_w - 1)
+    V = engine.input_transform(desc, plan, engine.channel_last(x.to(dev)))
+    if plan.n_pieces > 1:
+        assert V.shape == (plan.t_total, N * gH * gW + (n_h - 1) * gW + n_w - 1, Cp)
+        Vg = V[:, :N * gH * gW, :C].cpu().reshape(plan.t_total, N, gH, gW, C)
+        for a in range(n_h):
+            for c in range(n_w):
+                i = a * n_w + c
+                want = st["V"][:, :, i * C:(i + 1) * C].reshape(plan.t_total, N, nH, nW, C)
+                assert torch.equal(Vg[:, :, a:a + nH, c:c + nW], want), (a, c)     # piece (a, b) = piece 0 moved by (a, b) tiles
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2, stacked=2)
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=pad)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert _rel(y, ref) <= 2e-2 and _rel(y, y_oracle) <= 1e-2
+    y1 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2, stacked=True)
+    assert _rel(y, y1.cpu()) <= 2e-2
+    # a cached filter, and chunked passes, change nothing
+    Uc = engine.transform_filter(w.to(dev), xs, 1, pad, 2, stacked=2)
+    for chunk in (0, 1):
+        assert torch.equal(engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2, U=Uc, chunk_images=chunk,
+                                               stacked=2), y)
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
+def test_exact_on_small_integers(dev, case):
+    """x in -3..3, taps multiples of 4 (G of F(2,2) halves): every U, V and product is an integer, and
+    with at most 64 channels the sums stay below 2048, exact in fp16 too; only the result is rounded."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = 4.0 * torch.randint(-1, 2, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    ref = F.conv2d(x, w, b, padding=pad)
+    y = engine.conv_forward(x.half().to(dev), w.half().to(dev), b.half().to(dev), 1, pad, 2, stacked=2)
+    assert float(ref.abs().max()) < 2048
+    assert torch.equal(y.cpu(), ref.half())
+
+
+def _random_cases(seed, n):
+    rng = random.Random(seed)
+    out = []
+    while len(out) < n:
+        ks = [rng.choice([2, 3, 4, 5, 7, rng.randint(1, 10)]) for _ in range(2)]
+        pad = [rng.randint(0, k - 1) for k in ks]
+        sp = [rng.randint(max(k - 2 * p, 1), 16) + rng.randint(0, 8) for k, p in zip(ks, pad)]
+        N, C, K = rng.randint(1, 3), rng.choice([1, 3, 8, 17, 32, 40, 65, 128]), rng.choice([1, 4, 6, 9, 32, 33, 72])
+        out.append((N, C, K, tuple(sp), tuple(ks), tuple(pad), rng.choice([torch.float16, torch.bfloat16])))
+    return out
+
+
+RANDOM = _random_cases(5, 40)
+
+
+@pytest.mark.parametrize("case", RANDOM, ids=[str(i) for i in range(len(RANDOM))])
+def test_random_shapes(dev, case):
+    N, C, K, sp, ks, pad, dtype = case
+    g = torch.Generator().manual_seed(N * 1000 + C)
+    x = torch.randn(N, C, *sp, generator=g).to(dtype)
+    w = (torch.randn(K, C, *ks, generator=g) * (2.0 / (C * ks[0] * ks[1])) ** 0.5).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), None, padding=pad)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, 1, pad, 2, stacked=2)
+    assert tuple(y.shape) == tuple(ref.shape) and _rel(y, ref) <= 2e-2
+
+
+def test_what_the_plan_is_not_built_for(dev):
+    x = torch.randn(2, 8, 12, 12).half().to(dev)
+    w = torch.randn(4, 8, 5, 5).half().to(dev)
+    with pytest.raises(NotImplementedError):
+        engine.conv_forward(x, w, None, 2, 2, 2, stacked=2)                        # stride 2
+    with pytest.raises(NotImplementedError):
+        engine.conv_forward(x.float(), w.float(), None, 1, 2, 2, stacked=2)        # fp32 product
+    x3, w3 = torch.randn(1, 8, 6, 12, 12).half().to(dev), torch.randn(4, 8, 3, 5, 5).half().to(dev)
+    with pytest.raises(NotImplementedError):
+        engine.conv_forward(x3, w3, None, 1, 1, 2, stacked=2)                      # 3-D
+    # the weight gradient falls back to stacked pieces with their own V; the default picks this plan for the forward pass
+    dy = torch.randn(2, 4, 12, 12).half().to(dev)
+    dw = engine.conv_backward_weight(x, dy, w.shape, 1, 2, 2, stacked=2)
+    assert torch.equal(dw, engine.conv_backward_weight(x, dy, w.shape, 1, 2, 2, stacked=True))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
+
+
+def test_c4_layer_at_full_size(dev):
+    """N=32, C=K=128, 112x112, 7x7: against the stacked F(2,r) plan (own V per piece) and a sample of fp64."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(32, 128, 112, 112, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    w = (torch.randn(128, 128, 7, 7, generator=g) * (2.0 / (128 * 49)) ** 0.5).half().to(dev)
+    y = engine.conv_forward(x, w, None, 1, 3, 2, stacked=2)
+    y1 = engine.conv_forward(x, w, None, 1, 3, 2, stacked=True)
+    scale = float(y1.float().abs().max())
+    assert float((y.float() - y1.float()).abs().max()) <= 4e-3 * scale
+    sample = F.conv2d(x[:1].double().cpu(), w.double().cpu(), padding=3)
+    assert _rel(y[:1], sample) <= 2e-3

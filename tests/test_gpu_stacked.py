@@ -88,9 +88,11 @@ def test_cached_filter_chunks_and_size_check(dev):
     U = engine.transform_filter(w, xs, 1, 2, 4, stacked=True)
     for chunk in (0, 1, 2):
         assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4, U=U, chunk_images=chunk, stacked=True), y)
-    # the default for 16-bit 2-D plans is the stacked form
-    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), y)
-    assert torch.equal(engine.transform_filter(w, xs, 1, 2, 4), U)
+    # the default for 16-bit plans is a stacked form: at stride 2 this one, at stride 1 with 4..8 taps and
+    # at most 128 channels the one whose pieces share the transformed input (test_gpu_shared.py)
+    assert torch.equal(engine.conv_forward(x, w, None, 2, 2, 4), engine.conv_forward(x, w, None, 2, 2, 4, stacked=True))
+    assert torch.equal(engine.transform_filter(w, xs, 2, 2, 4), engine.transform_filter(w, xs, 2, 2, 4, stacked=True))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
     # a filter transformed for the other form has another size and is refused, not misread
     with pytest.raises(ValueError):
         engine.conv_forward(x, w, None, 1, 2, 4, U=U, stacked=False)
