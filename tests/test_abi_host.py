@@ -226,6 +226,50 @@ def test_modules_pick_tile_2_where_tile_4_loses_accuracy():
     assert pkg.WinoConv3d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
 
 
+def test_shared_input_plans():
+    """stacked = 2: pieces of two taps on the tile F(2,2), one transformed input for all of them over a
+    tile grid extended by the pieces' reach; 2-D, stride 1, output tile 2."""
+    lib = _lib.load()
+    d = engine.make_desc((2, 8, 20, 21), (4, 8, 7, 5), torch.float16, 1, (3, 2), 4, stacked=2)
+    assert d.stacked == 2 and d.m == 2                    # the Python layer forces tile 2 for this plan
+    plan = engine.plan_conv(d)
+    assert plan.n_pieces == 4 * 3 and plan.t_total == 9 and list(plan.m) == [1, 2, 2]
+    want = [((0, 2 * a, 2 * b), (1, 2 if 2 * a + 2 <= 7 else 1, 2 if 2 * b + 2 <= 5 else 1)) for a in range(4) for b in range(3)]
+    for i, (tap0, r) in enumerate(want):
+        assert tuple(plan.piece[i].tap0) == tap0 and tuple(plan.piece[i].r) == r and plan.piece[i].t_offset == 0
+    from oracle import split_plan as osp2
+    pieces, T = osp2.conv_pieces([1, 7, 5], 1, 2, degenerate_depth=True, pairs=True)
+    assert [tuple(a[0] for a in pc["axes"]) for pc in pieces] == [t for t, _ in want]
+    out, grid = engine.out_dims(d)
+    assert out == [1, 20, 21] and grid == [1, 10 + 3, 11 + 2]
+    # workspace: U (9, K, 12 Cp) + V (9, P + tail, Cp) + M (9, P, 8), each rounded to 256 bytes
+    nbytes = ctypes.c_size_t()
+    assert lib.wc_conv_workspace_bytes(ctypes.byref(d), ctypes.byref(nbytes)) == 0
+    P, tail = 2 * 13 * 13, 3 * 13 + 2
+    r256 = lambda v: (v + 255) // 256 * 256
+    assert nbytes.value == r256(2 * 9 * 4 * 12 * 32) + r256(2 * 9 * (P + tail) * 32) + r256(2 * 9 * P * 8)
+    # one piece per axis: nothing is extended
+    d1 = engine.make_desc((2, 8, 20, 21), (4, 8, 2, 1), torch.float16, 1, 0, 2, stacked=2)
+    assert engine.plan_conv(d1).n_pieces == 1 and engine.out_dims(d1)[1] == [1, 10, 11]
+    for kw in (dict(stride=2), dict(x=(1, 8, 9, 20, 20), w=(4, 8, 3, 5, 5))):
+        bad = engine.make_desc(kw.get("x", (2, 8, 20, 21)), kw.get("w", (4, 8, 5, 5)), torch.float16, kw.get("stride", 1), 2, 2,
+                               stacked=2)
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(bad)
+    bad = engine.make_desc((2, 8, 20, 21), (4, 8, 5, 5), torch.float16, 1, 2, 2, stacked=2)
+    bad.m = 4
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(bad)
+    # what the Python layer picks when nothing is said
+    s = engine._stack
+    assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 1, 4) == 2 and s(None, torch.bfloat16, 2, False, (8, 100, 4, 8), 1, 2) == 2
+    assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 2, 4) is True        # stride 2
+    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 4) is True        # more than 128 channels
+    assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) is True and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
+    assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) is True
+    assert s(2, torch.float32, 2, False) == 2 and s(True, torch.float16, 2, False) is True and s(False, torch.float16, 2, False) is False
+
+
 def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
     """The cached U of a module must be the F(2,3) one wherever wc_conv_forward runs its fused kernel."""
     import pytorch_winoconv_amd as pkg
