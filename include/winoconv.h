@@ -83,11 +83,11 @@ typedef struct {
                     *    GEMM adds them: M shrinks to one piece's size.  Same sum, other rounding.
                     *    Output tile 2, or 4 in 2-D.  The plan then reports t_offset = 0 for every piece and
                     *    t_total = prod(m + r_max - 1).
-                    * 2: (2-D, stride 1, m = 2; wc_conv_forward and the stages, fp16 / bf16 products) the kernel is cut
+                    * 2: (stride 1, m = 2; wc_conv_forward and the stages, fp16 / bf16 products) the kernel is cut
                     *    into pieces of two taps per axis (the last one of an odd extent has one), all on the tile
                     *    F(2,2).  Pieces that start at even taps see the same transformed input, moved by whole
                     *    tiles: V holds ONE piece, over a tile grid extended by the largest moves (wc_conv_out_dims
-                    *    reports that grid) plus (kH+1)/2-1 grid rows and (kW+1)/2-1 tiles of slack, U holds the
+                    *    reports that grid) plus the rows that the moved reads of its last tiles reach, U holds the
                     *    pieces side by side as for 1, and the batched GEMM reads each piece's rows of V at that
                     *    piece's tile offset.  Same sum as 0 and 1; V is written and read once instead of once
                     *    per piece. */

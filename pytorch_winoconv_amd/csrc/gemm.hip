@@ -66,8 +66,10 @@ struct GemmArgs {
   int n_blocks, per_xcd;
   // shifted operand (plans whose pieces share one transformed input): rows of V are ldv apart, and
   // after every run_blocks reduction blocks the V operand jumps on by `jump` elements
-  int ldv, run_blocks;
-  long long jump;
+  // (one run = the pieces along the width: consecutive rows of V), and after every plane_runs runs
+  // by jump2 more (3-D plans: on to the next depth plane of the tile grid)
+  int ldv, run_blocks, plane_runs;
+  long long jump, jump2;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -158,14 +160,18 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
 
   const int nk = g.Cp / BK;
   long long vshift = 0;
-  int run_left = SHIFT ? g.run_blocks : 0;
+  int run_left = SHIFT ? g.run_blocks : 0, plane_left = SHIFT ? g.plane_runs : 0;
   gload(0, 0);
   lstore(0);
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     if constexpr (SHIFT) {
-      if (--run_left == 0) { vshift += g.jump; run_left = g.run_blocks; }
+      if (--run_left == 0) {
+        vshift += g.jump;
+        run_left = g.run_blocks;
+        if (--plane_left == 0) { vshift += g.jump2; plane_left = g.plane_runs; }
+      }
     }
     if (kt + 1 < nk) gload(kt + 1, vshift);
     const T* st = lds + cur * STAGE;
@@ -351,7 +357,9 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
                          int dtype, void* stream) {
   WC_CHECK_ARG(V && U && M, "batched_gemm_shifted: null pointer");
   WC_CHECK_ARG(T_ > 0 && P > 0 && K > 0 && Cp > 0 && Cp % 32 == 0, "batched_gemm_shifted: T %d, P %d, K %d, Cp %d", T_, P, K, Cp);
-  WC_CHECK_ARG(sh.n_run > 0 && sh.n_runs > 0 && sh.run_rows >= sh.n_run && sh.tail == (sh.n_runs - 1) * sh.run_rows + sh.n_run - 1,
+  WC_CHECK_ARG(sh.n_run > 0 && sh.n_runs > 0 && sh.n_planes > 0 && sh.run_rows >= sh.n_run &&
+                   sh.plane_rows >= sh.n_runs * sh.run_rows &&
+                   sh.tail == (sh.n_planes - 1) * sh.plane_rows + (sh.n_runs - 1) * sh.run_rows + sh.n_run - 1,
                "batched_gemm_shifted: bad shift description");
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "batched_gemm_shifted: row stride %d", ldm);
   if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_shifted: 16-bit types only");
@@ -359,10 +367,12 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   GemmArgs g;
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.ldm = ldm;
-  g.Cp = sh.n_runs * sh.n_run * Cp;                      // reduction length = row length of U
+  g.Cp = sh.n_planes * sh.n_runs * sh.n_run * Cp;        // reduction length = row length of U
   g.ldv = Cp;
   g.run_blocks = sh.n_run * Cp / c.bk;                   // one run: the pieces of one piece row, contiguous rows of V
   g.jump = (long long)(sh.run_rows - sh.n_run) * Cp;     // on to the same tile one grid row further
+  g.plane_runs = sh.n_runs;
+  g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
@@ -393,7 +403,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;
   g.sV = (long long)P * Cp; g.sU = (long long)K * Cp; g.sM = (long long)P * ldm;
-  g.ldv = Cp; g.run_blocks = 0; g.jump = 0;
+  g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

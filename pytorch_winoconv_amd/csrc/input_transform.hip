@@ -46,10 +46,17 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
 
   if (shared) {
     // the first piece with the tile all pieces share, over the extended tile grid
-    WC_CHECK_ARG(flat && plan->m[1] == 2 && plan->m[2] == 2, "wc_input_transform: shared input needs a 2-D plan with output tile 2");
-    InKernel fn = pick_in_2d(d->dtype, kind_of(2, rp[1]), kind_of(2, rp[2]), vec);
-    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform F(2,%d) x F(2,%d) not built", rp[1], rp[2]);
-    a.base0 = 0; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
+    WC_CHECK_ARG(plan->m[1] == 2 && plan->m[2] == 2, "wc_input_transform: shared input needs output tile 2");
+    const int k0 = kind_of(plan->m[0], rp[0]), k1 = kind_of(2, rp[1]), k2 = kind_of(2, rp[2]);
+    InKernel fn = nullptr;
+    switch (k0) {
+      case KIND_11: fn = pick_in_2d(d->dtype, k1, k2, vec); break;
+      case KIND_21: fn = pick_in_3d_21(d->dtype, k1, k2, vec); break;
+      case KIND_22: fn = pick_in_3d_22(d->dtype, k1, k2, vec); break;
+      default: break;
+    }
+    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform F(2,%d) x F(2,%d) x F(2,%d) not built", rp[0], rp[1], rp[2]);
+    a.base0 = -d->pad[0]; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
     a.t_offset = 0;
     hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("input_transform_kernel");

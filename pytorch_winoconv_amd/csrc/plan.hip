@@ -136,8 +136,8 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
     return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
-  if (d->stacked == 2 && (d->ndim != 2 || d->stride != 1 || d->m != 2))
-    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need a 2-D problem, stride 1 and output tile 2");
+  if (d->stacked == 2 && (d->stride != 1 || d->m != 2))
+    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need stride 1 and output tile 2");
   if (d->whole_kernel) {
     if (d->ndim != 2 || d->stride != 1 || d->m != 2)
       return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");

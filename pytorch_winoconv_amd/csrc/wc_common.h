@@ -77,22 +77,28 @@ inline int stacked_row(const wc_conv_desc* d, const wc_plan* plan) {
 // a tile rows and b tiles further on.  V then holds one piece (row length Cp) over a tile grid
 // extended by the largest shifts (wc_conv_out_dims reports that grid), followed by `tail` rows that
 // only the products of the extension tiles read; the batched GEMM reads piece (a, b) of tile row p
-// at row p + a * grid_w + b.
+// at row p + a * grid_w + b (3-D: the depth axis likewise, whole planes of the grid further on).
 inline bool shared_input(const wc_conv_desc* d, const wc_plan* plan) { return d->stacked == 2 && plan->n_pieces > 1; }
 inline int v_row(const wc_conv_desc* d, const wc_plan* plan) {
   return shared_input(d, plan) ? wc_padded_channels(d->C) : stacked_row(d, plan);
 }
-struct SharedShift { int n_run, n_runs, run_rows, tail; };   // pieces per tile row, piece rows, tiles per grid row
+struct SharedShift {          // pieces (a, b, c) of the depth, height and width axes; tiles (d, h, w) of the extended grid
+  int n_run, n_runs, n_planes;  // pieces per axis: width, height, depth
+  int run_rows, plane_rows;     // tile rows of V between two tiles that are neighbours in height / in depth
+  int tail;                     // rows beyond the grid that the shifted reads of its last tiles reach
+};
 inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
   SharedShift s;
   s.n_run = (d->kernel[2] + 1) / 2;
   s.n_runs = (d->kernel[1] + 1) / 2;
+  s.n_planes = (d->kernel[0] + 1) / 2;
   s.run_rows = grid[2];
-  s.tail = (s.n_runs - 1) * s.run_rows + s.n_run - 1;
+  s.plane_rows = grid[1] * grid[2];
+  s.tail = (s.n_planes - 1) * s.plane_rows + (s.n_runs - 1) * s.run_rows + s.n_run - 1;
   return s;
 }
-// M[t] (P x K, row stride ldm) = sum over pieces (a, b) of V[t][p + a run_rows + b][.] U[t][k][(a n_run + b) Cp + .];
-// V (T, P + tail, Cp), U (T, K, n_runs n_run Cp); 16-bit types (gemm.hip)
+// M[t] (P x K, row stride ldm) = sum over pieces (a, b, c) of V[t][p + a plane_rows + b run_rows + c][.] x
+// U[t][k][((a n_runs + b) n_run + c) Cp + .]; V (T, P + tail, Cp), U (T, K, n_pieces Cp); 16-bit types (gemm.hip)
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream);
 

@@ -143,7 +143,8 @@ def input_transform(desc, plan, x_cl):
     P = n * grid[0] * grid[1] * grid[2]
     if desc.stacked == 2 and plan.n_pieces > 1:
         # one piece over the extended tile grid, plus the rows the shifted reads of the last tiles reach
-        tail = ((desc.kernel[1] + 1) // 2 - 1) * grid[2] + (desc.kernel[2] + 1) // 2 - 1
+        tail = (((desc.kernel[0] + 1) // 2 - 1) * grid[1] * grid[2] + ((desc.kernel[1] + 1) // 2 - 1) * grid[2]
+                + (desc.kernel[2] + 1) // 2 - 1)
         V = torch.zeros(plan.t_total, P + tail, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
     else:
         V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
@@ -179,11 +180,12 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
     16-bit plans (2-D: 1.15-1.3x for 5x5 and 7x7 kernels; 3-D: 1.05-1.4x; fewer bytes moved); for
     fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
-    plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit 2-D stride-1
+    plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit stride-1
     kernels of 4 to 8 taps over at most 128 input channels get the plan whose two-tap pieces share
     one transformed input (2; make_desc then uses output tile 2): 1.1x (5x5), 1.4x (4x4), 1.5x (7x7)
-    faster than stacked F(4,r) pieces at N=32, 128 channels, 112x112; with 256 channels or 9 taps the
-    larger product costs more than the smaller V saves."""
+    faster than stacked F(4,r) pieces at N=32, 128 channels, 112x112, and 1.5x (5x5x5) to 2x (4x4x4,
+    7x7x7) faster than stacked F(2,r) pieces in 3-D; with 256 channels or 9 taps the larger product
+    costs more than the smaller V saves."""
     if stacked is not None:
         return 2 if stacked == 2 else bool(stacked)
     if whole_kernel or (nd == 3 and m != 2):
@@ -191,7 +193,7 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
     if dtype != torch.float32:
-        if (nd == 2 and stride == 1 and w_shape is not None and 4 <= max(w_shape[2:]) <= 8
+        if (stride == 1 and w_shape is not None and 4 <= max(w_shape[2:]) <= 8
                 and (int(w_shape[1]) + 31) // 32 * 32 <= 128):
             return 2
         return True

@@ -251,11 +251,15 @@ def test_shared_input_plans():
     # one piece per axis: nothing is extended
     d1 = engine.make_desc((2, 8, 20, 21), (4, 8, 2, 1), torch.float16, 1, 0, 2, stacked=2)
     assert engine.plan_conv(d1).n_pieces == 1 and engine.out_dims(d1)[1] == [1, 10, 11]
-    for kw in (dict(stride=2), dict(x=(1, 8, 9, 20, 20), w=(4, 8, 3, 5, 5))):
-        bad = engine.make_desc(kw.get("x", (2, 8, 20, 21)), kw.get("w", (4, 8, 5, 5)), torch.float16, kw.get("stride", 1), 2, 2,
-                               stacked=2)
-        with pytest.raises(NotImplementedError):
-            engine.plan_conv(bad)
+    bad = engine.make_desc((2, 8, 20, 21), (4, 8, 5, 5), torch.float16, 2, 2, 2, stacked=2)      # stride 2
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(bad)
+    # 3-D: pieces depth-major, the grid extended on all three axes
+    d3 = engine.make_desc((1, 8, 9, 20, 20), (4, 8, 3, 5, 4), torch.float16, 1, (1, 2, 1), 2, stacked=2)
+    p3 = engine.plan_conv(d3)
+    assert p3.n_pieces == 2 * 3 * 2 and p3.t_total == 27 and list(p3.m) == [2, 2, 2]
+    assert tuple(p3.piece[7].tap0) == (2, 0, 2) and tuple(p3.piece[7].r) == (1, 2, 2)
+    assert engine.out_dims(d3) == ([9, 20, 19], [5 + 1, 10 + 2, 10 + 1])
     bad = engine.make_desc((2, 8, 20, 21), (4, 8, 5, 5), torch.float16, 1, 2, 2, stacked=2)
     bad.m = 4
     with pytest.raises(NotImplementedError):
@@ -266,7 +270,8 @@ def test_shared_input_plans():
     assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 2, 4) is True        # stride 2
     assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 4) is True        # more than 128 channels
     assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) is True and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
-    assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) is True
+    assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) == 2
+    assert s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 2) is True and s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 4) is False
     assert s(2, torch.float32, 2, False) == 2 and s(True, torch.float16, 2, False) is True and s(False, torch.float16, 2, False) is False
 
 
