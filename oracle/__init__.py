@@ -33,7 +33,9 @@ in tests/test_oracle_*.py):
                        the reference kernels' unrolled spot formulas.  The stacked
                        form of dwm_conv (pieces added by the batched product, which
                        the reference does not do) is pinned by the same fp64
-                       convolution and integer-exact checks.
+                       convolution and integer-exact checks; so is the form with
+                       pieces of two taps (split_plan.axis_pairs, dwm_conv(stacked=2)),
+                       a split the reference does not use either.
   Tables F(2,8..11) of the reference (matrix_conv.py:36-39) are not restated:
   nothing here uses them.
 """

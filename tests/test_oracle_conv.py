@@ -131,3 +131,35 @@ def test_stacked_pieces_give_the_same_convolution(case):
         wi = (torch.randint(-2, 3, ws, generator=g) * 4).float()
         yi = ow.dwm_conv(xi, wi, None, s, p, m, "fp32", stacked=True)
         assert torch.equal(yi.double(), _conv(xi.double(), wi.double(), None, s, p))
+
+
+@pytest.mark.parametrize("case", [
+    ((2, 3, 9, 10), (4, 3, 5, 5), 2), ((1, 2, 12, 11), (3, 2, 7, 4), (3, 1)), ((1, 3, 9, 9), (2, 3, 3, 3), 1),
+    ((1, 2, 8, 9), (2, 2, 10, 2), (4, 0)), ((1, 2, 6, 8, 7), (3, 2, 3, 5, 4), (1, 2, 1)), ((2, 2, 5, 6, 6), (2, 2, 1, 5, 5), (0, 2, 2)),
+])
+def test_pair_pieces_give_the_same_convolution(case):
+    """The split into pieces of two taps (not the reference's rule of three): pieces start at even
+    taps 0, 2, 4, ..., together they own every tap once, the stacked sum over them is the convolution
+    in fp64, and exactly so on small integers in fp32 (G of F(2,2) only halves)."""
+    from oracle import split_plan as sp
+    xs, ws, p = case
+    for k in range(1, 11):
+        pieces = sp.axis_pairs(k)
+        assert [t for t, _, _ in pieces] == list(range(0, k, 2))
+        assert sorted(t + j for t, _, n in pieces for j in range(n)) == list(range(k))
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(*xs, dtype=torch.float64, generator=g)
+    w = torch.randn(*ws, dtype=torch.float64, generator=g)
+    b = torch.randn(ws[0], dtype=torch.float64, generator=g)
+    st = {}
+    y = ow.dwm_conv(x, w, b, 1, p, 2, "fp64", st, stacked=2)
+    ref = _conv(x, w, b, 1, p)
+    assert y.shape == ref.shape and float((y - ref).abs().max() / ref.abs().max()) < 1e-12
+    n = 1
+    for k in ws[2:]:
+        n *= (k + 1) // 2
+    assert len(st["plan"]["pieces"]) == n and st["U"].shape[2] == n * xs[1]
+    xi = torch.randint(-3, 4, xs, generator=g).float()
+    wi = (torch.randint(-2, 3, ws, generator=g) * 8).float()
+    yi = ow.dwm_conv(xi, wi, None, 1, p, 2, "fp32", stacked=2)
+    assert torch.equal(yi.double(), _conv(xi.double(), wi.double(), None, 1, p))
