@@ -98,6 +98,8 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)xF(4,3)^2", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, "f16"),
+    ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 shared input F(2,2)^3", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16"),
+    ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 F(2,r)^3 stacked", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16-stacked"),
     ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
 ]
 VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),

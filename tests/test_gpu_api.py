@@ -192,19 +192,25 @@ def test_winoconv3d_module(dev):
     assert _nerr(mod(x), ref) < 1e-3
 
 
-def test_forward_is_capturable_in_a_hip_graph(dev):
+@pytest.mark.parametrize("ws,m,stacked", [
+    ((48, 32, 5, 5), 4, 0),        # DWM pieces, four kernels
+    ((48, 32, 5, 5), 2, 2),        # two-tap pieces sharing one transformed input (shifted GEMM operand)
+    ((48, 32, 3, 3), 2, 0),        # thin 16-bit 3x3 layer: filter transform + the one fused kernel
+])
+def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked):
     """The library allocates nothing, never synchronises and takes its stream from the caller, so a
-    whole forward pass (four kernels) can be captured once and replayed.  The graph is replayed
-    three times with new input contents, eager work and synchronisation between the replays, and
-    every replay must equal the eager result bit for bit."""
+    whole forward pass can be captured once and replayed.  The graph is replayed three times with new
+    input contents, eager work and synchronisation between the replays, and every replay must equal
+    the eager result bit for bit."""
     import ctypes
     from pytorch_winoconv_amd import _lib
     lib = _lib.load()
-    xs, ws = (2, 32, 20, 20), (48, 32, 5, 5)
+    xs = (2, 32, 20, 20)
+    pad = ws[2] // 2
     g = torch.Generator().manual_seed(11)
     x = torch.randn(*xs, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
     w = (torch.randn(*ws, generator=g) * 0.05).half().to(dev)
-    desc = pkg.engine.make_desc(xs, ws, torch.float16, 1, 2, 4)
+    desc = pkg.engine.make_desc(xs, ws, torch.float16, 1, pad, m, stacked=stacked)
     nbytes = ctypes.c_size_t()
     _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
     wsp = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
@@ -231,5 +237,5 @@ def test_forward_is_capturable_in_a_hip_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         got = y.clone()
-        want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, 2, 4, stacked=False)     # eager, own buffers
+        want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, pad, m, stacked=stacked)   # eager, own buffers
         assert torch.equal(got.permute(0, 3, 1, 2), want), i
