@@ -91,10 +91,11 @@ typedef struct {
                     *    pieces side by side as for 1, and the batched GEMM reads each piece's rows of V at that
                     *    piece's tile offset.  Same sum as 0 and 1; V is written and read once instead of once
                     *    per piece. */
-  int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2, at most 64 input
-                    *    channels (an even number up to 32, a multiple of 4 above) and at most 512 output
-                    *    channels run as one kernel: input transform, products and output transform of
-                    *    F(2x2, 3x3) without V and M in memory, the product kept in fp32 (x below 1 GiB);
+  int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2 whose input channels
+                    *    pad to 32, 64 or 128 (an even number up to 32, a multiple of 4 in 33..64 or 97..128)
+                    *    and that have at most 512 output channels (256 with 128 input channels) run as one
+                    *    kernel: input transform, products and output transform of F(2x2, 3x3) without V and
+                    *    M in memory, the product kept in fp32 (x below 1 GiB);
                     * 1: always filter transform -> input transform -> batched GEMM -> output transform. */
 } wc_conv_desc;
 

@@ -1,4 +1,4 @@
-// One-kernel F(2x2, 3x3) convolution for thin 16-bit layers (at most 64 input channels).
+// One-kernel F(2x2, 3x3) convolution for thin 16-bit layers (at most 128 input channels).
 //
 // Same arithmetic as the three-kernel path (input transform of src/split_kernel.cu:60-120, the
 // batched product of src/base_conv_launchers.cu:353-367, output transform of
@@ -89,8 +89,15 @@ static_assert(Mats<KIND_23>::bt(0, 0) == 1 && Mats<KIND_23>::bt(0, 2) == -1 && M
               Mats<KIND_23>::bt(3, 1) == 1 && Mats<KIND_23>::bt(3, 3) == -1, "B^T of F(2,3)");
 
 template <typename T, int CP>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
-  constexpr int VEC = CP / 16;            // channels per thread in the transform
+__global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
+  // Up to 64 channels a wavefront holds U of all 16 elements (4 wavefronts).  With 128 that is twice
+  // the register file, so SPLIT: 8 wavefronts, the upper four take the element rows 2 and 3 and hand
+  // their share of the output tile to the lower four through LDS.
+  constexpr bool SPLIT = CP > 64;
+  constexpr int NT = SPLIT ? 512 : 256;
+  constexpr int NROW = SPLIT ? 2 : 4;     // element rows per wavefront
+  constexpr int VEC = kThinTiles * CP / NT;   // channels per thread in the transform
+  constexpr int CVECS = CP / VEC;
   constexpr int KS = CP / 32;             // MFMA steps along the channels
   constexpr int PITCH = CP * 2 + 16;      // bytes per (element, tile) row in LDS; the pad spreads 16 rows over all banks
   constexpr int BUF = 16 * kThinTiles * PITCH;
@@ -99,13 +106,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int kbase = blockIdx.y * kThinK + wave * 16;
+  const int kbase = blockIdx.y * kThinK + (wave & 3) * 16;
+  const int row0i = SPLIT ? 2 * (wave >> 2) : 0;       // first element row of this wavefront
 
   // transform role: tile pl of the block, channels c .. c + VEC.  x is read through a buffer descriptor:
   // one 32-bit offset per load, and a window element outside the image is an offset beyond the
   // buffer, which reads as zero.
-  const int pl = tid >> 4;
-  const int c = (tid & 15) * VEC;
+  const int pl = tid / CVECS;
+  const int c = (tid % CVECS) * VEC;
   const bool c_ok = c < a.C;
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.x), 0, a.x_bytes, 0x00020000);
@@ -144,11 +152,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // this wavefront's part of U: row operand, lane = output channel kbase + lane % 16, 8 channels
   // from 8 * (lane / 16).  Rows beyond K repeat row K - 1: a row of U only reaches the same row of the
   // product, and those rows are never stored.
-  Frag u[16][KS];
+  Frag u[NROW * 4][KS];
   {
     const int ko = kbase + (lane & 15);
-    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + 8 * (lane >> 4);
-    static_for<0, 16>([&](auto t_) {
+    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + 8 * (lane >> 4) +
+                 (long long)row0i * 4 * a.K * CP;
+    static_for<0, NROW * 4>([&](auto t_) {
       constexpr int t = decltype(t_)::value;
       static_for<0, KS>([&](auto s_) {
         constexpr int s = decltype(s_)::value;
@@ -195,24 +204,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // Width half of the output transform in the accumulators, M[i][j] = U[i][j] V[i][j] over the channels:
     // z0[i] = M[i][0] + M[i][1] + M[i][2], and M[i][1] - (M[i][2] + M[i][3]) as zp[i] - zn[i] (no operand
     // needs its sign changed).  Consecutive MFMAs write different accumulators.
-    floatx4 z0[4], zp[4], zn[4];
+    floatx4 z0[NROW], zp[NROW], zn[NROW];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-    const unsigned char* vrow = buf + (lane & 15) * PITCH + 16 * (lane >> 4);
+    for (int i = 0; i < NROW; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const unsigned char* vrow = buf + (lane & 15) * PITCH + 16 * (lane >> 4) + row0i * 4 * kThinTiles * PITCH;
     static_for<0, KS>([&](auto s_) {
       constexpr int s = decltype(s_)::value;
       static_for<0, 4>([&](auto j_) {
         constexpr int j = decltype(j_)::value;
-        Frag v[4];
-        static_for<0, 4>([&](auto i_) {
+        Frag v[NROW];
+        static_for<0, NROW>([&](auto i_) {
           constexpr int i = decltype(i_)::value;
           v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + s * 64);
         });
-        static_for<0, 4>([&](auto i_) {
+        static_for<0, NROW>([&](auto i_) {
           constexpr int i = decltype(i_)::value;
           if constexpr (j <= 2) z0[i] = MF::run(u[i * 4 + j][s], v[i], z0[i]);
         });
-        static_for<0, 4>([&](auto i_) {
+        static_for<0, NROW>([&](auto i_) {
           constexpr int i = decltype(i_)::value;
           if constexpr (j == 1) zp[i] = MF::run(u[i * 4 + j][s], v[i], zp[i]);
           if constexpr (j >= 2) zn[i] = MF::run(u[i * 4 + j][s], v[i], zn[i]);
@@ -220,12 +229,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       });
     });
 
+    // Height half of the output transform: out[0][b] = z[0][b] + z[1][b] + z[2][b], out[1][b] = z[1][b] -
+    // z[2][b] - z[3][b] with z[i][0] = z0[i], z[i][1] = zp[i] - zn[i].
+    floatx4 out[2][2];
+    if constexpr (!SPLIT) {
+#pragma unroll
+      for (int ob = 0; ob < 2; ++ob) {
+        floatx4 z[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) z[i] = ob == 0 ? z0[i] : zp[i] - zn[i];
+        out[0][ob] = z[0] + z[1] + z[2];
+        out[1][ob] = z[1] - z[2] - z[3];
+      }
+    } else {
+      // the upper wavefronts (rows 2, 3) pass their share through LDS to the lower ones (rows 0, 1)
+      floatx4* xch = reinterpret_cast<floatx4*>(lds + 2 * BUF) + ((wave & 3) * 4) * 64 + lane;
+      const bool upper = wave >= 4;
+#pragma unroll
+      for (int ob = 0; ob < 2; ++ob) {
+        const floatx4 za = ob == 0 ? z0[0] : zp[0] - zn[0], zb = ob == 0 ? z0[1] : zp[1] - zn[1];
+        out[0][ob] = upper ? za : za + zb;
+        out[1][ob] = upper ? -za - zb : zb;
+      }
+      if (upper) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xch[q * 64] = out[q >> 1][q & 1];
+      }
+      __syncthreads();
+      if (!upper) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) out[q >> 1][q & 1] += xch[q * 64];
+      }
+    }
+
     // height half of the output transform, bias, store: lane = tile lane % 16, output channels
     // ko .. ko + 4.  Stores go through a buffer descriptor: an output position outside (oH, oW) gets
     // an offset beyond the buffer and is dropped.
     const int p = blk * kThinTiles + (lane & 15);
     const int ko = kbase + 4 * (lane >> 4);
-    if (p < a.P && ko < a.K) {
+    if (p < a.P && ko < a.K && (!SPLIT || wave < 4)) {
       const int q = fast_div(p, a.div_nW);
       const int tw = p - q * a.nW;
       const int b = fast_div(q, a.div_nH);
@@ -237,18 +279,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int r = 0; r < 4; ++r)
           if (ko + r < a.K) bv[r] = static_cast<float>(bias[ko + r]);
       }
-      floatx4 zw[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) zw[i] = zp[i] - zn[i];
       const unsigned o00 = (((unsigned)b * a.oH + 2 * th) * a.oW + 2 * tw) * a.K + ko;   // in elements
       const bool h1 = 2 * th + 1 < a.oH, w1 = 2 * tw + 1 < a.oW;
 #pragma unroll
       for (int oa = 0; oa < 2; ++oa) {
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob) {
-          floatx4 s4;
-          if (ob == 0) s4 = oa == 0 ? z0[0] + z0[1] + z0[2] : z0[1] - z0[2] - z0[3];
-          else s4 = oa == 0 ? zw[0] + zw[1] + zw[2] : zw[1] - zw[2] - zw[3];
+          const floatx4 s4 = out[oa][ob];
           const bool inside = (oa == 0 || h1) && (ob == 0 || w1);
           const unsigned off = o00 + (oa * a.oW + ob) * a.K;
           Pack<T, 4> o;
@@ -272,15 +309,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <typename T, int CP>
 int launch_thin(ThinArgs a, int k_groups, void* stream) {
-  constexpr int lds = 2 * 16 * kThinTiles * (CP * 2 + 16);
-  // two workgroups per CU stay resident (registers and LDS): 512 in all, shared among the groups
-  // of output channels, in whole multiples of the 8 XCDs
-  int wgs = std::min(a.n_blocks, std::max(kXcds, 512 / k_groups / kXcds * kXcds));
+  constexpr bool split = CP > 64;
+  constexpr int lds = 2 * 16 * kThinTiles * (CP * 2 + 16) + (split ? 4 * 4 * 64 * 16 : 0);
+  // workgroups that stay resident (registers and LDS): two per CU, one of the eight-wavefront form;
+  // shared among the groups of output channels, in whole multiples of the 8 XCDs
+  int wgs = std::min(a.n_blocks, std::max(kXcds, (split ? 256 : 512) / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
   WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-  hipLaunchKernelGGL((thin_conv3x3_kernel<T, CP>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256),
-                     lds, as_stream(stream), a);
+  hipLaunchKernelGGL((thin_conv3x3_kernel<T, CP>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups),
+                     dim3(split ? 512 : 256), lds, as_stream(stream), a);
   WC_CHECK_LAUNCH("thin_conv3x3_kernel");
   return WC_OK;
 }
@@ -293,12 +331,12 @@ bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan) {
   const wc_piece& pc = plan->piece[0];
   if (pc.r[0] != 1 || pc.r[1] != 3 || pc.r[2] != 3) return false;
   const int Cp = wc_padded_channels(d->C);
-  if (Cp > 64 || d->C % (Cp / 16) != 0) return false;
+  if (Cp > 128 || (Cp == 96) || d->C % (Cp == 32 ? 2 : 4) != 0) return false;
   if ((long long)d->N * d->in[1] * d->in[2] * d->C * 2 >= (1ll << 30)) return false;   // 32-bit offsets into x, two spare bits
   int out[3], grid[3];
   if (wc_conv_out_dims(d, out, grid) != WC_OK) return false;
   if ((long long)d->N * out[1] * out[2] * d->K * 2 >= (1ll << 31)) return false;      // and into y
-  return d->K <= 8 * kThinK;
+  return d->K <= (Cp == 128 ? 4 : 8) * kThinK;   // measured: no gain beyond (K = 512 at 128 channels: 0.97x)
 }
 
 int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x, const void* U, const void* bias,
@@ -328,8 +366,15 @@ int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x,
   a.div_nW = make_fast_div(a.nW);
   a.div_nH = make_fast_div(a.nH);
   const int k_groups = ceil_div(d->K, kThinK);
-  if (d->dtype == WC_F16) return Cp == 64 ? launch_thin<half_t, 64>(a, k_groups, stream) : launch_thin<half_t, 32>(a, k_groups, stream);
-  return Cp == 64 ? launch_thin<bf16_t, 64>(a, k_groups, stream) : launch_thin<bf16_t, 32>(a, k_groups, stream);
+  return dispatch_dtype(d->dtype, [&](auto t) -> int {
+    using T = decltype(t);
+    if constexpr (sizeof(T) == 2) {
+      if (Cp == 128) return launch_thin<T, 128>(a, k_groups, stream);
+      return Cp == 64 ? launch_thin<T, 64>(a, k_groups, stream) : launch_thin<T, 32>(a, k_groups, stream);
+    } else {
+      return fail(WC_ERR_UNSUPPORTED, "thin_conv_forward: 16-bit types only");
+    }
+  });
 }
 
 }  // namespace wc

@@ -283,11 +283,13 @@ def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
     assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float32) == 4
     assert pkg.WinoConv2d(64, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4
     assert pkg.WinoConv2d(64, 1024, 3, padding=1)._tile_for(torch.float16) == 4     # too many output channels
-    assert pkg.WinoConv2d(96, 64, 3, padding=1)._tile_for(torch.float16) == 4       # too many input channels
+    assert pkg.WinoConv2d(96, 64, 3, padding=1)._tile_for(torch.float16) == 4       # no kernel for channels padded to 96
+    assert pkg.WinoConv2d(128, 128, 3, padding=1)._tile_for(torch.float16) == 2 and pkg.WinoConv2d(160, 64, 3, padding=1)._tile_for(torch.float16) == 4
     assert pkg.WinoConv2d(64, 64, 5, padding=2)._tile_for(torch.float16) == 4
     assert pkg.WinoConv2d(64, 64, 3, stride=2, padding=1)._tile_for(torch.float16) == 4
     t = engine.thin_layer
     assert t(torch.float16, 2, 64, 512, (3, 3), 1) and not t(torch.float16, 2, 64, 513, (3, 3), 1)
+    assert t(torch.float16, 2, 128, 256, (3, 3), 1) and not t(torch.float16, 2, 128, 257, (3, 3), 1) and not t(torch.float16, 2, 96, 8, (3, 3), 1)
     assert t(torch.float16, 2, 64, 128, (3, 3), 1) and t(torch.bfloat16, 2, 16, 8, (3, 3), (1, 1))
     assert t(torch.float16, 2, 40, 8, (3, 3), 1) and not t(torch.float16, 2, 42, 8, (3, 3), 1)   # 4 channels per thread
     assert t(torch.float16, 2, 30, 8, (3, 3), 1) and not t(torch.float16, 2, 3, 8, (3, 3), 1)    # 2 channels per thread

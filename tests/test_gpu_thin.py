@@ -1,5 +1,5 @@
 """The one-kernel F(2x2, 3x3) path that wc_conv_forward takes for thin fp16 / bf16 3x3 stride-1 layers
-(at most 64 input channels; conv_thin.hip).  It computes what the three-kernel path computes
+(at most 128 input channels; conv_thin.hip).  It computes what the three-kernel path computes
 (input transform of src/split_kernel.cu:60-120, batched product of
 src/base_conv_launchers.cu:353-367, output transform of src/split_kernel.cu:126-203) without V and M
 in memory, so the product is not rounded to the storage type before the output transform.
@@ -31,6 +31,9 @@ SHAPES = [
     (2, 64, 64, 3, 3, 0),        # one output pixel
     (1, 24, 32, 6, 20, 2),       # padding wider than the kernel needs
     (5, 64, 64, 30, 30, 1),      # more tiles than one round of workgroups' first blocks
+    (2, 128, 64, 9, 11, 1),      # 128 channels: eight wavefronts, element rows split between two groups of four
+    (3, 100, 130, 14, 14, 1),
+    (6, 128, 128, 28, 28, 1),
 ]
 
 
@@ -107,7 +110,8 @@ def test_tile_request_and_cached_filter(dev, dtype):
 @pytest.mark.parametrize("case", [
     # x shape, w shape, stride, dtype: outside the fused kernel's range, same result with and without `unfused`
     ((2, 3, 9, 9), (8, 3, 3, 3), 1, torch.float16),          # odd channel count
-    ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float16),        # more than 64 input channels
+    ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float16),        # channels pad to 96: no kernel of that width
+    ((2, 160, 9, 9), (8, 160, 3, 3), 1, torch.float16),      # more than 128 input channels
     ((2, 64, 9, 9), (520, 64, 3, 3), 1, torch.float16),      # more than 512 output channels
     ((2, 64, 12, 12), (8, 64, 3, 3), 2, torch.float16),      # stride 2
     ((2, 64, 12, 12), (8, 64, 5, 5), 1, torch.float16),      # DWM plan
