@@ -9,14 +9,16 @@
 // What makes it fit: U of one wavefront's 16 output channels (16 elements x 16 x Cp) stays in
 // registers for the life of the workgroup, so LDS only carries the transformed input of the
 // 16 tiles in flight.  A workgroup (4 wavefronts, 16 output channels each) walks over blocks of
-// 16 tiles: every thread loads the 4 x 4 window of one tile for Cp / 16 channels, transforms it in
-// fp32 and stores the 16 elements to LDS in the storage type; after one barrier every wavefront
-// multiplies all 16 elements by its part of U on v_mfma_f32_16x16x32 (U as the row operand, so
-// a lane ends up with 4 consecutive output channels of one tile).  The width half of the output
-// transform happens in the MFMA accumulators (A^T has only 0 and +-1: elements are added into the
-// accumulators they belong to, with the sign applied to the operand), the height half in fp32
-// registers.  The window of the next block is loaded before the products of this one, and LDS is
-// double-buffered, so there is one barrier per block.
+// 16 tiles: every thread loads the 4 x 4 window of one tile for a few channels, transforms it
+// (fp16: packed fp16 adds; bf16: fp32) and stores the 16 elements to LDS in the storage type; after
+// one barrier every wavefront multiplies all 16 elements by its part of U on v_mfma_f32_16x16x32
+// (U as the row operand, so a lane ends up with 4 consecutive output channels of one tile).  The
+// width half of the output transform happens in the MFMA accumulators (A^T has only 0 and +-1:
+// a product is added into the accumulators it belongs to), the height half in fp32 registers.  The
+// window of the next block is requested before the products of this one, and LDS is
+// double-buffered, so there is one barrier per block.  With 128 channels U would take the whole
+// register file: eight wavefronts then share a block, four per pair of element rows, and the
+// upper four hand their share of each output tile to the lower four through LDS (a second barrier).
 #include "wc_transform.h"
 #include <algorithm>
 
