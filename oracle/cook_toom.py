@@ -124,6 +124,8 @@ def matrices(m, r):
         return cook_toom(POINTS_F43, 4, 3)
     if (m, r) == (4, 2):
         return cook_toom(POINTS_F42, 4, 2)
+    if (m, r) == (3, 3):
+        return cook_toom(POINTS_F42, 3, 3)      # the shared tile of three-tap pieces: same four finite points
     if m == 2 and r in POINTS_F2R:
         return cook_toom(POINTS_F2R[r], 2, r)
     raise ValueError("F(%d,%d) not on the hot path" % (m, r))

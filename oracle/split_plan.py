@@ -65,11 +65,11 @@ def split_plan(kD, kH, kW):
     return plan
 
 
-def axis_pairs(k):
-    """Chunks of two taps, the remainder last: [(first_tap, 1, n_taps), ...].  Not a split of the
-    reference (its rule is chunks of three, base_conv_launchers.h:58-388): pieces that start at
-    even taps see, with output tile 2, the same transformed input moved by whole tiles."""
-    return [(s, 1, min(2, k - s)) for s in range(0, k, 2)]
+def axis_pairs(k, n=2):
+    """Chunks of n taps, the remainder last: [(first_tap, 1, n_taps), ...].  Not the split of the
+    reference (chunks of three with 4 -> 2 + 2, base_conv_launchers.h:58-388): pieces that start at
+    multiples of the output tile n see the same transformed input moved by whole tiles."""
+    return [(s, 1, min(n, k - s)) for s in range(0, k, n)]
 
 
 def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=False, pairs=False):
@@ -89,7 +89,7 @@ def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=Fals
         per_axis = [[(0, 1, k)] for k in kernel]
     elif pairs:
         assert stride == 1
-        per_axis = [axis_pairs(k) for k in kernel]
+        per_axis = [axis_pairs(k, m if isinstance(m, int) else 2) for k in kernel]
     else:
         per_axis = [axis_pieces(k, stride) for k in kernel]
     # m: one output tile extent for all axes, or one per axis (depth, height, width)

@@ -137,7 +137,9 @@ __global__ __launch_bounds__(256) void filter_transform_pieces_kernel(const Filt
   switch (r2) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
 #define WC_PLANE(K0) \
   switch (r1) { case 1: WC_ROW(K0, KA) break; case 2: WC_ROW(K0, KB) break; default: WC_ROW(K0, KC) }
-  if constexpr (FLAT) {
+  if constexpr (MO == 3) {
+    WC_BODY(KIND_11, KIND_33, KIND_33);       // three-tap pieces on the shared tile F(3,3), 2-D only
+  } else if constexpr (FLAT) {
     WC_PLANE(KIND_11)
   } else {
     switch (r0) { case 1: WC_PLANE(KIND_21) break; case 2: WC_PLANE(KIND_22) break; default: WC_PLANE(KIND_23) }
@@ -228,14 +230,15 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
     for (int q = 0; q < 3; ++q) small_taps = small_taps && plan->piece[i].r[q] >= 1 && plan->piece[i].r[q] <= 3;
   const bool flat = plan->m[0] == 1;
   const int mo = plan->m[1];
-  if (small_taps && plan->m[2] == mo && (flat ? (mo == 2 || mo == 4) : (mo == 2 && plan->m[0] == 2))) {
+  if (small_taps && plan->m[2] == mo && (flat ? (mo == 2 || mo == 4 || (mo == 3 && a.stacked)) : (mo == 2 && plan->m[0] == 2))) {
     const long long n = (long long)d->K * a.Cp;
     WC_CHECK_ARG(n < (1ll << 31), "wc_filter_transform: problem too large");
     const dim3 grid((unsigned)ceil_div_ll(n, 256), (unsigned)plan->n_pieces);
     void (*fn)(FilterArgs) = dispatch_dtype(d->dtype, [&](auto t) -> void (*)(FilterArgs) {
       using T = decltype(t);
       return !flat ? &filter_transform_pieces_kernel<T, false, 2>
-                   : (mo == 4 ? &filter_transform_pieces_kernel<T, true, 4> : &filter_transform_pieces_kernel<T, true, 2>);
+                   : (mo == 4 ? &filter_transform_pieces_kernel<T, true, 4>
+                      : mo == 3 ? &filter_transform_pieces_kernel<T, true, 3> : &filter_transform_pieces_kernel<T, true, 2>);
     });
     hipLaunchKernelGGL(fn, grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("filter_transform_pieces_kernel");

@@ -25,7 +25,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   // F(2,r) tiles with 16-byte accesses; 3-D tiles and whole-kernel tiles (up to 64 elements) use 2.
   int want;
   if (!flat) want = 2;
-  else if (plan->m[1] == 4 || plan->piece[0].r[1] > 3 || plan->piece[0].r[2] > 3) want = 2;
+  else if (plan->m[1] >= 3 || plan->piece[0].r[1] > 3 || plan->piece[0].r[2] > 3) want = 2;
   else want = d->dtype == WC_F32 ? 4 : 8;
   int vec = 1;
   for (int v = want; v > 1; v /= 2)
@@ -46,8 +46,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
 
   if (shared) {
     // the first piece with the tile all pieces share, over the extended tile grid
-    WC_CHECK_ARG(plan->m[1] == 2 && plan->m[2] == 2, "wc_input_transform: shared input needs output tile 2");
-    const int k0 = kind_of(plan->m[0], rp[0]), k1 = kind_of(2, rp[1]), k2 = kind_of(2, rp[2]);
+    const int k0 = kind_of(plan->m[0], rp[0]), k1 = kind_of(plan->m[1], rp[1]), k2 = kind_of(plan->m[2], rp[2]);
     InKernel fn = nullptr;
     switch (k0) {
       case KIND_11: fn = pick_in_2d(d->dtype, k1, k2, vec); break;
@@ -55,7 +54,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       case KIND_22: fn = pick_in_3d_22(d->dtype, k1, k2, vec); break;
       default: break;
     }
-    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform F(2,%d) x F(2,%d) x F(2,%d) not built", rp[0], rp[1], rp[2]);
+    if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for the shared tile (%d, %d, %d taps) not built", rp[0], rp[1], rp[2]);
     a.base0 = -d->pad[0]; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
     a.t_offset = 0;
     hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);

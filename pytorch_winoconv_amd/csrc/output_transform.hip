@@ -330,6 +330,7 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
   if (k0 == KIND_11 && k1 == KD && k2 == KD) \
     return vec == 4 ? &output_transform_kernel<T, KIND_11, KD, KD, 2> : &output_transform_kernel<T, KIND_11, KD, KD, 1>;
   WC_WHOLE(KIND_24) WC_WHOLE(KIND_25) WC_WHOLE(KIND_26) WC_WHOLE(KIND_27)
+  WC_WHOLE(KIND_33)       // the shared tile of three-tap pieces
 #undef WC_WHOLE
   return nullptr;
 }

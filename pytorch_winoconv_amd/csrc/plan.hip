@@ -50,10 +50,10 @@ static int axis_chunks(int k, int* start, int* size) {
   return n;
 }
 
-// chunks of two taps, the remainder last (plans whose pieces share one transformed input)
-static int axis_pairs(int k, AxisPiece* out) {
+// chunks of `len` taps, the remainder last (plans whose pieces share one transformed input: len = output tile)
+static int axis_even_chunks(int k, int len, AxisPiece* out) {
   int n = 0;
-  for (int s = 0; s < k; s += 2) { out[n].tap0 = s; out[n].r = k - s >= 2 ? 2 : 1; ++n; }
+  for (int s = 0; s < k; s += len) { out[n].tap0 = s; out[n].r = k - s >= len ? len : k - s; ++n; }
   return n;
 }
 
@@ -126,8 +126,8 @@ static int check_desc(const wc_conv_desc* d) {
                  "2-D problem needs depth extent 1, kernel 1, pad 0");
   if (d->stride != 1 && d->stride != 2)
     return fail(WC_ERR_UNSUPPORTED, "stride %d not implemented (1 or 2)", d->stride);
-  if (d->m != 2 && d->m != 4)
-    return fail(WC_ERR_UNSUPPORTED, "output tile %d not implemented (2 or 4)", d->m);
+  if (d->m != 2 && d->m != 4 && !(d->m == 3 && d->stacked == 2))
+    return fail(WC_ERR_UNSUPPORTED, "output tile %d not implemented (2 or 4; 3 with stacked = 2)", d->m);
   if (d->m == 4 && d->ndim == 3 &&
       !(d->stride == 1 && d->kernel[0] == 3 && d->kernel[1] == 3 && d->kernel[2] == 3))
     return fail(WC_ERR_UNSUPPORTED, "output tile 4 in 3-D (2 x 4 x 4) is implemented for 3x3x3 kernels at stride 1");
@@ -136,8 +136,11 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
     return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
-  if (d->stacked == 2 && (d->stride != 1 || d->m != 2))
-    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need stride 1 and output tile 2");
+  if (d->stacked == 2 && (d->stride != 1 || (d->m != 2 && d->m != 3)))
+    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need stride 1 and output tile 2 or 3");
+  if (d->stacked == 2 && d->m == 3 &&
+      (d->ndim != 2 || d->kernel[1] < 3 || d->kernel[2] < 3 || (d->kernel[1] == 3 && d->kernel[2] == 3)))
+    return fail(WC_ERR_UNSUPPORTED, "output tile 3 is built for 2-D kernels of at least 3 taps per axis and more than 3 on one");
   if (d->whole_kernel) {
     if (d->ndim != 2 || d->stride != 1 || d->m != 2)
       return fail(WC_ERR_UNSUPPORTED, "whole-kernel tiles need a 2-D problem, stride 1 and output tile 2");
@@ -156,7 +159,7 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   int n[3];
   for (int a = 0; a < 3; ++a) {
     if (d->whole_kernel) { ax[a][0].tap0 = 0; ax[a][0].r = d->kernel[a]; n[a] = 1; }
-    else if (d->stacked == 2) n[a] = axis_pairs(d->kernel[a], ax[a]);
+    else if (d->stacked == 2) n[a] = axis_even_chunks(d->kernel[a], d->m, ax[a]);
     else n[a] = axis_pieces(d->kernel[a], d->stride, ax[a]);
   }
   if (n[0] * n[1] * n[2] > WC_MAX_PIECES)
@@ -178,7 +181,7 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
         p.t_offset = t;
         int e = 1;
         for (int q = 0; q < 3; ++q) {
-          if (kind_of(plan->m[q], p.r[q]) < 0)
+          if (!d->stacked && kind_of(plan->m[q], p.r[q]) < 0)      // stacked: only the shared tile counts (below)
             return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) on axis %d not implemented", plan->m[q], p.r[q], q);
           e *= plan->m[q] + p.r[q] - 1;
         }
@@ -191,7 +194,8 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
     stacked_taps(plan, rp);
     t = 1;
     for (int q = 0; q < 3; ++q) {
-      if (rp[q] > 3) return fail(WC_ERR_UNSUPPORTED, "stacked plans need pieces of at most 3 taps");
+      if (rp[q] > 3 || kind_of(plan->m[q], rp[q]) < 0)
+        return fail(WC_ERR_UNSUPPORTED, "stacked plans need pieces of at most 3 taps and a tile F(%d,%d)", plan->m[q], rp[q]);
       t *= plan->m[q] + rp[q] - 1;
     }
     for (int s = 0; s < np; ++s) plan->piece[s].t_offset = 0;
@@ -210,7 +214,7 @@ int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
     int m = a == 0 ? (flat_depth ? 1 : (d->m == 4 ? 2 : d->m)) : d->m;
     grid[a] = (out[a] + m - 1) / m;
     // a shared transformed input covers the tiles that the pieces reach beyond the output's own
-    if (d->stacked == 2) grid[a] += (d->kernel[a] + 1) / 2 - 1;
+    if (d->stacked == 2) grid[a] += (d->kernel[a] + m - 1) / m - 1;
   }
   return WC_OK;
 }

@@ -72,8 +72,8 @@ inline int stacked_row(const wc_conv_desc* d, const wc_plan* plan) {
   return wc_padded_channels(d->C) * (d->stacked ? plan->n_pieces : 1);
 }
 
-// Plans with stacked == 2: the pieces start at even taps and use one tile F(2, 2 or 1) per axis, so
-// the transformed input of the piece that starts at tap (2 a, 2 b) is that of the first piece
+// Plans with stacked == 2: the pieces start at multiples of the output tile m (2, or 3 in 2-D) and use one tile
+// F(m, m or less) per axis, so the transformed input of the piece that starts at tap (m a, m b) is that of the first piece
 // a tile rows and b tiles further on.  V then holds one piece (row length Cp) over a tile grid
 // extended by the largest shifts (wc_conv_out_dims reports that grid), followed by `tail` rows that
 // only the products of the extension tiles read; the batched GEMM reads piece (a, b) of tile row p
@@ -89,9 +89,10 @@ struct SharedShift {          // pieces (a, b, c) of the depth, height and width
 };
 inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
   SharedShift s;
-  s.n_run = (d->kernel[2] + 1) / 2;
-  s.n_runs = (d->kernel[1] + 1) / 2;
-  s.n_planes = (d->kernel[0] + 1) / 2;
+  const int len = d->m;                           // taps per piece = output tile (3 only in 2-D: one depth piece)
+  s.n_run = (d->kernel[2] + len - 1) / len;
+  s.n_runs = (d->kernel[1] + len - 1) / len;
+  s.n_planes = (d->kernel[0] + len - 1) / len;
   s.run_rows = grid[2];
   s.plane_rows = grid[1] * grid[2];
   s.tail = (s.n_planes - 1) * s.plane_rows + (s.n_runs - 1) * s.run_rows + s.n_run - 1;

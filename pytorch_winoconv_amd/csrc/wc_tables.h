@@ -15,6 +15,8 @@
 //                              path: Cook-Toom (wincnn.py:49-70) over the points 0, 1, -1, 2 for
 //                              r = 4, 0, 1, -1, 2, -2 for r = 5 and 0, 1, -1, 1/2, -1/2, 1/3, -1/3
 //                              for r = 6, 7 (matrix_conv.py:31-35)
+//   KIND_33  F(3,3)  alpha 5   Cook-Toom over the points 0, 1, -1, 2 (wincnn.py:49-70): the tile of the
+//                              DWM plans whose three-tap pieces share one transformed input
 // KIND_41 / KIND_42 serve the pieces of a decomposed (DWM) kernel when the output tile is 4.
 // AT is m x alpha, G is alpha x r, BT is alpha x alpha.
 #pragma once
@@ -23,13 +25,13 @@
 namespace wc {
 
 enum Kind { KIND_11 = 0, KIND_21 = 1, KIND_22 = 2, KIND_23 = 3, KIND_43 = 4, KIND_41 = 5, KIND_42 = 6,
-            KIND_24 = 7, KIND_25 = 8, KIND_26 = 9, KIND_27 = 10, KIND_COUNT = 11 };
+            KIND_24 = 7, KIND_25 = 8, KIND_26 = 9, KIND_27 = 10, KIND_33 = 11, KIND_COUNT = 12 };
 
 __host__ __device__ constexpr int kind_m(int k) {
-  return k == KIND_11 ? 1 : (k == KIND_43 || k == KIND_41 || k == KIND_42) ? 4 : 2;
+  return k == KIND_11 ? 1 : k == KIND_33 ? 3 : (k == KIND_43 || k == KIND_41 || k == KIND_42) ? 4 : 2;
 }
 __host__ __device__ constexpr int kind_r(int k) {
-  return k >= KIND_24 ? 4 + (k - KIND_24)
+  return k == KIND_33 ? 3 : k >= KIND_24 ? 4 + (k - KIND_24)
        : (k == KIND_11 || k == KIND_21 || k == KIND_41) ? 1 : (k == KIND_22 || k == KIND_42) ? 2 : 3;
 }
 __host__ __device__ constexpr int kind_alpha(int k) { return kind_m(k) + kind_r(k) - 1; }
@@ -42,6 +44,7 @@ inline int kind_of(int m, int r) {
   if (m == 4 && r == 3) return KIND_43;
   if (m == 4 && r == 1) return KIND_41;
   if (m == 4 && r == 2) return KIND_42;
+  if (m == 3 && r == 3) return KIND_33;
   return -1;
 }
 
@@ -86,6 +89,25 @@ template <> struct Mats<KIND_23> {
   }
   __host__ __device__ static constexpr float bt(int i, int j) {
     constexpr float t[4][4] = {{1, 0, -1, 0}, {0, 1, 1, 0}, {0, -1, 1, 0}, {0, 1, 0, -1}};
+    return t[i][j];
+  }
+};
+template <> struct Mats<KIND_33> {
+  static constexpr int m = 3, r = 3, alpha = 5;
+  __host__ __device__ static constexpr float at(int i, int j) {
+    constexpr float t[3][5] = {{1, 1, 1, 1, 0}, {0, 1, -1, 2, 0}, {0, 1, 1, 4, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float g(int i, int j) {
+    constexpr float t[5][3] = {{1.f / 2, 0, 0},
+                               {-1.f / 2, -1.f / 2, -1.f / 2},
+                               {-1.f / 6, 1.f / 6, -1.f / 6},
+                               {1.f / 6, 1.f / 3, 2.f / 3},
+                               {0, 0, 1}};
+    return t[i][j];
+  }
+  __host__ __device__ static constexpr float bt(int i, int j) {
+    constexpr float t[5][5] = {{2, -1, -2, 1, 0}, {0, -2, -1, 1, 0}, {0, 2, -3, 1, 0}, {0, -1, 0, 1, 0}, {0, 2, -1, -2, 1}};
     return t[i][j];
   }
 };
@@ -256,6 +278,7 @@ __host__ __device__ inline float table_g(int kind, int i, int j) {
     case KIND_25: return Mats<KIND_25>::g(i, j);
     case KIND_26: return Mats<KIND_26>::g(i, j);
     case KIND_27: return Mats<KIND_27>::g(i, j);
+    case KIND_33: return Mats<KIND_33>::g(i, j);
     default: return Mats<KIND_43>::g(i, j);
   }
 }
@@ -271,6 +294,7 @@ __host__ __device__ inline float table_at(int kind, int i, int j) {
     case KIND_25: return Mats<KIND_25>::at(i, j);
     case KIND_26: return Mats<KIND_26>::at(i, j);
     case KIND_27: return Mats<KIND_27>::at(i, j);
+    case KIND_33: return Mats<KIND_33>::at(i, j);
     default: return Mats<KIND_43>::at(i, j);
   }
 }

@@ -69,8 +69,12 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
     d.stacked = 2 if stacked == 2 else int(bool(stacked))
-    if d.stacked == 2:
-        d.m = 2                      # the shared-input plan exists for output tile 2 only
+    if d.stacked == 2 and d.m == 4:
+        # the shared-input plan exists for output tiles 2 and 3: a caller who asked for tile 4 gets 3 where
+        # _stack picks that plan for its speed (fp16, 2-D, at least 3 taps per axis and 5 on one; F(3,3):
+        # fp16 error 3e-3 of the output range, between F(2,r) and F(4,r); too coarse for bf16), else 2
+        ks = d.kernel[1:]
+        d.m = 3 if (nd == 2 and dtype == torch.float16 and min(ks) >= 3 and max(ks) >= 5) else 2
     d.unfused = int(bool(unfused))
     return d
 
@@ -143,8 +147,8 @@ def input_transform(desc, plan, x_cl):
     P = n * grid[0] * grid[1] * grid[2]
     if desc.stacked == 2 and plan.n_pieces > 1:
         # one piece over the extended tile grid, plus the rows the shifted reads of the last tiles reach
-        tail = (((desc.kernel[0] + 1) // 2 - 1) * grid[1] * grid[2] + ((desc.kernel[1] + 1) // 2 - 1) * grid[2]
-                + (desc.kernel[2] + 1) // 2 - 1)
+        per = [(k + desc.m - 1) // desc.m for k in desc.kernel]        # pieces per axis
+        tail = (per[0] - 1) * grid[1] * grid[2] + (per[1] - 1) * grid[2] + per[2] - 1
         V = torch.zeros(plan.t_total, P + tail, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
     else:
         V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
@@ -182,10 +186,13 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
     plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit stride-1
     kernels of 4 to 8 taps over at most 128 input channels get the plan whose two-tap pieces share
-    one transformed input (2; make_desc then uses output tile 2): 1.1x (5x5), 1.4x (4x4), 1.5x (7x7)
+    one transformed input (2; make_desc then uses output tile 2): 1.2x (5x5), 1.45x (4x4), 1.5x (7x7)
     faster than stacked F(4,r) pieces at N=32, 128 channels, 112x112, and 1.5x (5x5x5) to 2x (4x4x4,
     7x7x7) faster than stacked F(2,r) pieces in 3-D; with 256 channels or 9 taps the larger product
-    costs more than the smaller V saves."""
+    costs more than the smaller V saves.  Where the caller accepts tile 4 (fp16, 2-D, 5 to 10 taps, at
+    least 3 on the other axis, at most 256 channels) the shared tile is F(3,3) with the reference's
+    three-tap pieces (make_desc: output tile 3): 1.4x (5x5) to 1.8x (7x7, 9x9) faster than stacked
+    F(4,r) pieces, also at 256 channels."""
     if stacked is not None:
         return 2 if stacked == 2 else bool(stacked)
     if whole_kernel or (nd == 3 and m != 2):
@@ -193,9 +200,13 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
     if dtype != torch.float32:
-        if (stride == 1 and w_shape is not None and 4 <= max(w_shape[2:]) <= 8
-                and (int(w_shape[1]) + 31) // 32 * 32 <= 128):
-            return 2
+        if stride == 1 and w_shape is not None:
+            ks = [int(k) for k in w_shape[2:]]
+            cp = (int(w_shape[1]) + 31) // 32 * 32
+            tile3 = dtype == torch.float16 and nd == 2 and m == 4 and min(ks) >= 3 and 5 <= max(ks) <= 10 and cp <= 256
+            tile2 = 4 <= max(ks) <= 8 and cp <= 128
+            if tile3 or tile2:
+                return 2
         return True
     if w_shape is None or nd != 2:
         return False

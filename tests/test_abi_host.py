@@ -230,8 +230,8 @@ def test_shared_input_plans():
     """stacked = 2: pieces of two taps on the tile F(2,2), one transformed input for all of them over a
     tile grid extended by the pieces' reach; 2-D, stride 1, output tile 2."""
     lib = _lib.load()
-    d = engine.make_desc((2, 8, 20, 21), (4, 8, 7, 5), torch.float16, 1, (3, 2), 4, stacked=2)
-    assert d.stacked == 2 and d.m == 2                    # the Python layer forces tile 2 for this plan
+    d = engine.make_desc((2, 8, 20, 21), (4, 8, 7, 5), torch.float16, 1, (3, 2), 2, stacked=2)
+    assert d.stacked == 2 and d.m == 2
     plan = engine.plan_conv(d)
     assert plan.n_pieces == 4 * 3 and plan.t_total == 9 and list(plan.m) == [1, 2, 2]
     want = [((0, 2 * a, 2 * b), (1, 2 if 2 * a + 2 <= 7 else 1, 2 if 2 * b + 2 <= 5 else 1)) for a in range(4) for b in range(3)]
@@ -264,12 +264,30 @@ def test_shared_input_plans():
     bad.m = 4
     with pytest.raises(NotImplementedError):
         engine.plan_conv(bad)
+    # tile 3: the reference's three-tap pieces on the shared tile F(3,3); what a caller who asked for tile 4 gets
+    # in fp16 (bf16: tile 2); 2-D, at least 3 taps per axis and more than 3 on one
+    d = engine.make_desc((2, 8, 20, 21), (4, 8, 7, 5), torch.float16, 1, (3, 2), 4, stacked=2)
+    assert d.m == 3 and engine.make_desc((2, 8, 20, 21), (4, 8, 7, 5), torch.bfloat16, 1, (3, 2), 4, stacked=2).m == 2
+    plan = engine.plan_conv(d)
+    assert plan.n_pieces == 3 * 2 and plan.t_total == 25 and list(plan.m) == [1, 3, 3]
+    assert [tuple(plan.piece[i].tap0) for i in range(6)] == [(0, 3 * a, 3 * b) for a in range(3) for b in range(2)]
+    assert [tuple(plan.piece[i].r) for i in range(6)] == [(1, 3, 3), (1, 3, 2), (1, 3, 3), (1, 3, 2), (1, 1, 3), (1, 1, 2)]
+    assert engine.out_dims(d) == ([1, 20, 21], [1, 7 + 2, 7 + 1])
+    for ws in ((4, 8, 3, 3), (4, 8, 5, 2)):
+        bad = engine.make_desc((2, 8, 20, 21), ws, torch.float16, 1, 1, 3, stacked=2)
+        with pytest.raises(NotImplementedError):
+            engine.plan_conv(bad)
+    bad = engine.make_desc((2, 8, 20, 21), (4, 8, 5, 5), torch.float16, 1, 1, 3)       # tile 3 without the shared plan
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(bad)
     # what the Python layer picks when nothing is said
     s = engine._stack
     assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 1, 4) == 2 and s(None, torch.bfloat16, 2, False, (8, 100, 4, 8), 1, 2) == 2
     assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 2, 4) is True        # stride 2
-    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 4) is True        # more than 128 channels
-    assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) is True and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
+    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 2) is True        # more than 128 channels with tile 2
+    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 4) == 2 and s(None, torch.float16, 2, False, (128, 300, 5, 5), 1, 4) is True
+    assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 2) is True and s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) == 2
+    assert s(None, torch.bfloat16, 2, False, (128, 128, 9, 9), 1, 4) is True and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
     assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) == 2
     assert s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 2) is True and s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 4) is False
     assert s(2, torch.float32, 2, False) == 2 and s(True, torch.float16, 2, False) is True and s(False, torch.float16, 2, False) is False

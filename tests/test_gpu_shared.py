@@ -116,6 +116,55 @@ def test_exact_on_small_integers(dev, case):
     assert torch.equal(y.cpu(), ref.half())
 
 
+TILE3 = [c for c in CASES if len(c[0]) == 4 and min(c[1][2:]) >= 3 and max(c[1][2:]) >= 4]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", TILE3)
+def test_three_tap_pieces_on_the_shared_tile_f33(dev, dtype, case):
+    """Output tile 3: the reference's pieces of three taps (3+3+1 for 7), every one on the tile F(3,3)
+    (Cook-Toom over 0, 1, -1, 2), sharing one transformed input.  Stages against the oracle to the
+    rounding of the storage type (the matrices are no longer 0 / +-1, so fp32 evaluation order shows);
+    result against fp64: fp16 2e-2 of the output range (measured 3e-3), bf16 6e-2 (measured 2-4e-2:
+    the Python layer never picks this tile for bf16)."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / (ws[1] * ws[2] * ws[3])) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    st = {}
+    y_oracle = ow.dwm_conv(x, w, b, 1, pad, 3, "fp16" if dtype == torch.float16 else "bf16", st, stacked=2)
+    desc = engine.make_desc(xs, ws, dtype, 1, pad, 3, stacked=2)
+    plan = engine.plan_conv(desc)
+    n_h, n_w = (ws[2] + 2) // 3, (ws[3] + 2) // 3
+    assert list(plan.m) == [1, 3, 3] and plan.t_total == 25 and plan.n_pieces == n_h * n_w == len(st["plan"]["pieces"])
+    C, N = xs[1], xs[0]
+    Cp = _lib.load().wc_padded_channels(C)
+    tol = 1.5e-3 if dtype == torch.float16 else 1.2e-2
+    U = engine.filter_transform(desc, plan, w.to(dev))
+    for i in range(plan.n_pieces):
+        assert _rel(U[:, :, i * Cp:i * Cp + C], st["U"][:, :, i * C:(i + 1) * C]) <= tol
+    (_, oH, oW), (_, gH, gW) = engine.out_dims(desc)
+    nH, nW = (oH + 2) // 3, (oW + 2) // 3
+    assert (gH, gW) == (nH + n_h - 1, nW + n_w - 1)
+    V = engine.input_transform(desc, plan, engine.channel_last(x.to(dev)))
+    Vg = V[:, :N * gH * gW, :C].cpu().reshape(25, N, gH, gW, C)
+    for a in range(n_h):
+        for c in range(n_w):
+            i = a * n_w + c
+            want = st["V"][:, :, i * C:(i + 1) * C].reshape(25, N, nH, nW, C)
+            assert _rel(Vg[:, :, a:a + nH, c:c + nW], want) <= tol, (a, c)
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 3, stacked=2)
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=pad)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert _rel(y, ref) <= (2e-2 if dtype == torch.float16 else 6e-2) and _rel(y, y_oracle) <= (1e-2 if dtype == torch.float16 else 6e-2)
+    if dtype == torch.float16 and max(ws[2:]) >= 5:
+        # what a caller who asks for tile 4 gets by default
+        assert torch.equal(engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 4), y)
+        Uc = engine.transform_filter(w.to(dev), xs, 1, pad, 4)
+        assert torch.equal(engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 4, U=Uc, chunk_images=1), y)
+
+
 def _random_cases(seed, n):
     rng = random.Random(seed)
     out = []
@@ -155,6 +204,9 @@ def test_random_shapes(dev, case):
     ref = _conv(x.double(), w.double(), None, pad)
     y = engine.conv_forward(x.to(dev), w.to(dev), None, 1, pad, 2, stacked=2)
     assert tuple(y.shape) == tuple(ref.shape) and _rel(y, ref) <= 2e-2
+    if len(ks) == 2 and min(ks) >= 3 and max(ks) >= 4 and dtype == torch.float16:
+        y3 = engine.conv_forward(x.to(dev), w.to(dev), None, 1, pad, 3, stacked=2)
+        assert tuple(y3.shape) == tuple(ref.shape) and _rel(y3, ref) <= 2e-2
 
 
 def _bad_tile_4(xs, ws):
@@ -177,7 +229,8 @@ def test_what_the_plan_is_not_built_for(dev):
     dy = torch.randn(2, 4, 12, 12).half().to(dev)
     dw = engine.conv_backward_weight(x, dy, w.shape, 1, 2, 2, stacked=2)
     assert torch.equal(dw, engine.conv_backward_weight(x, dy, w.shape, 1, 2, 2, stacked=True))
-    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 2), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 3, stacked=2))
 
 
 def test_c4_layer_at_full_size(dev):
@@ -189,5 +242,7 @@ def test_c4_layer_at_full_size(dev):
     y1 = engine.conv_forward(x, w, None, 1, 3, 2, stacked=True)
     scale = float(y1.float().abs().max())
     assert float((y.float() - y1.float()).abs().max()) <= 4e-3 * scale
+    y3 = engine.conv_forward(x, w, None, 1, 3, 3, stacked=2)                     # three-tap pieces on F(3,3)
+    assert float((y3.float() - y1.float()).abs().max()) <= 1.5e-2 * scale
     sample = F.conv2d(x[:1].double().cpu(), w.double().cpu(), padding=3)
     assert _rel(y[:1], sample) <= 2e-3

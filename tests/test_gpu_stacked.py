@@ -92,7 +92,8 @@ def test_cached_filter_chunks_and_size_check(dev):
     # at most 128 channels the one whose pieces share the transformed input (test_gpu_shared.py)
     assert torch.equal(engine.conv_forward(x, w, None, 2, 2, 4), engine.conv_forward(x, w, None, 2, 2, 4, stacked=True))
     assert torch.equal(engine.transform_filter(w, xs, 2, 2, 4), engine.transform_filter(w, xs, 2, 2, 4, stacked=True))
-    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 4), engine.conv_forward(x, w, None, 1, 2, 3, stacked=2))
+    assert torch.equal(engine.conv_forward(x, w, None, 1, 2, 2), engine.conv_forward(x, w, None, 1, 2, 2, stacked=2))
     # a filter transformed for the other form has another size and is refused, not misread
     with pytest.raises(ValueError):
         engine.conv_forward(x, w, None, 1, 2, 4, U=U, stacked=False)

@@ -48,7 +48,7 @@ def test_generator_satisfies_fir_identity_exactly(m, r, points):
 
 
 @pytest.mark.parametrize("m,r", [(1, 1), (2, 1), (2, 2), (2, 3), (4, 1), (4, 2), (4, 3),
-                                 (2, 4), (2, 5), (2, 6), (2, 7)])
+                                 (2, 4), (2, 5), (2, 6), (2, 7), (3, 3)])
 def test_tables_in_use_satisfy_fir_identity_exactly(m, r):
     AT, G, BT = ct.matrices(m, r)
     as_frac = lambda M: [[Fraction(v).limit_denominator(1000) for v in row] for row in M]
@@ -158,4 +158,16 @@ def test_kernel_spot_formulas():
 
 def test_unsupported_pair_is_rejected():
     with pytest.raises(ValueError):
-        ct.matrices(3, 3)
+        ct.matrices(3, 2)
+
+
+def test_f33_of_the_shared_input_plans():
+    """F(3,3) over the points 0, 1, -1, 2 (the reference's point set for five-element tiles,
+    matrix_conv.py:32): exact rationals of the generator against the literals the HIP tables hold."""
+    AT, G, BT = ct.cook_toom_exact(ct.POINTS_F42, 3, 3)
+    F_ = Fraction
+    assert AT == [[1, 1, 1, 1, 0], [0, 1, -1, 2, 0], [0, 1, 1, 4, 1]]
+    assert G == [[F_(1, 2), 0, 0], [F_(-1, 2), F_(-1, 2), F_(-1, 2)], [F_(-1, 6), F_(1, 6), F_(-1, 6)],
+                 [F_(1, 6), F_(1, 3), F_(2, 3)], [0, 0, 1]]
+    assert BT == [[2, -1, -2, 1, 0], [0, -2, -1, 1, 0], [0, 2, -3, 1, 0], [0, -1, 0, 1, 0], [0, 2, -1, -2, 1]]
+    _fir_identity_exact(AT, G, BT, 3, 3)
