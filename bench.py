@@ -74,9 +74,10 @@ def cpu_baseline(sample_images=32, repeats=3):
 SUITE = [
     # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size).
     # c3, 64 and 128 channels: the default is the fused F(2,3) kernel; the three-kernel F(4,3) line stands beside it.
-    # c4: the 16-bit default adds the DWM pieces in the batched GEMM, at stride 1 with pieces of two taps
-    # that share one transformed input, else with the reference's pieces of three ("stacked"); two lines
-    # with the reference's structure (pieces added after their output transforms) stand beside them.
+    # c4: the 16-bit default adds the DWM pieces in the batched GEMM; at stride 1 the pieces share one
+    # transformed input (tile 3 / F(3,3) with the reference's three-tap pieces where the caller asks for tile 4,
+    # tile 2 / F(2,2) with two-tap pieces where it asks for 2), else each has its own ("stacked"); two lines with
+    # the reference's structure (pieces added after their output transforms) stand beside them.
     ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(2,3) x13", "vgg", None, 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(4,3) x13", "vgg", None, 1, 1, 4, "f32"),
@@ -86,6 +87,8 @@ SUITE = [
     ("c3 fp16 N64 C128 28x28 F(4,3) three kernels", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, "f16"),
     ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 1, 1, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 5x5 s1 DWM shared input F(3,3)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s1 DWM shared input F(3,3)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM shared input F(2,2)", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM shared input F(2,2)", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 2, "f16-stacked"),

@@ -67,7 +67,7 @@ typedef struct {
   int kernel[3];   /* kD, kH, kW (kD = 1 when ndim == 2)                        */
   int pad[3];      /* symmetric zero padding per axis                           */
   int stride;      /* 1 or 2, same on every axis                                */
-  int m;           /* Winograd output tile: 2, or 4 (2-D: 4 x 4; 3-D: 2 x 4 x 4, 3x3x3 stride 1 only) */
+  int m;           /* Winograd output tile: 2, or 4 (2-D: 4 x 4; 3-D: 2 x 4 x 4, 3x3x3 stride 1 only), or 3 (with stacked = 2) */
   int dtype;       /* wc_dtype                                                  */
   int chunk_images;/* images per pass of wc_conv_forward; 0 = choose automatically */
   int whole_kernel;/* 0: kernels > 3 are decomposed into pieces of <= 3 taps (DWM, dwm.py:107-146);
@@ -90,7 +90,8 @@ typedef struct {
                     *    reports that grid) plus the rows that the moved reads of its last tiles reach, U holds the
                     *    pieces side by side as for 1, and the batched GEMM reads each piece's rows of V at that
                     *    piece's tile offset.  Same sum as 0 and 1; V is written and read once instead of once
-                    *    per piece. */
+                    *    per piece.  With m = 3 (2-D, at least 3 taps per axis and more than 3 on one) the pieces
+                    *    have three taps, the reference's split without its 4 -> 2 + 2 exception, on the tile F(3,3). */
   int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2 whose input channels
                     *    pad to 32, 64 or 128 (an even number up to 32, a multiple of 4 in 33..64 or 97..128)
                     *    and that have at most 512 output channels (256 with 128 input channels) run as one
