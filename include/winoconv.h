@@ -92,11 +92,13 @@ typedef struct {
                     *    piece's tile offset.  Same sum as 0 and 1; V is written and read once instead of once
                     *    per piece.  With m = 3 (2-D, at least 3 taps per axis and more than 3 on one) the pieces
                     *    have three taps, the reference's split without its 4 -> 2 + 2 exception, on the tile F(3,3). */
-  int unfused;     /* wc_conv_forward only.  0: fp16 / bf16 3x3 stride-1 2-D layers with m = 2 whose input channels
-                    *    pad to 32, 64 or 128 (an even number up to 32, a multiple of 4 in 33..64 or 97..128)
-                    *    and that have at most 512 output channels (256 with 128 input channels) run as one
-                    *    kernel: input transform, products and output transform of F(2x2, 3x3) without V and
-                    *    M in memory, the product kept in fp32 (x below 1 GiB);
+  int unfused;     /* wc_conv_forward only.  0: 3x3 stride-1 2-D layers with m = 2 run as ONE kernel (input transform,
+                    *    products and output transform of F(2x2, 3x3) without V and M in memory, the product
+                    *    kept in fp32; x below 1 GiB) if they have
+                    *    - at most 4 input channels (any dtype, at most 512 output channels): first layers, or
+                    *    - fp16 / bf16 data and input channels that pad to 32, 64 or 128 (an even number up to
+                    *      32, a multiple of 4 in 33..64 or 97..128), at most 512 output channels (256 with
+                    *      128 input channels);
                     * 1: always filter transform -> input transform -> batched GEMM -> output transform. */
 } wc_conv_desc;
 
@@ -173,7 +175,7 @@ int wc_output_transform(const wc_conv_desc* desc, const wc_plan* plan,
  * The workspace holds U, V and M (the reference's tmp_weight_buffer, tmp_input_buffer,
  * tmp_product_buffer: dwm.py:122-125); images are processed in chunks that bound the size
  * of V and M.  `U_cached` (may be NULL) is a filter already transformed
- * by wc_filter_transform; `w` may then be NULL.  Thin 16-bit 3x3 layers take one fused kernel
+ * by wc_filter_transform; `w` may then be NULL.  Thin 3x3 layers take one fused kernel
  * instead (see wc_conv_desc.unfused); the workspace then only holds U. */
 int wc_conv_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
 int wc_conv_u_elems(const wc_conv_desc* desc, size_t* elems);

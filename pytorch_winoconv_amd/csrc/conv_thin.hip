@@ -1,4 +1,5 @@
-// One-kernel F(2x2, 3x3) convolution for thin 16-bit layers (at most 128 input channels).
+// One-kernel F(2x2, 3x3) convolution for thin layers: fp16 / bf16 with at most 128 input channels, and any
+// storage type with at most 4 (tiny_conv3x3_kernel, further down).
 //
 // Same arithmetic as the three-kernel path (input transform of src/split_kernel.cu:60-120, the
 // batched product of src/base_conv_launchers.cu:353-367, output transform of
@@ -58,7 +59,7 @@ struct ThinArgs {
   const void* U;
   const void* bias;
   void* y;
-  int H, W, C, K;
+  int H, W, C, K, Cp;
   int oH, oW, nH, nW;
   int pad1, pad2;
   int P;          // tiles of the whole batch
@@ -70,6 +71,57 @@ struct ThinArgs {
   int k_whole;    // K is a multiple of 4: a lane's 4 output channels go out in one store
   FastDiv div_nW, div_nH;
 };
+
+// Bias and store of one lane's share of an output tile: tile p, output channels ko .. ko + 4, the 2 x 2
+// output positions in out[oa][ob].  Stores go through a buffer descriptor: an output position outside
+// (oH, oW) gets an offset beyond the buffer and is dropped.
+template <typename T>
+__device__ __forceinline__ void store_tile(const ThinArgs& a, __amdgpu_buffer_rsrc_t ydesc, int p, int ko,
+                                           const floatx4 (&out)[2][2]) {
+  const int q = fast_div(p, a.div_nW);
+  const int tw = p - q * a.nW;
+  const int b = fast_div(q, a.div_nH);
+  const int th = q - b * a.nH;
+  const T* bias = static_cast<const T*>(a.bias);
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (ko + r < a.K) bv[r] = static_cast<float>(bias[ko + r]);
+  }
+  const unsigned o00 = (((unsigned)b * a.oH + 2 * th) * a.oW + 2 * tw) * a.K + ko;   // in elements
+  const bool h1 = 2 * th + 1 < a.oH, w1 = 2 * tw + 1 < a.oW;
+#pragma unroll
+  for (int oa = 0; oa < 2; ++oa) {
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob) {
+      const floatx4 s4 = out[oa][ob];
+      const bool inside = (oa == 0 || h1) && (ob == 0 || w1);
+      const unsigned off = o00 + (oa * a.oW + ob) * a.K;
+      Pack<T, 4> o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o.v[r] = static_cast<T>(s4[r] + bv[r]);
+      if (a.k_whole) {
+        const unsigned byte_off = inside ? off * (unsigned)sizeof(T) : kOutside;
+        if constexpr (sizeof(T) == 4) {
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o), ydesc, byte_off, 0, 0);
+        } else {
+          typedef unsigned u2 __attribute__((ext_vector_type(2)));
+          __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, o), ydesc, byte_off, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const unsigned byte_off = inside && ko + r < a.K ? (off + r) * (unsigned)sizeof(T) : kOutside;
+          if constexpr (sizeof(T) == 4)
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, o.v[r]), ydesc, byte_off, 0, 0);
+          else
+            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, o.v[r]), ydesc, byte_off, 0, 0);
+        }
+      }
+    }
+  }
+}
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
@@ -264,49 +316,130 @@ __global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_pe
       }
     }
 
-    // height half of the output transform, bias, store: lane = tile lane % 16, output channels
-    // ko .. ko + 4.  Stores go through a buffer descriptor: an output position outside (oH, oW) gets
-    // an offset beyond the buffer and is dropped.
+    // lane = tile lane % 16, output channels ko .. ko + 4
     const int p = blk * kThinTiles + (lane & 15);
     const int ko = kbase + 4 * (lane >> 4);
-    if (p < a.P && ko < a.K && (!SPLIT || wave < 4)) {
-      const int q = fast_div(p, a.div_nW);
-      const int tw = p - q * a.nW;
-      const int b = fast_div(q, a.div_nH);
-      const int th = q - b * a.nH;
-      const T* bias = static_cast<const T*>(a.bias);
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bias) {
+    if (p < a.P && ko < a.K && (!SPLIT || wave < 4)) store_tile<T>(a, ydesc, p, ko, out);
+  }
+}
+
+// The same for at most 4 input channels (first layers: grey or RGB images), any storage type.  Padding 3
+// channels to the 32 of the batched GEMM makes V ten times the input, and M is 4x the output whatever
+// the channel count, so the three-kernel path spends its time on buffers; here the product runs on
+// v_mfma_f32_16x16x4_f32 in fp32 with a reduction of exactly 4 channels, U (16 elements x 16 output
+// channels x 4) is 16 registers per lane, and a block is 64 tiles: a thread transforms one channel of
+// one tile, a wavefront multiplies four column blocks of 16 tiles.
+template <typename T>
+__global__ __launch_bounds__(256) void tiny_conv3x3_kernel(ThinArgs a) {
+  constexpr int TILES = 64;
+  constexpr int BUF = 16 * TILES * 4;     // floats per buffer, [element][tile][channel]
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  float* ldsf = reinterpret_cast<float*>(lds);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kbase = blockIdx.y * kThinK + wave * 16;
+  const int pl = tid >> 2, c = tid & 3;
+  const bool c_ok = c < a.C;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(a.x), 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ydesc = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+  Pack<T, 1> raw[16];
+
+  auto load_window = [&](int blk) {      // offsets as in thin_conv3x3_kernel
+    const int p = blk * TILES + pl;
+    const bool valid = p < a.P && c_ok;
+    const int q = fast_div(p, a.div_nW);
+    const int tw = p - q * a.nW;
+    const int b = fast_div(q, a.div_nH);
+    const int th = q - b * a.nH;
+    const int y0 = 2 * th - a.pad1, x0 = 2 * tw - a.pad2;
+    const unsigned row0 = (unsigned)(b * a.H + y0) * (unsigned)a.row_bytes;
+    const unsigned col0 = (unsigned)(x0 * a.C + c) * (unsigned)sizeof(T);
+    unsigned rowoff[4], coloff[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (ko + r < a.K) bv[r] = static_cast<float>(bias[ko + r]);
-      }
-      const unsigned o00 = (((unsigned)b * a.oH + 2 * th) * a.oW + 2 * tw) * a.K + ko;   // in elements
-      const bool h1 = 2 * th + 1 < a.oH, w1 = 2 * tw + 1 < a.oW;
+    for (int i = 0; i < 4; ++i) {
+      rowoff[i] = valid && (unsigned)(y0 + i) < (unsigned)a.H ? row0 + i * a.row_bytes : 0x80000000u;
+      coloff[i] = (unsigned)(x0 + i) < (unsigned)a.W ? col0 + i * a.C * (unsigned)sizeof(T) : 0x40000000u;
+    }
 #pragma unroll
-      for (int oa = 0; oa < 2; ++oa) {
+    for (int i1 = 0; i1 < 4; ++i1)
 #pragma unroll
-        for (int ob = 0; ob < 2; ++ob) {
-          const floatx4 s4 = out[oa][ob];
-          const bool inside = (oa == 0 || h1) && (ob == 0 || w1);
-          const unsigned off = o00 + (oa * a.oW + ob) * a.K;
-          Pack<T, 4> o;
+      for (int i2 = 0; i2 < 4; ++i2) raw[i1 * 4 + i2] = buffer_load_pack<T, 1>(rsrc, rowoff[i1] + coloff[i2]);
+  };
+
+  const int nwg = gridDim.x;
+  int blk = xcd_remap(blockIdx.x, a.per_xcd);
+  if (blk < a.n_blocks) load_window(blk);
+
+  // U as the row operand: lane = output channel kbase + lane % 16, input channel lane / 16 (U's rows are
+  // Cp long, channels beyond C hold zeros)
+  float u[16];
+  {
+    const int ko = min(kbase + (lane & 15), a.K - 1);
+    const T* U = static_cast<const T*>(a.U) + (long long)ko * a.Cp + (lane >> 4);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o.v[r] = static_cast<T>(s4[r] + bv[r]);
-          if (a.k_whole) {
-            typedef unsigned u2 __attribute__((ext_vector_type(2)));
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, o), ydesc,
-                                                  inside ? off * (unsigned)sizeof(T) : kOutside, 0, 0);
-          } else {
+    for (int t = 0; t < 16; ++t) u[t] = static_cast<float>(U[(long long)t * a.K * a.Cp]);
+  }
+
+  for (int it = 0; blk < a.n_blocks; blk += nwg, ++it) {
+    float* buf = ldsf + (it & 1) * BUF;
+    {
+      float d[16], t2[16];
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, o.v[r]), ydesc,
-                                                    inside && ko + r < a.K ? (off + r) * (unsigned)sizeof(T) : kOutside, 0, 0);
-          }
+      for (int e = 0; e < 16; ++e) d[e] = static_cast<float>(raw[e].v[0]);
+      bt23<1, 4>(d, t2);
+      bt23<4, 1>(t2, d);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) buf[(e * TILES + pl) * 4 + c] = d[e];
+    }
+    __syncthreads();
+    if (blk + nwg < a.n_blocks) load_window(blk + nwg);
+
+#pragma unroll 1
+    for (int cb = 0; cb < TILES / 16; ++cb) {
+      floatx4 z0[4], zp[4], zn[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const float* vcol = buf + (cb * 16 + (lane & 15)) * 4 + (lane >> 4);
+      static_for<0, 4>([&](auto j_) {
+        constexpr int j = decltype(j_)::value;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = vcol[(i * 4 + j) * TILES * 4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if constexpr (j <= 2) z0[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(u[i * 4 + j], v[i], z0[i], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (j == 1) zp[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(u[i * 4 + j], v[i], zp[i], 0, 0, 0);
+          if constexpr (j >= 2) zn[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(u[i * 4 + j], v[i], zn[i], 0, 0, 0);
         }
+      });
+      floatx4 out[2][2];
+#pragma unroll
+      for (int ob = 0; ob < 2; ++ob) {
+        floatx4 z[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) z[i] = ob == 0 ? z0[i] : zp[i] - zn[i];
+        out[0][ob] = z[0] + z[1] + z[2];
+        out[1][ob] = z[1] - z[2] - z[3];
       }
+      const int p = blk * TILES + cb * 16 + (lane & 15);
+      const int ko = kbase + 4 * (lane >> 4);
+      if (p < a.P && ko < a.K) store_tile<T>(a, ydesc, p, ko, out);
     }
   }
+}
+
+template <typename T>
+int launch_tiny(ThinArgs a, int k_groups, void* stream) {
+  constexpr int lds = 2 * 16 * 64 * 4 * 4;
+  a.n_blocks = ceil_div(a.P, 64);
+  int wgs = std::min(a.n_blocks, std::max(kXcds, 1024 / k_groups / kXcds * kXcds));
+  a.per_xcd = ceil_div(wgs, kXcds);
+  hipLaunchKernelGGL((tiny_conv3x3_kernel<T>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256), lds,
+                     as_stream(stream), a);
+  WC_CHECK_LAUNCH("tiny_conv3x3_kernel");
+  return WC_OK;
 }
 
 template <typename T, int CP>
@@ -328,16 +461,19 @@ int launch_thin(ThinArgs a, int k_groups, void* stream) {
 }  // namespace
 
 bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan) {
-  if (d->ndim != 2 || d->dtype == WC_F32 || d->whole_kernel) return false;
+  if (d->ndim != 2 || d->whole_kernel) return false;
   if (plan->n_pieces != 1 || plan->tap_step != 1 || plan->m[0] != 1 || plan->m[1] != 2 || plan->m[2] != 2) return false;
   const wc_piece& pc = plan->piece[0];
   if (pc.r[0] != 1 || pc.r[1] != 3 || pc.r[2] != 3) return false;
-  const int Cp = wc_padded_channels(d->C);
-  if (Cp > 128 || (Cp == 96) || d->C % (Cp == 32 ? 2 : 4) != 0) return false;
-  if ((long long)d->N * d->in[1] * d->in[2] * d->C * 2 >= (1ll << 30)) return false;   // 32-bit offsets into x, two spare bits
+  const long long es = d->dtype == WC_F32 ? 4 : 2;
+  if ((long long)d->N * d->in[1] * d->in[2] * d->C * es >= (1ll << 30)) return false;   // 32-bit offsets into x, two spare bits
   int out[3], grid[3];
   if (wc_conv_out_dims(d, out, grid) != WC_OK) return false;
-  if ((long long)d->N * out[1] * out[2] * d->K * 2 >= (1ll << 31)) return false;      // and into y
+  if ((long long)d->N * out[1] * out[2] * d->K * es >= (1ll << 31)) return false;      // and into y
+  if (d->C <= 4) return d->K <= 8 * kThinK;          // tiny_conv3x3_kernel, any storage type
+  if (d->dtype == WC_F32) return false;
+  const int Cp = wc_padded_channels(d->C);
+  if (Cp > 128 || (Cp == 96) || d->C % (Cp == 32 ? 2 : 4) != 0) return false;
   return d->K <= (Cp == 128 ? 4 : 8) * kThinK;   // measured: no gain beyond (K = 512 at 128 channels: 0.97x)
 }
 
@@ -350,24 +486,26 @@ int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x,
   const int Cp = wc_padded_channels(d->C);
   const long long P = (long long)d->N * grid[1] * grid[2];
   WC_CHECK_ARG(P < (1ll << 31) - kThinTiles, "thin_conv_forward: too many tiles");
-  WC_CHECK_ARG((reinterpret_cast<uintptr_t>(x) & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 7) == 0 &&
+  WC_CHECK_ARG((reinterpret_cast<uintptr_t>(x) & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(U) & 15) == 0,
-               "thin_conv_forward: x and y must be 8-byte aligned, U 16-byte aligned");
+               "thin_conv_forward: x must be 8-byte aligned, y and U 16-byte aligned");
+  const int es = d->dtype == WC_F32 ? 4 : 2;
   ThinArgs a;
   a.x = x; a.U = U; a.bias = bias; a.y = y;
-  a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.K = d->K;
+  a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.K = d->K; a.Cp = Cp;
   a.oH = out[1]; a.oW = out[2]; a.nH = grid[1]; a.nW = grid[2];
   a.pad1 = d->pad[1]; a.pad2 = d->pad[2];
   a.P = (int)P;
   a.n_blocks = (int)ceil_div_ll(P, kThinTiles);
   a.per_xcd = 0;
-  a.x_bytes = (int)((long long)d->N * d->in[1] * d->in[2] * d->C * 2);
-  a.y_bytes = (int)((long long)d->N * out[1] * out[2] * d->K * 2);
+  a.x_bytes = (int)((long long)d->N * d->in[1] * d->in[2] * d->C * es);
+  a.y_bytes = (int)((long long)d->N * out[1] * out[2] * d->K * es);
   a.k_whole = d->K % 4 == 0;
-  a.row_bytes = d->in[2] * d->C * 2;
+  a.row_bytes = d->in[2] * d->C * es;
   a.div_nW = make_fast_div(a.nW);
   a.div_nH = make_fast_div(a.nH);
   const int k_groups = ceil_div(d->K, kThinK);
+  if (d->C <= 4) return dispatch_dtype(d->dtype, [&](auto t) -> int { return launch_tiny<decltype(t)>(a, k_groups, stream); });
   return dispatch_dtype(d->dtype, [&](auto t) -> int {
     using T = decltype(t);
     if constexpr (sizeof(T) == 2) {

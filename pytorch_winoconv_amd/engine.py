@@ -219,12 +219,17 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
 
 def thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
     """True for the layers wc_conv_forward runs as one fused F(2x2, 3x3) kernel (wc_conv_desc.unfused):
-    fp16 / bf16, 2-D, 3x3, stride 1, input channels padded to 32, 64 or 128 (an even number up to 32, a
-    multiple of 4 in 33..64 and 97..128) and at most 512 output channels (256 with 128 input channels).  Callers that cache U use it to
-    transform the filter with tile 2."""
-    if dtype == torch.float32 or nd != 2 or tuple(kernel) != (3, 3):
+    2-D, 3x3, stride 1 and either at most 4 input channels (any type, at most 512 output channels) or
+    fp16 / bf16 with input channels padded to 32, 64 or 128 (an even number up to 32, a multiple of 4 in
+    33..64 and 97..128) and at most 512 output channels (256 with 128 input channels).  Callers that
+    cache U use it to transform the filter with tile 2."""
+    if nd != 2 or tuple(kernel) != (3, 3):
         return False
     if (stride if isinstance(stride, int) else max(stride)) != 1:
+        return False
+    if in_channels <= 4:
+        return out_channels <= 512
+    if dtype == torch.float32:
         return False
     cp = (in_channels + 31) // 32 * 32
     return (cp in (32, 64, 128) and in_channels % (2 if cp == 32 else 4) == 0

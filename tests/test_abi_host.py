@@ -221,7 +221,7 @@ def test_modules_pick_tile_2_where_tile_4_loses_accuracy():
     assert wide._tile_for(torch.float16) == 4 and wide._tile_for(torch.float32) == 4
     assert wide._tile_for(torch.bfloat16) == 2          # 8 mantissa bits
     assert thin._tile_for(torch.float16) == 2            # too few channels to average the rounding error down
-    assert thin._tile_for(torch.float32) == 4
+    assert thin._tile_for(torch.float32) == 2            # 3 channels: the fused first-layer kernel, tile 2
     assert pkg.WinoConv2d(3, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4   # an explicit choice stands
     assert pkg.WinoConv3d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
 
@@ -310,7 +310,9 @@ def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
     assert t(torch.float16, 2, 128, 256, (3, 3), 1) and not t(torch.float16, 2, 128, 257, (3, 3), 1) and not t(torch.float16, 2, 96, 8, (3, 3), 1)
     assert t(torch.float16, 2, 64, 128, (3, 3), 1) and t(torch.bfloat16, 2, 16, 8, (3, 3), (1, 1))
     assert t(torch.float16, 2, 40, 8, (3, 3), 1) and not t(torch.float16, 2, 42, 8, (3, 3), 1)   # 4 channels per thread
-    assert t(torch.float16, 2, 30, 8, (3, 3), 1) and not t(torch.float16, 2, 3, 8, (3, 3), 1)    # 2 channels per thread
+    assert t(torch.float16, 2, 30, 8, (3, 3), 1) and not t(torch.float16, 2, 7, 8, (3, 3), 1)    # 2 channels per thread
+    assert t(torch.float16, 2, 3, 64, (3, 3), 1) and t(torch.float32, 2, 3, 64, (3, 3), 1) and t(torch.float32, 2, 1, 512, (3, 3), 1)   # first layers
+    assert not t(torch.float32, 2, 5, 64, (3, 3), 1) and not t(torch.float32, 2, 3, 600, (3, 3), 1)
     assert not t(torch.float16, 3, 64, 64, (3, 3), 1) and not t(torch.float32, 2, 64, 64, (3, 3), 1)
 
 

@@ -109,13 +109,13 @@ def test_tile_request_and_cached_filter(dev, dtype):
 
 @pytest.mark.parametrize("case", [
     # x shape, w shape, stride, dtype: outside the fused kernel's range, same result with and without `unfused`
-    ((2, 3, 9, 9), (8, 3, 3, 3), 1, torch.float16),          # odd channel count
+    ((2, 5, 9, 9), (8, 5, 3, 3), 1, torch.float16),          # odd channel count above 4
     ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float16),        # channels pad to 96: no kernel of that width
     ((2, 160, 9, 9), (8, 160, 3, 3), 1, torch.float16),      # more than 128 input channels
     ((2, 64, 9, 9), (520, 64, 3, 3), 1, torch.float16),      # more than 512 output channels
     ((2, 64, 12, 12), (8, 64, 3, 3), 2, torch.float16),      # stride 2
     ((2, 64, 12, 12), (8, 64, 5, 5), 1, torch.float16),      # DWM plan
-    ((2, 64, 9, 9), (8, 64, 3, 3), 1, torch.float32),
+    ((2, 64, 9, 9), (8, 64, 3, 3), 1, torch.float32),       # fp32 with more than 4 channels
     ((2, 64, 5, 9, 9), (8, 64, 3, 3, 3), 1, torch.float16),  # 3-D
 ])
 def test_outside_the_range_nothing_changes(dev, case):
@@ -143,3 +143,52 @@ def test_resnet_layer_at_full_size(dev):
     assert float((y12.float() - y1.float() - y2.float()).abs().max()) <= 6e-3 * scale
     sample = F.conv2d(x[:2].double().cpu(), w1.double().cpu(), padding=1)
     assert _rel(y1[:2], sample) <= 2e-3
+
+
+TINY = [
+    # N, C, K, H, W, pad: at most 4 input channels, any storage type (tiny_conv3x3_kernel)
+    (2, 3, 64, 12, 12, 1),
+    (1, 1, 8, 7, 9, 1),
+    (3, 4, 70, 13, 11, 0),
+    (2, 2, 6, 9, 9, 1),
+    (1, 3, 130, 20, 21, 2),
+    (9, 3, 32, 17, 16, 1),       # more than one block of 64 tiles
+    (2, 3, 64, 3, 3, 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", TINY)
+def test_first_layers_exact_on_small_integers(dev, dtype, shape):
+    """Same construction as above; the product of these layers runs in fp32 whatever the storage type."""
+    N, C, K, H, W, pad = shape
+    g = torch.Generator().manual_seed(13)
+    x = torch.randint(-3, 4, (N, C, H, W), generator=g).double()
+    w = 4.0 * torch.randint(-2, 3, (K, C, 3, 3), generator=g).double()
+    b = torch.randint(-8, 9, (K,), generator=g).double()
+    ref = F.conv2d(x, w, b, padding=pad).float().to(dtype)
+    y = engine.conv_forward(x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev), 1, pad, 2)
+    assert tuple(y.shape) == tuple(ref.shape) and torch.equal(y.cpu(), ref)
+    assert torch.equal(engine.conv_forward(x.to(dtype).to(dev), w.to(dtype).to(dev), None, 1, pad, 2).cpu(),
+                       F.conv2d(x, w, None, padding=pad).float().to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", TINY)
+def test_first_layers_against_fp64_and_three_kernel_path(dev, dtype, shape):
+    N, C, K, H, W, pad = shape
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(N, C, H, W, generator=g).to(dtype)
+    w = (torch.randn(K, C, 3, 3, generator=g) * (2.0 / (9 * C)) ** 0.5).to(dtype)
+    b = torch.randn(K, generator=g).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=pad)
+    xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
+    y = engine.conv_forward(xd, wd, bd, 1, pad, 2)
+    y3 = engine.conv_forward(xd, wd, bd, 1, pad, 2, unfused=True)
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    assert _rel(y, ref) <= tol and _rel(y3, ref) <= tol and _rel(y, y3.cpu()) <= tol
+    assert _rel(y, ref) <= 1.5 * _rel(y3, ref) + (1e-6 if dtype == torch.float32 else 1e-4)
+    U = engine.transform_filter(wd, x.shape, 1, pad, 2)
+    assert torch.equal(engine.conv_forward(xd, wd, bd, 1, pad, 2, U=U), y)
+    if dtype != torch.float32 or True:
+        assert not torch.equal(y3, y) or dtype == torch.float32      # other roundings: the fused kernel did run
