@@ -15,6 +15,10 @@
 // filter block and "B" the input block: a lane then holds 4 consecutive output channels of
 // one tile row per accumulator group and stores them as one 8-byte (fp16) / 16-byte (fp32)
 // write.  fp16 and bf16 accumulate in fp32; fp32 uses v_mfma_f32_32x32x2_f32.
+//
+// Plans whose pieces share one transformed input read V at a row offset per piece: gemm_kernel
+// with SHIFT walks the operand pointer piece by piece; gemm_rows_kernel serves the pieces of one
+// run (neighbours along the width) from a single operand tile that is n_run - 1 rows taller.
 #include "wc_common.h"
 #include <cstdlib>
 
@@ -70,6 +74,9 @@ struct GemmArgs {
   // by jump2 more (3-D plans: on to the next depth plane of the tile grid)
   int ldv, run_blocks, plane_runs;
   long long jump, jump2;
+  // the same plans for gemm_rows_kernel: pieces per run, runs in all, and what the first row of
+  // a run moves by from one run to the next / beyond that from one plane to the next (rows of V)
+  int n_run, total_runs, run_rows, plane_extra;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -263,6 +270,237 @@ static GemmConfig make_config() {
                     stages > out_tile ? stages : out_tile, 64 * NWP * NWK};
 }
 
+// The shifted product with the pieces of one run served by ONE operand tile.  Piece b of a run
+// multiplies rows p + b of V, so a tile of BM + n_run - 1 rows holds what all n_run pieces of the
+// run need from one block of 32 channels: the reduction runs (run, channel block, piece) with the
+// piece innermost, V is loaded once per (run, channel block) instead of once per piece, and only
+// the filter block changes from step to step.  The shifted gemm_kernel is bound by L2-to-LDS
+// traffic (every piece loads its own copy of nearly the same rows); this form loads
+// (BM + n_run - 1 + n_run BN) rows per run and channel block instead of n_run (BM + BN).
+// LDS: two stages of V (BM + kRunExtra rows) and two of U (BN rows); the V block of the next
+// (run, channel block) is requested at the first piece of the current one and parked in
+// registers until the last piece.  The accumulation order differs from gemm_kernel's (pieces of a
+// run alternate), so results agree to fp32 rounding, not bit for bit.
+constexpr int kRunExtra = 8;       // pieces per run are at most kRunExtra + 1
+
+template <typename T, int WM, int WN, int NWP, int NWK, int PF>
+__global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm_rows_kernel(GemmArgs g) {
+  using MF = Mfma<T>;
+  constexpr int BK = 32;
+  constexpr int NT = 64 * NWP * NWK;
+  constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
+  constexpr int EPC = 16 / sizeof(T);
+  constexpr int CPR = BK / EPC;
+  constexpr int RPP = NT / CPR;                    // rows covered by one pass of the workgroup
+  constexpr int NLV = BM / RPP, NLU = BN / RPP;
+  constexpr int VSTAGE = (BM + kRunExtra) * BK, USTAGE = BN * BK;
+  static_assert(sizeof(T) == 2 && CPR == 4 && RPP % 16 == 0, "16-bit operands in 64-byte swizzled rows");
+  static_assert(BM % RPP == 0 && BN % RPP == 0 && kRunExtra <= RPP, "tile rows must be a multiple of the load pass");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  T* ldsV = lds;
+  T* ldsU = lds + 2 * VSTAGE;
+
+  const int blk = xcd_remap(blockIdx.x, g.per_xcd);
+  if (blk >= g.n_blocks) return;
+  const int kt_ = blk % g.tiles_k;
+  const int pt = (blk / g.tiles_k) % g.tiles_p;
+  const int t = blk / (g.tiles_k * g.tiles_p);
+  const int p0 = pt * BM, k0 = kt_ * BN;
+  const int n_run = g.n_run;
+
+  const T* Vt = static_cast<const T*>(g.V) + (long long)t * g.sV;
+  const T* Ut = static_cast<const T*>(g.U) + (long long)t * g.sU;
+
+  const int tid = threadIdx.x;
+  const int lrow = tid / CPR, lpart = tid % CPR;
+  // rows past the last tile of the grid still lie inside V's tail for every piece of the run
+  const int last_row = g.P - 1 + n_run - 1;
+  const T* vptr[NLV + 1];
+  int vloff[NLV + 1];
+#pragma unroll
+  for (int i = 0; i <= NLV; ++i) {
+    const int row = lrow + i * RPP;                // i == NLV: the n_run - 1 rows beyond the tile
+    vptr[i] = Vt + (long long)min(p0 + row, last_row) * g.ldv + lpart * EPC;
+    vloff[i] = row * BK + (lpart ^ swizzle(row)) * EPC;
+  }
+  const bool has_extra = lrow < n_run - 1;
+  const T* uptr[NLU];
+  int uloff[NLU];
+#pragma unroll
+  for (int i = 0; i < NLU; ++i) {
+    const int row = lrow + i * RPP;
+    uptr[i] = Ut + (long long)min(k0 + row, g.K - 1) * g.Cp + lpart * EPC;
+    uloff[i] = row * BK + (lpart ^ swizzle(row)) * EPC;
+  }
+
+  Chunk16 vregs[NLV + 1], uregs[PF][NLU];
+  auto vload = [&](long long off) {
+#pragma unroll
+    for (int i = 0; i < NLV; ++i) vregs[i] = *reinterpret_cast<const Chunk16*>(vptr[i] + off);
+    if (has_extra) vregs[NLV] = *reinterpret_cast<const Chunk16*>(vptr[NLV] + off);
+  };
+  auto vstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NLV; ++i) *reinterpret_cast<Chunk16*>(ldsV + buf * VSTAGE + vloff[i]) = vregs[i];
+    if (has_extra) *reinterpret_cast<Chunk16*>(ldsV + buf * VSTAGE + vloff[NLV]) = vregs[NLV];
+  };
+  auto uload = [&](int set, long long off) {
+#pragma unroll
+    for (int i = 0; i < NLU; ++i) uregs[set][i] = *reinterpret_cast<const Chunk16*>(uptr[i] + off);
+  };
+  auto ustore = [&](int set, int buf) {
+#pragma unroll
+    for (int i = 0; i < NLU; ++i) *reinterpret_cast<Chunk16*>(ldsU + buf * USTAGE + uloff[i]) = uregs[set][i];
+  };
+
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave / NWK, wk = wave % NWK;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int xrow = wp * WM * 32 + l32;             // first V row of this lane (piece 0)
+  const int woff = (wk * WN * 32 + l32) * BK;
+  const int fzw = swizzle(l32);
+  auto koff = [&](int kk, int fz) {                // element kk*kstep + lhi*kpack of a swizzled row
+    const int e = kk * MF::kstep + lhi * MF::kpack;
+    return (((e / EPC) ^ fz) * EPC) + e % EPC;
+  };
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // A group is one (run, channel block); its V block sits at element offset nv of a V row, the
+  // filter block of its piece b at offset (run n_run + b) ldv + 32 cc of a U row.  Filter blocks
+  // travel through PF register sets (step s in set s % PF), requested PF steps ahead: a step is
+  // only WM WN MFMAs per reduction block long, shorter than a round trip to L2.
+  const int ncc = g.ldv / BK;
+  const int groups = g.total_runs * ncc;
+  const int nsteps = groups * n_run;
+  long long nv = 0;                                // V offset of the next group to load
+  int ncc_left = ncc, plane_left = g.plane_runs;
+  long long row_shift = 0;
+  auto advance_v = [&]() {
+    if (--ncc_left > 0) { nv += BK; return; }
+    ncc_left = ncc;
+    row_shift += g.run_rows;
+    if (--plane_left == 0) { row_shift += g.plane_extra; plane_left = g.plane_runs; }
+    nv = row_shift * g.ldv;
+  };
+  long long lu_run = 0;                            // U cursor of the next step to load
+  int lu_b = 0, lu_cc = 0;
+  auto next_u = [&]() {                            // offset of the cursor's step, then move it on
+    const long long off = lu_run + (long long)lu_b * g.ldv + lu_cc * BK;
+    if (++lu_b == n_run) {
+      lu_b = 0;
+      if (++lu_cc == ncc) { lu_cc = 0; lu_run += (long long)n_run * g.ldv; }
+    }
+    return off;
+  };
+  vload(0);
+  advance_v();
+#pragma unroll
+  for (int s = 0; s < PF; ++s)
+    if (s < nsteps) uload(s, next_u());
+  vstore(0);
+  ustore(0, 0);
+  __syncthreads();
+  int gi = 0, b = 0;
+  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int step = s0 + u;
+      if (PF > 1 && step >= nsteps) break;
+      const bool more = gi + 1 < groups;
+      const bool last = b == n_run - 1;
+      if (b == 0 && more) vload(nv);
+      if (step + PF < nsteps) uload(u, next_u());
+      const T* stv = ldsV + (gi & 1) * VSTAGE;
+      const T* stu = ldsU + (step & 1) * USTAGE;
+      const int xoff = (xrow + b) * BK;
+      const int fzx = swizzle(l32 + b);
+      constexpr int KK = BK / MF::kstep;
+      typename MF::Frag xf[2][WM], wf[2][WN];
+      auto fload = [&](int kk, int sb) {
+        const int kx = koff(kk, fzx), kw = koff(kk, fzw);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+          xf[sb][i] = *reinterpret_cast<const typename MF::Frag*>(stv + xoff + i * 32 * BK + kx);
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          wf[sb][j] = *reinterpret_cast<const typename MF::Frag*>(stu + woff + j * 32 * BK + kw);
+      };
+      fload(0, 0);
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        if (kk + 1 < KK) fload(kk + 1, (kk + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[kk & 1][j], xf[kk & 1][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (last && more) { vstore((gi + 1) & 1); advance_v(); }
+      if (step + 1 < nsteps) ustore((u + 1) % PF, (step + 1) & 1);
+      __syncthreads();
+      if (last) { b = 0; ++gi; } else ++b;
+    }
+  }
+
+  // Epilogue as in gemm_kernel: the tile goes through LDS so that global stores are whole rows.
+  constexpr int EI = NWP * NWK == 4 ? WM : WM / 2;
+  constexpr int CS = BN + EPC;
+  constexpr int SROWS = 32 * NWP * EI;
+  T* cs = lds;
+  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
+  constexpr int CPRO = BN / EPC;
+  constexpr int RPPO = NT / CPRO;
+  static_assert(EI >= 1 && WM % EI == 0 && NT % CPRO == 0 && SROWS % RPPO == 0, "output tile shape");
+  const int orow = tid / CPRO, ocol = (tid % CPRO) * EPC;
+#pragma unroll
+  for (int i0 = 0; i0 < WM; i0 += EI) {
+    if (i0 > 0) __syncthreads();
+#pragma unroll
+    for (int ii = 0; ii < EI; ++ii)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          Pack<T, 4> o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i0 + ii][j][4 * q + e]);
+          *reinterpret_cast<Pack<T, 4>*>(cs + (wp * EI * 32 + ii * 32 + l32) * CS + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi) = o;
+        }
+    __syncthreads();
+    if (k0 + ocol < g.ldm) {
+#pragma unroll
+      for (int r = 0; r < SROWS / RPPO; ++r) {
+        const int srow = orow + r * RPPO;
+        const int row = (srow / (EI * 32)) * WM * 32 + i0 * 32 + srow % (EI * 32);
+        if (p0 + row < g.P)
+          *reinterpret_cast<Chunk16*>(Mt + (long long)(p0 + row) * g.ldm + k0 + ocol) =
+              *reinterpret_cast<const Chunk16*>(cs + srow * CS + ocol);
+      }
+    }
+  }
+}
+
+template <typename T, int WM, int WN, int NWP, int NWK, int PF>
+static GemmConfig make_rows_config() {
+  constexpr int EPC = 16 / sizeof(T);
+  constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
+  constexpr int EI = NWP * NWK == 4 ? WM : WM / 2;
+  constexpr size_t stages = (size_t)2 * (BM + kRunExtra + BN) * 32 * sizeof(T);
+  constexpr size_t out_tile = (size_t)32 * NWP * EI * (BN + EPC) * sizeof(T);
+  return GemmConfig{&gemm_rows_kernel<T, WM, WN, NWP, NWK, PF>, BM, BN, 32, stages > out_tile ? stages : out_tile,
+                    64 * NWP * NWK};
+}
+
 // Tile shapes: 0..4 four wavefronts, largest first; 5 (16-bit types) 128 x 256 with eight wavefronts.
 template <typename T> struct Configs;
 template <> struct Configs<half_t> {
@@ -359,6 +597,22 @@ static GemmConfig choose_shifted(int T_, int P, int K) {
   return make_config<T, 1, 1, 32, 2, 2, true>();               // 64 x 64
 }
 
+// Tiles of gemm_rows_kernel.  Measured at N=32, 128 channels, 112x112, 5x5 / 7x7 kernels and at
+// 3-D 5x5x5 kernels: 256 x 128 with four wavefronts is 8-15 % faster than the tile per piece
+// (eight wavefronts are slower than either: their 64 x 64 wavefront tiles read more of LDS per
+// MFMA, and that is the bound once the operand traffic is halved); 128 x 128 wins 8-10 % below about
+// 2000 big tiles (256 channels at 56x56, small 3-D problems); small problems keep the tile per
+// piece (no kernel: fn == nullptr).
+template <typename T>
+static GemmConfig choose_rows(int T_, int P, int K, bool always) {
+  auto blocks = [&](const GemmConfig& c) { return (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_; };
+  GemmConfig big = make_rows_config<T, 4, 2, 2, 2, 1>();       // 256 x 128
+  if (blocks(big) >= 2048 && !always) return big;                         // four rounds of two workgroups per CU
+  GemmConfig mid = make_rows_config<T, 2, 2, 2, 2, 2>();       // 128 x 128
+  if (blocks(mid) >= 512 || always) return mid;
+  return GemmConfig{nullptr, 0, 0, 0, 0, 0};
+}
+
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream) {
   WC_CHECK_ARG(V && U && M, "batched_gemm_shifted: null pointer");
@@ -370,6 +624,17 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "batched_gemm_shifted: row stride %d", ldm);
   if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_shifted: 16-bit types only");
   GemmConfig c = dtype == WC_F16 ? choose_shifted<half_t>(T_, P, K) : choose_shifted<bf16_t>(T_, P, K);
+  // Runs of two and more pieces over more than 64 output channels, on problems that fill the chip
+  // with 128-row tiles: one operand tile per run.  WINOCONV_GEMM_ROWS=0 keeps the tile per piece,
+  // =2 takes the 128 x 128 tile of gemm_rows_kernel for every plan with runs (what the tests use
+  // to reach it with small shapes).
+  const char* rows_env = std::getenv("WINOCONV_GEMM_ROWS");
+  const int rows_mode = rows_env ? std::atoi(rows_env) : 1;
+  bool rows = sh.n_run >= 2 && sh.n_run <= kRunExtra + 1 && rows_mode != 0 && (K > 64 || rows_mode == 2);
+  if (rows) {
+    GemmConfig r = dtype == WC_F16 ? choose_rows<half_t>(T_, P, K, rows_mode == 2) : choose_rows<bf16_t>(T_, P, K, rows_mode == 2);
+    if (r.fn) c = r; else rows = false;
+  }
   GemmArgs g;
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.ldm = ldm;
@@ -379,6 +644,8 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   g.jump = (long long)(sh.run_rows - sh.n_run) * Cp;     // on to the same tile one grid row further
   g.plane_runs = sh.n_runs;
   g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
+  g.n_run = sh.n_run; g.total_runs = sh.n_planes * sh.n_runs;
+  g.run_rows = sh.run_rows; g.plane_extra = sh.plane_rows - sh.n_runs * sh.run_rows;
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
@@ -389,7 +656,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
     WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
-  WC_CHECK_LAUNCH("gemm_kernel (shifted operand)");
+  WC_CHECK_LAUNCH(rows ? "gemm_rows_kernel" : "gemm_kernel (shifted operand)");
   return WC_OK;
 }
 
@@ -410,6 +677,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.P = P; g.K = K; g.Cp = Cp; g.ldm = ldm;
   g.sV = (long long)P * Cp; g.sU = (long long)K * Cp; g.sM = (long long)P * ldm;
   g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
+  g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

@@ -116,6 +116,15 @@ def test_exact_on_small_integers(dev, case):
     assert torch.equal(y.cpu(), ref.half())
 
 
+@pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
+def test_one_operand_tile_per_run_is_exact_on_small_integers(dev, case, monkeypatch):
+    """The product kernel that serves all pieces of a run from one tile of V (chosen by size; here
+    forced, so that small shapes with partial tiles, one to five pieces per run and 3-D plane jumps
+    reach it): same integer inputs as above, so the other order of its sums changes nothing."""
+    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+    test_exact_on_small_integers(dev, case)
+
+
 TILE3 = [c for c in CASES if len(c[0]) == 4 and min(c[1][2:]) >= 3 and max(c[1][2:]) >= 4]
 
 
@@ -207,6 +216,12 @@ def test_random_shapes(dev, case):
     if len(ks) == 2 and min(ks) >= 3 and max(ks) >= 4 and dtype == torch.float16:
         y3 = engine.conv_forward(x.to(dev), w.to(dev), None, 1, pad, 3, stacked=2)
         assert tuple(y3.shape) == tuple(ref.shape) and _rel(y3, ref) <= 2e-2
+
+
+@pytest.mark.parametrize("case", RANDOM[::2], ids=[str(i) for i in range(0, len(RANDOM), 2)])
+def test_random_shapes_with_one_operand_tile_per_run(dev, case, monkeypatch):
+    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+    test_random_shapes(dev, case)
 
 
 def _bad_tile_4(xs, ws):
