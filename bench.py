@@ -95,7 +95,8 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-stacked"),
-    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 4, "f16"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),

@@ -283,7 +283,7 @@ static GemmConfig make_config() {
 // run alternate), so results agree to fp32 rounding, not bit for bit.
 constexpr int kRunExtra = 8;       // pieces per run are at most kRunExtra + 1
 
-template <typename T, int WM, int WN, int NWP, int NWK, int PF>
+template <typename T, int WM, int WN, int NWP, int NWK>
 __global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm_rows_kernel(GemmArgs g) {
   using MF = Mfma<T>;
   constexpr int BK = 32;
@@ -335,24 +335,26 @@ __global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm
     uloff[i] = row * BK + (lpart ^ swizzle(row)) * EPC;
   }
 
-  Chunk16 vregs[NLV + 1], uregs[PF][NLU];
+  Chunk16 vregs[NLV + 1], uregs[NLU];
+  auto vload_extra = [&](long long off) {
+    if (has_extra) vregs[NLV] = *reinterpret_cast<const Chunk16*>(vptr[NLV] + off);
+  };
   auto vload = [&](long long off) {
 #pragma unroll
     for (int i = 0; i < NLV; ++i) vregs[i] = *reinterpret_cast<const Chunk16*>(vptr[i] + off);
-    if (has_extra) vregs[NLV] = *reinterpret_cast<const Chunk16*>(vptr[NLV] + off);
   };
   auto vstore = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < NLV; ++i) *reinterpret_cast<Chunk16*>(ldsV + buf * VSTAGE + vloff[i]) = vregs[i];
     if (has_extra) *reinterpret_cast<Chunk16*>(ldsV + buf * VSTAGE + vloff[NLV]) = vregs[NLV];
   };
-  auto uload = [&](int set, long long off) {
+  auto uload = [&](long long off) {
 #pragma unroll
-    for (int i = 0; i < NLU; ++i) uregs[set][i] = *reinterpret_cast<const Chunk16*>(uptr[i] + off);
+    for (int i = 0; i < NLU; ++i) uregs[i] = *reinterpret_cast<const Chunk16*>(uptr[i] + off);
   };
-  auto ustore = [&](int set, int buf) {
+  auto ustore = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < NLU; ++i) *reinterpret_cast<Chunk16*>(ldsU + buf * USTAGE + uloff[i]) = uregs[set][i];
+    for (int i = 0; i < NLU; ++i) *reinterpret_cast<Chunk16*>(ldsU + buf * USTAGE + uloff[i]) = uregs[i];
   };
 
   const int lane = tid & 63, wave = tid >> 6;
@@ -375,13 +377,14 @@ __global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   // A group is one (run, channel block); its V block sits at element offset nv of a V row, the
-  // filter block of its piece b at offset (run n_run + b) ldv + 32 cc of a U row.  Filter blocks
-  // travel through PF register sets (step s in set s % PF), requested PF steps ahead: a step is
-  // only WM WN MFMAs per reduction block long, shorter than a round trip to L2.
+  // filter block of its piece b at offset (run n_run + b) ldv + 32 cc of a U row.  Every group
+  // is the same straight line of loads, waits and stores (first piece, middle pieces, last piece;
+  // the last group requests a block it never uses), so that the compiler can count what is in
+  // flight at each wait.  Loads return in order: the filter block of the next step is requested
+  // BEFORE the V block of the next group, and the end of the first step waits for it alone.
   const int ncc = g.ldv / BK;
   const int groups = g.total_runs * ncc;
-  const int nsteps = groups * n_run;
-  long long nv = 0;                                // V offset of the next group to load
+  long long nv = 0;                                // V offset of the next group
   int ncc_left = ncc, plane_left = g.plane_runs;
   long long row_shift = 0;
   auto advance_v = [&]() {
@@ -391,65 +394,77 @@ __global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm
     if (--plane_left == 0) { row_shift += g.plane_extra; plane_left = g.plane_runs; }
     nv = row_shift * g.ldv;
   };
-  long long lu_run = 0;                            // U cursor of the next step to load
-  int lu_b = 0, lu_cc = 0;
-  auto next_u = [&]() {                            // offset of the cursor's step, then move it on
-    const long long off = lu_run + (long long)lu_b * g.ldv + lu_cc * BK;
+  long long lu_run = 0;                            // U cursor: the next step to request
+  int lu_b = 0, lu_cc = 0, lu_left = groups * n_run;
+  auto next_u = [&]() {                            // its offset (0 past the end), then move it on
+    const long long off = lu_left > 0 ? lu_run + (long long)lu_b * g.ldv + lu_cc * BK : 0;
+    --lu_left;
     if (++lu_b == n_run) {
       lu_b = 0;
       if (++lu_cc == ncc) { lu_cc = 0; lu_run += (long long)n_run * g.ldv; }
     }
     return off;
   };
+  auto multiply = [&](const T* stv, const T* stu, int b) {
+    const int xoff = (xrow + b) * BK;
+    const int fzx = swizzle(l32 + b);
+    constexpr int KK = BK / MF::kstep;
+    typename MF::Frag xf[2][WM], wf[2][WN];
+    auto fload = [&](int kk, int sb) {
+      const int kx = koff(kk, fzx), kw = koff(kk, fzw);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        xf[sb][i] = *reinterpret_cast<const typename MF::Frag*>(stv + xoff + i * 32 * BK + kx);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        wf[sb][j] = *reinterpret_cast<const typename MF::Frag*>(stu + woff + j * 32 * BK + kw);
+    };
+    fload(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) fload(kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[kk & 1][j], xf[kk & 1][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  vload_extra(0);
+  uload(next_u());
   vload(0);
   advance_v();
-#pragma unroll
-  for (int s = 0; s < PF; ++s)
-    if (s < nsteps) uload(s, next_u());
   vstore(0);
-  ustore(0, 0);
+  ustore(0);
   __syncthreads();
-  int gi = 0, b = 0;
-  for (int s0 = 0; s0 < nsteps; s0 += PF) {
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-      const int step = s0 + u;
-      if (PF > 1 && step >= nsteps) break;
-      const bool more = gi + 1 < groups;
-      const bool last = b == n_run - 1;
-      if (b == 0 && more) vload(nv);
-      if (step + PF < nsteps) uload(u, next_u());
-      const T* stv = ldsV + (gi & 1) * VSTAGE;
-      const T* stu = ldsU + (step & 1) * USTAGE;
-      const int xoff = (xrow + b) * BK;
-      const int fzx = swizzle(l32 + b);
-      constexpr int KK = BK / MF::kstep;
-      typename MF::Frag xf[2][WM], wf[2][WN];
-      auto fload = [&](int kk, int sb) {
-        const int kx = koff(kk, fzx), kw = koff(kk, fzw);
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-          xf[sb][i] = *reinterpret_cast<const typename MF::Frag*>(stv + xoff + i * 32 * BK + kx);
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-          wf[sb][j] = *reinterpret_cast<const typename MF::Frag*>(stu + woff + j * 32 * BK + kw);
-      };
-      fload(0, 0);
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        if (kk + 1 < KK) fload(kk + 1, (kk + 1) & 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-#pragma unroll
-          for (int j = 0; j < WN; ++j) acc[i][j] = MF::run(wf[kk & 1][j], xf[kk & 1][i], acc[i][j]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (last && more) { vstore((gi + 1) & 1); advance_v(); }
-      if (step + 1 < nsteps) ustore((u + 1) % PF, (step + 1) & 1);
+  int ub = 0;                                      // U stage of the current step
+  for (int gi = 0; gi < groups; ++gi) {
+    const long long vnext = gi + 1 < groups ? nv : 0;
+    const T* stv = ldsV + (gi & 1) * VSTAGE;
+    // first piece: request the next filter block, then the next group's V block
+    vload_extra(vnext);
+    uload(next_u());
+    vload(vnext);
+    multiply(stv, ldsU + ub * USTAGE, 0);
+    ustore(ub ^ 1);
+    __syncthreads();
+    ub ^= 1;
+    for (int b = 1; b < n_run - 1; ++b) {
+      uload(next_u());
+      multiply(stv, ldsU + ub * USTAGE, b);
+      ustore(ub ^ 1);
       __syncthreads();
-      if (last) { b = 0; ++gi; } else ++b;
+      ub ^= 1;
     }
+    // last piece: the V block moves from registers to the other stage
+    uload(next_u());
+    multiply(stv, ldsU + ub * USTAGE, n_run - 1);
+    vstore((gi + 1) & 1);
+    ustore(ub ^ 1);
+    __syncthreads();
+    ub ^= 1;
+    advance_v();
   }
 
   // Epilogue as in gemm_kernel: the tile goes through LDS so that global stores are whole rows.
@@ -490,14 +505,14 @@ __global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm
   }
 }
 
-template <typename T, int WM, int WN, int NWP, int NWK, int PF>
+template <typename T, int WM, int WN, int NWP, int NWK>
 static GemmConfig make_rows_config() {
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
   constexpr int EI = NWP * NWK == 4 ? WM : WM / 2;
   constexpr size_t stages = (size_t)2 * (BM + kRunExtra + BN) * 32 * sizeof(T);
   constexpr size_t out_tile = (size_t)32 * NWP * EI * (BN + EPC) * sizeof(T);
-  return GemmConfig{&gemm_rows_kernel<T, WM, WN, NWP, NWK, PF>, BM, BN, 32, stages > out_tile ? stages : out_tile,
+  return GemmConfig{&gemm_rows_kernel<T, WM, WN, NWP, NWK>, BM, BN, 32, stages > out_tile ? stages : out_tile,
                     64 * NWP * NWK};
 }
 
@@ -606,9 +621,9 @@ static GemmConfig choose_shifted(int T_, int P, int K) {
 template <typename T>
 static GemmConfig choose_rows(int T_, int P, int K, bool always) {
   auto blocks = [&](const GemmConfig& c) { return (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_; };
-  GemmConfig big = make_rows_config<T, 4, 2, 2, 2, 1>();       // 256 x 128
+  GemmConfig big = make_rows_config<T, 4, 2, 2, 2>();       // 256 x 128
   if (blocks(big) >= 2048 && !always) return big;                         // four rounds of two workgroups per CU
-  GemmConfig mid = make_rows_config<T, 2, 2, 2, 2, 2>();       // 128 x 128
+  GemmConfig mid = make_rows_config<T, 2, 2, 2, 2>();       // 128 x 128
   if (blocks(mid) >= 512 || always) return mid;
   return GemmConfig{nullptr, 0, 0, 0, 0, 0};
 }
