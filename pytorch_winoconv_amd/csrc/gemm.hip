@@ -621,6 +621,11 @@ static GemmConfig choose_shifted(int T_, int P, int K) {
 template <typename T>
 static GemmConfig choose_rows(int T_, int P, int K, bool always) {
   auto blocks = [&](const GemmConfig& c) { return (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_; };
+  if (K <= 64 && !always) {
+    GemmConfig tall = make_rows_config<T, 4, 1, 2, 2>();       // 256 x 64
+    if (blocks(tall) >= 512) return tall;
+    return GemmConfig{nullptr, 0, 0, 0, 0, 0};
+  }
   GemmConfig big = make_rows_config<T, 4, 2, 2, 2>();       // 256 x 128
   if (blocks(big) >= 2048 && !always) return big;                         // four rounds of two workgroups per CU
   GemmConfig mid = make_rows_config<T, 2, 2, 2, 2>();       // 128 x 128
@@ -645,7 +650,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   // to reach it with small shapes).
   const char* rows_env = std::getenv("WINOCONV_GEMM_ROWS");
   const int rows_mode = rows_env ? std::atoi(rows_env) : 1;
-  bool rows = sh.n_run >= 2 && sh.n_run <= kRunExtra + 1 && rows_mode != 0 && (K > 64 || rows_mode == 2);
+  bool rows = sh.n_run >= 2 && sh.n_run <= kRunExtra + 1 && rows_mode != 0 && (K > 32 || rows_mode == 2);
   if (rows) {
     GemmConfig r = dtype == WC_F16 ? choose_rows<half_t>(T_, P, K, rows_mode == 2) : choose_rows<bf16_t>(T_, P, K, rows_mode == 2);
     if (r.fn) c = r; else rows = false;
