@@ -185,11 +185,14 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     16-bit plans (2-D: 1.15-1.3x for 5x5 and 7x7 kernels; 3-D: 1.05-1.4x; fewer bytes moved); for
     fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
     plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit stride-1
-    kernels of 4 to 8 taps over at most 128 input channels get the plan whose two-tap pieces share
-    one transformed input (2; make_desc then uses output tile 2): 1.2x (5x5), 1.45x (4x4), 1.5x (7x7)
-    faster than stacked F(4,r) pieces at N=32, 128 channels, 112x112, and 1.5x (5x5x5) to 2x (4x4x4,
-    7x7x7) faster than stacked F(2,r) pieces in 3-D; with 256 channels or 9 taps the larger product
-    costs more than the smaller V saves.  Where the caller accepts tile 4 (fp16, 2-D, 5 to 10 taps, at
+    kernels of 4 to 10 taps over at most 256 input channels (3-D: 4 to 8 taps over at most 128, or
+    4 taps over at most 256) get the plan whose two-tap pieces share one transformed input (2;
+    make_desc then uses output tile 2).  Against stacked F(2,r) pieces it measured, in 2-D, 1.7x
+    (4x4, 7x7), 1.5x (5x5) and 1.15x (9x9) faster at N=16, 256 channels, 56x56, 1.9x (9x9) and 3x
+    (10x10) at N=32, 128 channels, 112x112, and the same speed at 512 channels; in 3-D 1.5x (5x5x5)
+    to 2x (4x4x4, 7x7x7) with 64 and 128 channels, 1.5x (4x4x4) and 0.9x (5x5x5) with 256.  It is
+    also 1.2x (5x5), 1.45x (4x4) and 1.6x (7x7) faster than stacked F(4,r) pieces at N=32, 128
+    channels, 112x112.  Where the caller accepts tile 4 (fp16, 2-D, 5 to 10 taps, at
     least 3 on the other axis, at most 256 channels) the shared tile is F(3,3) with the reference's
     three-tap pieces (make_desc: output tile 3): 1.4x (5x5) to 1.8x (7x7, 9x9) faster than stacked
     F(4,r) pieces, also at 256 channels."""
@@ -204,7 +207,10 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
             ks = [int(k) for k in w_shape[2:]]
             cp = (int(w_shape[1]) + 31) // 32 * 32
             tile3 = dtype == torch.float16 and nd == 2 and m == 4 and min(ks) >= 3 and 5 <= max(ks) <= 10 and cp <= 256
-            tile2 = 4 <= max(ks) <= 8 and cp <= 128
+            if nd == 2:
+                tile2 = 4 <= max(ks) <= 10 and cp <= 256
+            else:
+                tile2 = (4 <= max(ks) <= 8 and cp <= 128) or (max(ks) == 4 and cp <= 256)
             if tile3 or tile2:
                 return 2
         return True

@@ -284,10 +284,12 @@ def test_shared_input_plans():
     s = engine._stack
     assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 1, 4) == 2 and s(None, torch.bfloat16, 2, False, (8, 100, 4, 8), 1, 2) == 2
     assert s(None, torch.float16, 2, False, (128, 128, 5, 5), 2, 4) is True        # stride 2
-    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 2) is True        # more than 128 channels with tile 2
+    assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 2) == 2 and s(None, torch.float16, 2, False, (128, 300, 5, 5), 1, 2) is True
     assert s(None, torch.float16, 2, False, (128, 160, 5, 5), 1, 4) == 2 and s(None, torch.float16, 2, False, (128, 300, 5, 5), 1, 4) is True
-    assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 2) is True and s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) == 2
-    assert s(None, torch.bfloat16, 2, False, (128, 128, 9, 9), 1, 4) is True and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
+    assert s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 2) == 2 and s(None, torch.float16, 2, False, (128, 128, 9, 9), 1, 4) == 2
+    assert s(None, torch.float16, 2, False, (128, 128, 11, 3), 1, 2) is True
+    assert s(None, torch.float16, 3, False, (8, 160, 5, 5, 5), 1, 2) is True and s(None, torch.float16, 3, False, (8, 160, 4, 4, 4), 1, 2) == 2
+    assert s(None, torch.bfloat16, 2, False, (128, 128, 9, 9), 1, 4) == 2 and s(None, torch.float16, 2, False, (8, 8, 3, 3), 1, 4) is True
     assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) == 2
     assert s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 2) is True and s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 4) is False
     assert s(2, torch.float32, 2, False) == 2 and s(True, torch.float16, 2, False) is True and s(False, torch.float16, 2, False) is False
