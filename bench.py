@@ -76,7 +76,8 @@ SUITE = [
     # c3, 64 and 128 channels: the default is the fused F(2,3) kernel; the three-kernel F(4,3) line stands beside it.
     # c4: the 16-bit default adds the DWM pieces in the batched GEMM; at stride 1 the pieces share one
     # transformed input (tile 3 / F(3,3) with the reference's three-tap pieces where the caller asks for tile 4,
-    # tile 2 / F(2,2) with two-tap pieces where it asks for 2), else each has its own ("stacked"); two lines with
+    # tile 2 / F(2,2) with two-tap pieces where it asks for 2; 7x7 at stride 2: F(2,2) on the parity phases of x),
+    # else each has its own ("stacked"); two lines with
     # the reference's structure (pieces added after their output transforms) stand beside them.
     ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
     ("c2 vgg16 fp32 N8 F(2,3) x13 (first layer: one fused kernel)", "vgg", None, 1, 1, 2, "f32"),
@@ -97,8 +98,9 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM shared input F(2,2) on the parity phases", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-stacked"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),

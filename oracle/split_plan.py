@@ -87,6 +87,10 @@ def conv_pieces(kernel, stride=1, m=2, degenerate_depth=False, whole_kernel=Fals
     if whole_kernel:
         assert stride == 1
         per_axis = [[(0, 1, k)] for k in kernel]
+    elif pairs and stride == 2:
+        # parity phases first (as axis_pieces does), then pairs of a phase's taps: (q + 2 s, 2, <= 2 taps)
+        per_axis = [[(q + 2 * s, 2, min(2, (k - q + 1) // 2 - s))
+                     for q in range(min(2, k)) for s in range(0, (k - q + 1) // 2, 2)] for k in kernel]
     elif pairs:
         assert stride == 1
         per_axis = [axis_pairs(k, m if isinstance(m, int) else 2) for k in kernel]

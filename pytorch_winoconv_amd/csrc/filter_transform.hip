@@ -227,7 +227,8 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   stacked_taps(plan, a.rp);
   bool small_taps = true;
   for (int i = 0; i < plan->n_pieces; ++i)
-    for (int q = 0; q < 3; ++q) small_taps = small_taps && plan->piece[i].r[q] >= 1 && plan->piece[i].r[q] <= 3;
+    for (int q = 0; q < 3; ++q)     // a stacked plan may hold pieces without taps (r = 0): their block of U is zero
+      small_taps = small_taps && plan->piece[i].r[q] >= (a.stacked ? 0 : 1) && plan->piece[i].r[q] <= 3;
   const bool flat = plan->m[0] == 1;
   const int mo = plan->m[1];
   if (small_taps && plan->m[2] == mo && (flat ? (mo == 2 || mo == 4 || (mo == 3 && a.stacked)) : (mo == 2 && plan->m[0] == 2))) {

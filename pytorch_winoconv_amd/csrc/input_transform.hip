@@ -55,10 +55,18 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
       default: break;
     }
     if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for the shared tile (%d, %d, %d taps) not built", rp[0], rp[1], rp[2]);
-    a.base0 = -d->pad[0]; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
     a.t_offset = 0;
-    hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
-    WC_CHECK_LAUNCH("input_transform_kernel");
+    // stride 2: one launch per parity phase, each into its own columns of V
+    const int n0 = shared_phases(d, 0), n1 = shared_phases(d, 1), n2 = shared_phases(d, 2);
+    for (int q0 = 0; q0 < n0; ++q0)
+      for (int q1 = 0; q1 < n1; ++q1)
+        for (int q2 = 0; q2 < n2; ++q2) {
+          const int ph = (q0 * n1 + q1) * n2 + q2;
+          a.base0 = q0 - d->pad[0]; a.base1 = q1 - d->pad[1]; a.base2 = q2 - d->pad[2];
+          a.V = static_cast<char*>(V) + (long long)ph * Cp * (d->dtype == WC_F32 ? 4 : 2);
+          hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
+          WC_CHECK_LAUNCH("input_transform_kernel");
+        }
     return WC_OK;
   }
   // 2-D DWM plans: all pieces in one launch

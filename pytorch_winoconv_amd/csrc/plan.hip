@@ -136,8 +136,8 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
     return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
-  if (d->stacked == 2 && (d->stride != 1 || (d->m != 2 && d->m != 3)))
-    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need stride 1 and output tile 2 or 3");
+  if (d->stacked == 2 && d->m != 2 && !(d->m == 3 && d->stride == 1))
+    return fail(WC_ERR_UNSUPPORTED, "plans with a shared transformed input need output tile 2, or 3 at stride 1");
   if (d->stacked == 2 && d->m == 3 &&
       (d->ndim != 2 || d->kernel[1] < 3 || d->kernel[2] < 3 || (d->kernel[1] == 3 && d->kernel[2] == 3)))
     return fail(WC_ERR_UNSUPPORTED, "output tile 3 is built for 2-D kernels of at least 3 taps per axis and more than 3 on one");
@@ -151,10 +151,62 @@ static int check_desc(const wc_conv_desc* d) {
   return WC_OK;
 }
 
+// Stride 2 with a shared transformed input (see shared_phases in wc_common.h): positions of two
+// phase taps per axis, depth outermost; inside a position the 2^d parity phases, depth parity
+// outermost.  Piece (position, phase) owns the taps q + 2 j, j in [2 pos, 2 pos + 2) that the
+// kernel has; a phase that runs out of taps before the others leaves pieces without any (r = 0:
+// their block of U is zero).  All pieces use the tile F(2, 2) (F(2, 1) on an axis of one or two taps).
+static int plan_shared_stride2(const wc_conv_desc* d, wc_plan* plan) {
+  int npos[3], nq[3];
+  for (int a = 0; a < 3; ++a) {
+    nq[a] = shared_phases(d, a);
+    npos[a] = (shared_taps(d, a) + 1) / 2;
+  }
+  const int np_total = npos[0] * npos[1] * npos[2] * nq[0] * nq[1] * nq[2];
+  if (np_total > WC_MAX_PIECES) return fail(WC_ERR_UNSUPPORTED, "%d pieces exceed %d", np_total, WC_MAX_PIECES);
+  std::memset(plan, 0, sizeof(*plan));
+  plan->tap_step = 2;
+  const bool flat_depth = (d->in[0] == 1 && d->kernel[0] == 1 && d->pad[0] == 0);
+  plan->m[0] = flat_depth ? 1 : 2;
+  plan->m[1] = plan->m[2] = 2;
+  int np = 0;
+  int pos[3], q[3];
+  for (pos[0] = 0; pos[0] < npos[0]; ++pos[0])
+    for (pos[1] = 0; pos[1] < npos[1]; ++pos[1])
+      for (pos[2] = 0; pos[2] < npos[2]; ++pos[2])
+        for (q[0] = 0; q[0] < nq[0]; ++q[0])
+          for (q[1] = 0; q[1] < nq[1]; ++q[1])
+            for (q[2] = 0; q[2] < nq[2]; ++q[2]) {
+              wc_piece& p = plan->piece[np++];
+              bool empty = false;
+              for (int a = 0; a < 3; ++a) {
+                const int taps = (d->kernel[a] - q[a] + 1) / 2;     // taps of this parity
+                int r = taps - 2 * pos[a];
+                r = r < 0 ? 0 : (r > 2 ? 2 : r);
+                p.r[a] = r;
+                p.tap0[a] = q[a] + 4 * pos[a];
+                empty = empty || r == 0;
+              }
+              if (empty)
+                for (int a = 0; a < 3; ++a) { p.r[a] = 0; p.tap0[a] = 0; }
+              p.t_offset = 0;
+            }
+  plan->n_pieces = np;
+  int t = 1;
+  for (int a = 0; a < 3; ++a) {
+    const int rp = shared_taps(d, a) >= 2 ? 2 : 1;
+    if (kind_of(plan->m[a], rp) < 0) return fail(WC_ERR_UNSUPPORTED, "F(%d,%d) not implemented", plan->m[a], rp);
+    t *= plan->m[a] + rp - 1;
+  }
+  plan->t_total = t;
+  return WC_OK;
+}
+
 int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   int rc = check_desc(d);
   if (rc) return rc;
   WC_CHECK_ARG(plan != nullptr, "wc_plan_conv: null plan");
+  if (d->stacked == 2 && d->stride == 2) return plan_shared_stride2(d, plan);
   AxisPiece ax[3][8];
   int n[3];
   for (int a = 0; a < 3; ++a) {
@@ -214,7 +266,7 @@ int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
     int m = a == 0 ? (flat_depth ? 1 : (d->m == 4 ? 2 : d->m)) : d->m;
     grid[a] = (out[a] + m - 1) / m;
     // a shared transformed input covers the tiles that the pieces reach beyond the output's own
-    if (d->stacked == 2) grid[a] += (d->kernel[a] + m - 1) / m - 1;
+    if (d->stacked == 2) grid[a] += (shared_taps(d, a) + m - 1) / m - 1;
   }
   return WC_OK;
 }

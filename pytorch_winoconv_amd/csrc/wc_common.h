@@ -78,9 +78,18 @@ inline int stacked_row(const wc_conv_desc* d, const wc_plan* plan) {
 // extended by the largest shifts (wc_conv_out_dims reports that grid), followed by `tail` rows that
 // only the products of the extension tiles read; the batched GEMM reads piece (a, b) of tile row p
 // at row p + a * grid_w + b (3-D: the depth axis likewise, whole planes of the grid further on).
+// At stride 2 the taps of each axis are first separated by parity (y[o] = sum_q sum_j x[2 (o + j) + q - pad] w[2 j + q]):
+// the even and the odd samples of x are the "phases" of a stride-1 problem whose kernel has ceil(k / 2) taps per
+// axis and 2^d times the channels.  A row of V then holds the phases side by side (depth parity outermost), and
+// the pieces are (position, phase) pairs, the phases of one position next to each other along the rows of U.
 inline bool shared_input(const wc_conv_desc* d, const wc_plan* plan) { return d->stacked == 2 && plan->n_pieces > 1; }
+inline int shared_taps(const wc_conv_desc* d, int axis) {
+  return d->stride == 2 ? (d->kernel[axis] + 1) / 2 : d->kernel[axis];
+}
+inline int shared_phases(const wc_conv_desc* d, int axis) { return d->stride == 2 && d->kernel[axis] >= 2 ? 2 : 1; }
+inline int shared_phases(const wc_conv_desc* d) { return shared_phases(d, 0) * shared_phases(d, 1) * shared_phases(d, 2); }
 inline int v_row(const wc_conv_desc* d, const wc_plan* plan) {
-  return shared_input(d, plan) ? wc_padded_channels(d->C) : stacked_row(d, plan);
+  return shared_input(d, plan) ? wc_padded_channels(d->C) * shared_phases(d) : stacked_row(d, plan);
 }
 struct SharedShift {          // pieces (a, b, c) of the depth, height and width axes; tiles (d, h, w) of the extended grid
   int n_run, n_runs, n_planes;  // pieces per axis: width, height, depth
@@ -90,9 +99,9 @@ struct SharedShift {          // pieces (a, b, c) of the depth, height and width
 inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
   SharedShift s;
   const int len = d->m;                           // taps per piece = output tile (3 only in 2-D: one depth piece)
-  s.n_run = (d->kernel[2] + len - 1) / len;
-  s.n_runs = (d->kernel[1] + len - 1) / len;
-  s.n_planes = (d->kernel[0] + len - 1) / len;
+  s.n_run = (shared_taps(d, 2) + len - 1) / len;
+  s.n_runs = (shared_taps(d, 1) + len - 1) / len;
+  s.n_planes = (shared_taps(d, 0) + len - 1) / len;
   s.run_rows = grid[2];
   s.plane_rows = grid[1] * grid[2];
   s.tail = (s.n_planes - 1) * s.plane_rows + (s.n_runs - 1) * s.run_rows + s.n_run - 1;

@@ -74,7 +74,7 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
         # _stack picks that plan for its speed (fp16, 2-D, at least 3 taps per axis and 5 on one; F(3,3):
         # fp16 error 3e-3 of the output range, between F(2,r) and F(4,r); too coarse for bf16), else 2
         ks = d.kernel[1:]
-        d.m = 3 if (nd == 2 and dtype == torch.float16 and min(ks) >= 3 and max(ks) >= 5) else 2
+        d.m = 3 if (nd == 2 and d.stride == 1 and dtype == torch.float16 and min(ks) >= 3 and max(ks) >= 5) else 2
     d.unfused = int(bool(unfused))
     return d
 
@@ -147,9 +147,15 @@ def input_transform(desc, plan, x_cl):
     P = n * grid[0] * grid[1] * grid[2]
     if desc.stacked == 2 and plan.n_pieces > 1:
         # one piece over the extended tile grid, plus the rows the shifted reads of the last tiles reach
-        per = [(k + desc.m - 1) // desc.m for k in desc.kernel]        # pieces per axis
+        # (stride 2: the even and the odd samples of each axis are phases side by side in a row of V,
+        # and the pieces are cut from the ceil(k / 2) taps of a phase)
+        taps = [(k + 1) // 2 if desc.stride == 2 else k for k in desc.kernel]
+        phases = 1
+        for k in desc.kernel:
+            phases *= 2 if (desc.stride == 2 and k >= 2) else 1
+        per = [(t + desc.m - 1) // desc.m for t in taps]               # pieces per axis
         tail = (per[0] - 1) * grid[1] * grid[2] + (per[1] - 1) * grid[2] + per[2] - 1
-        V = torch.zeros(plan.t_total, P + tail, lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
+        V = torch.zeros(plan.t_total, P + tail, phases * lib.wc_padded_channels(desc.C), dtype=x_cl.dtype, device=x_cl.device)
     else:
         V = torch.empty(plan.t_total, P, _row(desc, plan), dtype=x_cl.dtype, device=x_cl.device)
     check(lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(x_cl), n, _ptr(V), _stream(x_cl)))
@@ -195,7 +201,11 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     channels, 112x112.  Where the caller accepts tile 4 (fp16, 2-D, 5 to 10 taps, at
     least 3 on the other axis, at most 256 channels) the shared tile is F(3,3) with the reference's
     three-tap pieces (make_desc: output tile 3): 1.4x (5x5) to 1.8x (7x7, 9x9) faster than stacked
-    F(4,r) pieces, also at 256 channels."""
+    F(4,r) pieces, also at 256 channels.  At stride 2 the shared-input plan works on the parity phases
+    of x (four times the channels, half the taps) and pays where a phase has four taps: 7x7 and 8x8
+    kernels, 2-D, at most 128 channels: 1.15x (128 channels) to 1.55x (64, and 3 -> 64 at 224x224)
+    faster than stacked F(4,r) pieces and as accurate as F(2,r); kernels of 5 or 6 taps (three per
+    phase: pieces without taps) are 1.8x slower that way and keep their stacked pieces."""
     if stacked is not None:
         return 2 if stacked == 2 else bool(stacked)
     if whole_kernel or (nd == 3 and m != 2):
@@ -203,6 +213,10 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
     if dtype != torch.float32:
+        if stride == 2 and nd == 2 and w_shape is not None:
+            # four taps per parity phase (7 or 8 taps) cut into two full pieces per axis
+            if all((int(k) + 1) // 2 == 4 for k in w_shape[2:]) and int(w_shape[1]) <= 128:
+                return 2
         if stride == 1 and w_shape is not None:
             ks = [int(k) for k in w_shape[2:]]
             cp = (int(w_shape[1]) + 31) // 32 * 32

@@ -251,9 +251,6 @@ def test_shared_input_plans():
     # one piece per axis: nothing is extended
     d1 = engine.make_desc((2, 8, 20, 21), (4, 8, 2, 1), torch.float16, 1, 0, 2, stacked=2)
     assert engine.plan_conv(d1).n_pieces == 1 and engine.out_dims(d1)[1] == [1, 10, 11]
-    bad = engine.make_desc((2, 8, 20, 21), (4, 8, 5, 5), torch.float16, 2, 2, 2, stacked=2)      # stride 2
-    with pytest.raises(NotImplementedError):
-        engine.plan_conv(bad)
     # 3-D: pieces depth-major, the grid extended on all three axes
     d3 = engine.make_desc((1, 8, 9, 20, 20), (4, 8, 3, 5, 4), torch.float16, 1, (1, 2, 1), 2, stacked=2)
     p3 = engine.plan_conv(d3)
@@ -293,6 +290,41 @@ def test_shared_input_plans():
     assert s(None, torch.float32, 2, False, (128, 128, 5, 5), 1, 4) is True and s(None, torch.float16, 3, False, (8, 8, 5, 5, 5), 1, 2) == 2
     assert s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 2) is True and s(None, torch.float16, 3, False, (8, 8, 3, 3, 3), 1, 4) is False
     assert s(2, torch.float32, 2, False) == 2 and s(True, torch.float16, 2, False) is True and s(False, torch.float16, 2, False) is False
+
+
+def test_shared_input_plans_at_stride_2():
+    """Stride 2: positions of two phase taps per axis, inside a position the parity phases; a piece owns
+    the taps q + 2 j (j = 2 pos, 2 pos + 1) that exist, pieces past a phase's last tap have none.  Every tap
+    of the kernel is owned once; the grid grows by the positions beyond the first."""
+    from pytorch_winoconv_amd import engine
+    for kh, kw in ((7, 7), (5, 5), (3, 3), (8, 4), (2, 1), (10, 9)):
+        d = engine.make_desc((2, 8, 30, 31), (4, 8, kh, kw), torch.float16, 2, (kh // 2, kw // 2), 2, stacked=2)
+        plan = engine.plan_conv(d)
+        ph = [2 if k >= 2 else 1 for k in (kh, kw)]
+        pos = [((k + 1) // 2 + 1) // 2 for k in (kh, kw)]
+        assert plan.n_pieces == ph[0] * ph[1] * pos[0] * pos[1] and plan.tap_step == 2
+        owned = []
+        for i in range(plan.n_pieces):
+            pc = plan.piece[i]
+            rest, q = divmod(i, ph[0] * ph[1])
+            qh, qw = divmod(q, ph[1])
+            a, b = divmod(rest, pos[1])
+            if pc.r[1] and pc.r[2]:
+                assert (pc.tap0[1], pc.tap0[2]) == (qh + 4 * a, qw + 4 * b) and pc.r[0] == 1
+            else:
+                assert tuple(pc.r) == (0, 0, 0)
+            owned += [(pc.tap0[1] + 2 * i1, pc.tap0[2] + 2 * i2) for i1 in range(pc.r[1]) for i2 in range(pc.r[2])]
+        assert sorted(owned) == [(i1, i2) for i1 in range(kh) for i2 in range(kw)]
+        out, grid = engine.out_dims(d)
+        oh, ow_ = (30 + 2 * (kh // 2) - kh) // 2 + 1, (31 + 2 * (kw // 2) - kw) // 2 + 1
+        assert out == [1, oh, ow_] and grid == [1, (oh + 1) // 2 + pos[0] - 1, (ow_ + 1) // 2 + pos[1] - 1]
+    bad = engine.make_desc((2, 8, 30, 31), (4, 8, 7, 7), torch.float16, 2, 3, 3, stacked=2)      # tile 3 is for stride 1
+    with pytest.raises(NotImplementedError):
+        engine.plan_conv(bad)
+    s = engine._stack
+    assert s(None, torch.float16, 2, False, (64, 64, 7, 7), 2, 4) == 2 and s(None, torch.bfloat16, 2, False, (64, 3, 8, 7), 2, 2) == 2
+    assert s(None, torch.float16, 2, False, (64, 64, 5, 5), 2, 4) is True and s(None, torch.float16, 2, False, (64, 160, 7, 7), 2, 4) is True
+    assert s(None, torch.float16, 3, False, (64, 64, 7, 7, 7), 2, 2) is True and s(None, torch.float32, 2, False, (64, 64, 7, 7), 2, 2) is False
 
 
 def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():

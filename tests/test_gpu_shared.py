@@ -224,6 +224,71 @@ def test_random_shapes_with_one_operand_tile_per_run(dev, case, monkeypatch):
     test_random_shapes(dev, case)
 
 
+STRIDE2 = [
+    # x shape, w shape, pad
+    ((2, 8, 20, 21), (4, 8, 7, 7), 3), ((1, 5, 9, 12), (3, 5, 3, 3), 1), ((2, 16, 17, 14), (8, 16, 5, 4), (2, 1)),
+    ((1, 8, 11, 13), (6, 8, 2, 1), 0), ((1, 40, 31, 30), (33, 40, 8, 7), (4, 3)), ((2, 24, 23, 25), (8, 24, 10, 9), 4),
+    ((1, 8, 9, 10, 11), (4, 8, 3, 5, 3), 1), ((1, 4, 7, 9, 8), (5, 4, 4, 4, 4), (2, 1, 2)), ((1, 64, 33, 35), (72, 64, 7, 7), 3),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", STRIDE2)
+def test_stride_2_on_the_parity_phases(dev, dtype, case, monkeypatch):
+    """Stride 2 with a shared transformed input: the even and the odd samples of x are phases side
+    by side in the rows of V, the pieces are pairs of a phase's taps.  Against fp64 convolution and
+    against the CPU oracle's restatement (pieces with their own V) in the same storage type; once
+    more through the product kernel that serves a run of pieces from one operand tile."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(*xs, generator=g).to(dtype)
+    fan = ws[1]
+    for k in ws[2:]:
+        fan *= k
+    w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    conv = F.conv2d if len(xs) == 4 else F.conv3d
+    ref = conv(x.double(), w.double(), b.double(), 2, pad)
+    y = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 2, pad, 2, stacked=2)
+    assert tuple(y.shape) == tuple(ref.shape) and _rel(y, ref) <= 2e-2
+    yo = ow.dwm_conv(x, w, b, 2, pad, 2, "fp16" if dtype == torch.float16 else "bf16", stacked=2)
+    assert _rel(y, yo.double()) <= (3e-3 if dtype == torch.float16 else 2e-2)
+    U = engine.transform_filter(w.to(dev), xs, 2, pad, 2, stacked=2)
+    assert torch.equal(engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 2, pad, 2, U=U, stacked=2), y)
+    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+    y2 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 2, pad, 2, stacked=2)
+    assert _rel(y2, ref) <= 2e-2 and _rel(y2, y.double().cpu()) <= (3e-3 if dtype == torch.float16 else 2e-2)
+
+
+@pytest.mark.parametrize("case", [c for c in STRIDE2 if c[0][1] <= 16])
+def test_stride_2_is_exact_on_small_integers(dev, case):
+    """x in -3..3, taps multiples of 4 (8 in 3-D): every U, V and product is an integer; with at most 16
+    channels in each of the 4 (8) phases the sums stay below 2048, exact in fp16."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(4)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = (4.0 if len(ws) == 4 else 8.0) * torch.randint(-1, 2, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    conv = F.conv2d if len(xs) == 4 else F.conv3d
+    ref = conv(x, w, b, 2, pad)
+    y = engine.conv_forward(x.half().to(dev), w.half().to(dev), b.half().to(dev), 2, pad, 2, stacked=2)
+    assert float(ref.abs().max()) < 2048
+    assert torch.equal(y.cpu(), ref.half())
+
+
+def test_c4_stride_2_layer_at_full_size(dev):
+    """BASELINE configuration c4, 7x7 stride 2 (fp16, N=32, 128 channels, 112x112): the default plan is
+    the shared-input one; checked against torch's own GPU convolution accumulated in fp32."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(32, 128, 112, 112, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    w = (torch.randn(128, 128, 7, 7, generator=g) * (2.0 / (128 * 49)) ** 0.5).half().to(dev)
+    assert engine._stack(None, torch.float16, 2, False, w.shape, 2, 4) == 2
+    y = engine.conv_forward(x, w, None, 2, 3, 4)
+    ref = F.conv2d(x.float(), w.float(), None, 2, 3)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert float((y.float() - ref).abs().max() / ref.abs().max()) <= 2e-2
+
+
 def _bad_tile_4(xs, ws):
     d = engine.make_desc(xs, ws, torch.float16, 1, 1, 2, stacked=2)
     d.m = 4
@@ -234,7 +299,7 @@ def test_what_the_plan_is_not_built_for(dev):
     x = torch.randn(2, 8, 12, 12).half().to(dev)
     w = torch.randn(4, 8, 5, 5).half().to(dev)
     with pytest.raises(NotImplementedError):
-        engine.conv_forward(x, w, None, 2, 2, 2, stacked=2)                        # stride 2
+        engine.conv_forward(x, w, None, 2, 2, 3, stacked=2)                        # tile 3 at stride 2
     with pytest.raises(NotImplementedError):
         engine.conv_forward(x.float(), w.float(), None, 1, 2, 2, stacked=2)        # fp32 product
     x3, w3 = torch.randn(1, 8, 6, 12, 12).half().to(dev), torch.randn(4, 8, 3, 3, 3).half().to(dev)

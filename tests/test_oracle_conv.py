@@ -163,3 +163,30 @@ def test_pair_pieces_give_the_same_convolution(case):
     wi = (torch.randint(-2, 3, ws, generator=g) * 8).float()
     yi = ow.dwm_conv(xi, wi, None, 1, p, 2, "fp32", stacked=2)
     assert torch.equal(yi.double(), _conv(xi.double(), wi.double(), None, 1, p))
+
+
+@pytest.mark.parametrize("case", [
+    ((2, 3, 13, 12), (4, 3, 7, 7), 3), ((1, 2, 12, 11), (3, 2, 5, 4), (2, 1)), ((1, 3, 9, 9), (2, 3, 3, 3), 1),
+    ((1, 2, 15, 9), (2, 2, 8, 2), (4, 0)), ((1, 2, 8, 9, 7), (3, 2, 3, 5, 2), 1), ((1, 2, 9, 10), (2, 2, 1, 6), (0, 2)),
+])
+def test_pair_pieces_of_the_parity_phases_give_the_stride_2_convolution(case):
+    """Stride 2 with two-tap pieces: the taps of an axis are separated by parity, then each parity's
+    taps are cut into pairs.  Together the pieces own every tap once, their tap step is 2, and the
+    stacked sum over them is the strided convolution: in fp64, and exactly on small integers in fp32."""
+    from oracle import split_plan as sp
+    xs, ws, p = case
+    for k in range(1, 11):
+        pieces, _ = sp.conv_pieces([1, 1, k], stride=2, m=2, degenerate_depth=True, pairs=True)
+        taps = sorted(pc["axes"][2][0] + 2 * j for pc in pieces for j in range(pc["axes"][2][2]))
+        assert taps == list(range(k)) and all(pc["axes"][2][1] == 2 and 1 <= pc["axes"][2][2] <= 2 for pc in pieces)
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(*xs, dtype=torch.float64, generator=g)
+    w = torch.randn(*ws, dtype=torch.float64, generator=g)
+    b = torch.randn(ws[0], dtype=torch.float64, generator=g)
+    y = ow.dwm_conv(x, w, b, 2, p, 2, "fp64", stacked=2)
+    ref = _conv(x, w, b, 2, p)
+    assert y.shape == ref.shape and float((y - ref).abs().max() / ref.abs().max()) < 1e-12
+    xi = torch.randint(-3, 4, xs, generator=g).float()
+    wi = (torch.randint(-2, 3, ws, generator=g) * 8).float()
+    yi = ow.dwm_conv(xi, wi, None, 2, p, 2, "fp32", stacked=2)
+    assert torch.equal(yi.double(), _conv(xi.double(), wi.double(), None, 2, p))
