@@ -41,6 +41,7 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   const long long blocks = ceil_div_ll(a.total, 256);
   a.per_xcd = (int)ceil_div_ll(blocks, kXcds);
   a.x_bytes = 0;
+  a.nq1 = a.nq2 = 1; a.q_cols = 0;
   WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "wc_input_transform: problem too large");
   const dim3 launch_grid((unsigned)(a.per_xcd * kXcds));
 
@@ -56,17 +57,12 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
     }
     if (!fn) return fail(WC_ERR_UNSUPPORTED, "input transform for the shared tile (%d, %d, %d taps) not built", rp[0], rp[1], rp[2]);
     a.t_offset = 0;
-    // stride 2: one launch per parity phase, each into its own columns of V
+    // stride 2: the parity phases are the second grid dimension, each writes its own columns of V
     const int n0 = shared_phases(d, 0), n1 = shared_phases(d, 1), n2 = shared_phases(d, 2);
-    for (int q0 = 0; q0 < n0; ++q0)
-      for (int q1 = 0; q1 < n1; ++q1)
-        for (int q2 = 0; q2 < n2; ++q2) {
-          const int ph = (q0 * n1 + q1) * n2 + q2;
-          a.base0 = q0 - d->pad[0]; a.base1 = q1 - d->pad[1]; a.base2 = q2 - d->pad[2];
-          a.V = static_cast<char*>(V) + (long long)ph * Cp * (d->dtype == WC_F32 ? 4 : 2);
-          hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
-          WC_CHECK_LAUNCH("input_transform_kernel");
-        }
+    a.base0 = -d->pad[0]; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
+    a.nq1 = n1; a.nq2 = n2; a.q_cols = Cp;
+    hipLaunchKernelGGL(fn, dim3(launch_grid.x, (unsigned)(n0 * n1 * n2)), dim3(256), 0, as_stream(stream), a);
+    WC_CHECK_LAUNCH("input_transform_kernel");
     return WC_OK;
   }
   // 2-D DWM plans: all pieces in one launch

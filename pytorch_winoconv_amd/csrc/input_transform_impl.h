@@ -29,6 +29,10 @@ struct InArgs {
   long long total;           // P * n_cvec
   int per_xcd;
   int x_bytes;               // bytes of the images one launch covers (kernels that read x through a buffer descriptor)
+  // input_transform_kernel only: blockIdx.y enumerates the parity phases of a stride-2 plan whose
+  // pieces share one transformed input (depth parity outermost; 1, 1, 0 otherwise): phase
+  // (q0, q1, q2) reads from base + q and writes its own q_cols columns of a row of V
+  int nq1, nq2, q_cols;
 };
 
 // Tile coordinates and channel offset of one thread
@@ -109,7 +113,9 @@ template <typename T, int K0, int K1, int K2, int VEC>
 __global__ __launch_bounds__(256) void input_transform_kernel(InArgs a) {
   InWhere w;
   if (!in_decode(a, xcd_remap(blockIdx.x, a.per_xcd), VEC, w)) return;
-  transform_window<T, K0, K1, K2, VEC>(a, w, a.base0, a.base1, a.base2, a.t_offset);
+  const int ph = blockIdx.y;
+  const int q2 = ph % a.nq2, q1 = (ph / a.nq2) % a.nq1, q0 = ph / (a.nq2 * a.nq1);
+  transform_window<T, K0, K1, K2, VEC>(a, w, a.base0 + q0, a.base1 + q1, a.base2 + q2, a.t_offset, ph * a.q_cols);
 }
 
 // All pieces of a 2-D DWM plan in one launch: a thread transforms the windows of its tile piece
