@@ -203,9 +203,12 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     three-tap pieces (make_desc: output tile 3): 1.4x (5x5) to 1.8x (7x7, 9x9) faster than stacked
     F(4,r) pieces, also at 256 channels.  At stride 2 the shared-input plan works on the parity phases
     of x (four times the channels, half the taps) and pays where a phase has four taps: 7x7 and 8x8
-    kernels, 2-D, at most 128 channels: 1.15x (128 channels) to 1.55x (64, and 3 -> 64 at 224x224)
-    faster than stacked F(4,r) pieces and as accurate as F(2,r); kernels of 5 or 6 taps (three per
-    phase: pieces without taps) are 1.8x slower that way and keep their stacked pieces."""
+    kernels, 2-D, at most 256 channels: 1.2x (7x7, 128 channels), 1.45-1.6x (64 channels, and 3 -> 64
+    at 224x224) and 1.75x (8x8) faster than stacked F(4,r) pieces and as accurate as F(2,r) (equal
+    speed at 256 channels, slower at 512); kernels of 5 or 6 taps (three per phase: pieces without
+    taps) are 1.8x slower that way and keep their stacked pieces.  In 3-D (two or four taps per
+    phase on every axis, at most 128 channels): 4x4x4 1.75x, 7x7x7 2.5x (64 channels) and 1.65x (128)
+    faster than stacked F(2,r) pieces at N=4, 16x28x28."""
     if stacked is not None:
         return 2 if stacked == 2 else bool(stacked)
     if whole_kernel or (nd == 3 and m != 2):
@@ -213,9 +216,11 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
     if dtype != torch.float32:
-        if stride == 2 and nd == 2 and w_shape is not None:
-            # four taps per parity phase (7 or 8 taps) cut into two full pieces per axis
-            if all((int(k) + 1) // 2 == 4 for k in w_shape[2:]) and int(w_shape[1]) <= 128:
+        if stride == 2 and w_shape is not None:
+            taps = [(int(k) + 1) // 2 for k in w_shape[2:]]      # per parity phase
+            if nd == 2 and all(t == 4 for t in taps) and int(w_shape[1]) <= 256:
+                return 2
+            if nd == 3 and all(t in (2, 4) for t in taps) and max(int(k) for k in w_shape[2:]) >= 4 and int(w_shape[1]) <= 128:
                 return 2
         if stride == 1 and w_shape is not None:
             ks = [int(k) for k in w_shape[2:]]

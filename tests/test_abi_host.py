@@ -323,8 +323,8 @@ def test_shared_input_plans_at_stride_2():
         engine.plan_conv(bad)
     s = engine._stack
     assert s(None, torch.float16, 2, False, (64, 64, 7, 7), 2, 4) == 2 and s(None, torch.bfloat16, 2, False, (64, 3, 8, 7), 2, 2) == 2
-    assert s(None, torch.float16, 2, False, (64, 64, 5, 5), 2, 4) is True and s(None, torch.float16, 2, False, (64, 160, 7, 7), 2, 4) is True
-    assert s(None, torch.float16, 3, False, (64, 64, 7, 7, 7), 2, 2) is True and s(None, torch.float32, 2, False, (64, 64, 7, 7), 2, 2) is False
+    assert s(None, torch.float16, 2, False, (64, 64, 5, 5), 2, 4) is True and s(None, torch.float16, 2, False, (64, 300, 7, 7), 2, 4) is True
+    assert s(None, torch.float16, 3, False, (64, 64, 7, 7, 7), 2, 2) == 2 and s(None, torch.float16, 3, False, (64, 64, 3, 3, 3), 2, 2) is True and s(None, torch.float32, 2, False, (64, 64, 7, 7), 2, 2) is False
 
 
 def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
