@@ -289,6 +289,26 @@ def test_c4_stride_2_layer_at_full_size(dev):
     assert float((y.float() - ref).abs().max() / ref.abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("nd,cin,cout,k,sp", [(2, 16, 24, 7, (37, 41)), (3, 8, 16, 7, (13, 12, 15)), (3, 8, 8, 4, (9, 12, 11))])
+def test_modules_train_through_the_stride_2_plan(dev, nd, cin, cout, k, sp):
+    """WinoConv2d / WinoConv3d at stride 2 with the kernel sizes whose default is the shared-input plan:
+    output and all three gradients against fp64 autograd (the weight gradient has no shared-input form
+    and runs on stacked pieces, the input gradient is a stride-1 convolution of the zero-filled dy)."""
+    import pytorch_winoconv_amd as pkg
+    torch.manual_seed(0)
+    mod = (pkg.WinoConv2d if nd == 2 else pkg.WinoConv3d)(cin, cout, k, stride=2, padding=k // 2).to(dev).half()
+    assert engine._stack(None, torch.float16, nd, False, mod.weight.shape, 2, 2) == 2
+    x = torch.randn(2, cin, *sp, device=dev).half().requires_grad_(True)
+    y = mod(x)
+    xr, wr, br = (t.detach().double().requires_grad_(True) for t in (x, mod.weight, mod.bias))
+    yr = (F.conv2d if nd == 2 else F.conv3d)(xr, wr, br, 2, k // 2)
+    gy = torch.randn_like(yr)
+    y.backward(gy.half())
+    yr.backward(gy)
+    for got, want in ((y, yr), (x.grad, xr.grad), (mod.weight.grad, wr.grad), (mod.bias.grad, br.grad)):
+        assert float((got.detach().double() - want.detach()).abs().max() / want.detach().abs().max()) <= 2e-2
+
+
 def _bad_tile_4(xs, ws):
     d = engine.make_desc(xs, ws, torch.float16, 1, 1, 2, stacked=2)
     d.m = 4
