@@ -47,27 +47,48 @@ def synthetic(n):
     return x, w
 
 
+def cpu_model():
+    """Model name of the host CPU as the kernel reports it."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
+
+
 def cpu_baseline(sample_images=32, repeats=3):
-    """CPU restatement of the reference algorithm on `sample_images` images of the workload."""
+    """CPU restatement of the reference algorithm on `sample_images` images of the workload, and
+    torch's own CPU convolution on the same sample (each warmed, then the median of `repeats`)."""
+    import statistics
     import torch
     from oracle import winograd as ow
     x, w = synthetic(sample_images)
-    ow.dwm_conv(x[:1], w, None, 1, PAD, M_TILE, "fp32")          # warm-up
-    best = float("inf")
-    for _ in range(repeats):
-        t0 = time.perf_counter()
-        ow.dwm_conv(x, w, None, 1, PAD, M_TILE, "fp32")
-        best = min(best, time.perf_counter() - t0)
+
+    def timed(fn):
+        fn()                                                     # warm-up
+        ts = []
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts), min(ts)
+
     flops = 2.0 * sample_images * K * C * H * W * R * R
-    t0 = time.perf_counter()
-    torch.nn.functional.conv2d(x, w, padding=PAD)
-    t_direct = time.perf_counter() - t0
+    med, best = timed(lambda: ow.dwm_conv(x, w, None, 1, PAD, M_TILE, "fp32"))
+    d_med, d_best = timed(lambda: torch.nn.functional.conv2d(x, w, padding=PAD))
     return {
-        "value": flops / best / 1e12, "unit": "effective TFLOP/s", "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": "%d of the %d images of the same layer, fp32, oracle.winograd.dwm_conv F(4x4,3x3), "
-                  "best of %d; torch CPU conv2d fp32 on the same sample: %.4f effective TFLOP/s"
-                  % (sample_images, N, repeats, flops / t_direct / 1e12),
+        "value": flops / med / 1e12, "unit": "effective TFLOP/s", "cores": torch.get_num_threads(),
+        "kind": "port", "cpu_model": cpu_model(),
+        "sample": "%d of the %d images of the same layer, fp32, oracle.winograd.dwm_conv F(4x4,3x3), warmed, "
+                  "median of %d" % (sample_images, N, repeats),
+        "best": flops / best / 1e12,
+        "torch_cpu_conv2d": {"value": flops / d_med / 1e12, "best": flops / d_best / 1e12,
+                             "unit": "effective TFLOP/s", "sample": "the same %d images, fp32, warmed, median of %d"
+                                                                    % (sample_images, repeats)},
     }
 
 
@@ -254,6 +275,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--prewarm", type=float, default=0.5, metavar="SECONDS",
+                    help="run untimed steps for this long before the warm-up steps (clocks settle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--suite", action="store_true",
                     help="also time every other benchmark configuration (adds a 'suite' list)")
@@ -321,6 +344,14 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
+    # Untimed steps for a fixed wall time first: a GPU that has been idle needs a few tenths of a second of
+    # work to reach its steady clocks, far more than a handful of 0.25 ms warm-up steps provide.
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < args.prewarm:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+    prewarm_s = time.perf_counter() - t_pre
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -383,7 +414,7 @@ def main():
         "metric": "effective TFLOP/s (direct-conv-equivalent), 3x3 conv fp16 N=64 C=K=256 56x56, 1 MI355X",
         "value": direct_flops / (ms_per_step * 1e-3) / 1e12,
         "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prewarm_s": round(prewarm_s, 3),
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",

@@ -5,9 +5,11 @@
  * Plain pointers, ints and sizes only: no torch, no HIP types (a stream is passed
  * as `void*` holding a hipStream_t; NULL is the default stream).  Every function
  * returns 0 on success or a negative wc_status; wc_last_error() then gives a
- * thread-local message.  No function allocates device memory, synchronises the
- * device or keeps state between calls: work is enqueued on the caller's stream
- * and scratch memory comes from the caller (`workspace`).
+ * thread-local message.  No function allocates device memory or synchronises the
+ * device: work is enqueued on the caller's stream and scratch memory comes from the
+ * caller (`workspace`).  Nothing a call computes depends on earlier calls; the library
+ * only remembers which of its kernels it has already granted more than 64 KB of LDS on
+ * which device (and what the test hook wc_test_gemm_override last set).
  *
  * Data layouts (row-major, innermost last).  "Channel-last" means NHWC / NDHWC.
  *   x   (N, D, H, W, C)        D = 1 for 2-D problems
@@ -32,7 +34,11 @@
 extern "C" {
 #endif
 
-/* storage type of every tensor of a call; arithmetic inside the kernels is always fp32 */
+/* Storage type of every tensor of a call.  Sums and products inside the kernels are fp32 (MFMA
+ * accumulators included), and values are rounded to the storage type once, when V, M and y are
+ * written - with one exception: the one-kernel path of thin fp16 layers (wc_conv_desc.unfused = 0)
+ * transforms its input windows with fp16 adds, the arithmetic type of the reference's own kernels
+ * (src/calculation_kernels.cu:786-806); its bf16 form and everything else add in fp32. */
 typedef enum { WC_F32 = 0, WC_F16 = 1, WC_BF16 = 2 } wc_dtype;
 
 typedef enum {
@@ -107,6 +113,13 @@ const char* wc_version(void);
 /* Replaces the reference's cout + exit(-1) error convention
  * (src/winograd_conv.cpp:80-84,116-126; src/base_conv_launchers.h:384-387). */
 const char* wc_last_error(void);
+
+/* Test hook, no counterpart in the reference: forces tile shape `config` (an index into the
+ * library's list of shapes; -1 = choose by problem size) on wc_batched_gemm, and for plans that
+ * share one transformed input the kernel with one operand tile per piece (rows_mode 0), the
+ * choice by size (1, the default) or one tile per run of pieces wherever the plan has runs (2).
+ * Process-wide; production code never calls it. */
+int wc_test_gemm_override(int config, int rows_mode);
 
 /* ---- planning (host only) --------------------------------------------------------------- */
 /* Stride-1 split plan in the reference's own terms; replaces splitControl()

@@ -43,6 +43,7 @@ _i64_5 = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "wc_version": (ctypes.c_char_p, []),
     "wc_last_error": (ctypes.c_char_p, []),
+    "wc_test_gemm_override": (_i, [_i, _i]),
     "wc_plan_dwm": (_i, [_i, _i, _i, c_int_p] + [c_int_p] * 8),
     "wc_plan_conv": (_i, [_desc_p, _plan_p]),
     "wc_conv_out_dims": (_i, [_desc_p, c_int_p, c_int_p]),

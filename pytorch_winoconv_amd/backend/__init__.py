@@ -121,6 +121,10 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     if algo not in ("dwm", "whole"):
         raise ValueError("winograd_conv: algo must be 'dwm' or 'whole', got %r" % (algo,))
     whole = algo == "whole"
+    if Weight.dim() == 5:
+        if bias is not None and bias.dtype != Input.dtype and bias.dim() == 1 and bias.numel() == Weight.shape[4]:
+            bias = bias.to(Input.dtype)
+        engine.check_operands(Input, int(Weight.shape[4]), bias, U)
     _require_gpu(Input, Weight, Output, bias, U)
     if Input.dim() != 5 or Weight.dim() != 5 or Output.dim() != 5:
         raise ValueError("winograd_conv: expected 5-D channel-last Input/Output and a 5-D Weight")
@@ -138,12 +142,13 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
         padding = (0 if flat else padding, padding, padding)
     w_kc = Weight.permute(4, 3, 0, 1, 2)                 # (K, C, kD, kH, kW) view, no copy
     stacked = engine._stack(stacked, Input.dtype, 2 if flat else 3, whole, (K, C, kH, kW), stride, m)
+    unfused = engine.misaligned(Input, Output, U)        # the one-kernel path of thin layers wants 16-byte alignment
     if flat:
         desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole,
-                         stacked)
+                         stacked, unfused)
     else:
         desc = make_desc((B, C, D, H, W), (K, C, kD, kH, kW), Input.dtype, stride, padding, m, chunk_images, whole,
-                         stacked)
+                         stacked, unfused)
     engine.check_u(desc, U)
     out, _ = out_dims(desc)
     _check_out(Output, (B, out[0], out[1], out[2], K), Input, "winograd_conv")
@@ -152,7 +157,7 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     ws = torch.empty(nbytes.value, dtype=torch.uint8, device=Input.device)
     strides = (ctypes.c_int64 * 5)(*w_kc.stride())
     if bias is not None:
-        bias = bias.to(Input.dtype).contiguous()
+        bias = bias.contiguous()
     _lib.check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(Input), _ptr(w_kc), strides, _ptr(U),
                                    _ptr(bias), _ptr(Output), _ptr(ws), nbytes.value, _stream(Input)))
 

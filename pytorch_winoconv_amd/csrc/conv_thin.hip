@@ -450,8 +450,7 @@ int launch_thin(ThinArgs a, int k_groups, void* stream) {
   // shared among the groups of output channels, in whole multiples of the 8 XCDs
   int wgs = std::min(a.n_blocks, std::max(kXcds, (split ? 256 : 512) / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
-  WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>), lds)) return rc;
   hipLaunchKernelGGL((thin_conv3x3_kernel<T, CP>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups),
                      dim3(split ? 512 : 256), lds, as_stream(stream), a);
   WC_CHECK_LAUNCH("thin_conv3x3_kernel");

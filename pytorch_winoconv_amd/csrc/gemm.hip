@@ -20,7 +20,6 @@
 // with SHIFT walks the operand pointer piece by piece; gemm_rows_kernel serves the pieces of one
 // run (neighbours along the width) from a single operand tile that is n_run - 1 rows taller.
 #include "wc_common.h"
-#include <cstdlib>
 
 namespace wc {
 
@@ -566,11 +565,8 @@ template <> struct Configs<float> {
 // of the best tile on each.
 template <typename T>
 static GemmConfig choose(int T_, int P, int K, int Cp) {
-  const char* force = std::getenv("WINOCONV_GEMM_CONFIG");
-  if (force) {
-    const int i = std::atoi(force);
-    if (i >= 0 && i < Configs<T>::n) return Configs<T>::get(i);
-  }
+  const int force = test_gemm_config();
+  if (force >= 0 && force < Configs<T>::n) return Configs<T>::get(force);
   constexpr int n_auto = 5;
   // fp32 is bound by the MFMA rate: the 64 x 64 tile fills the chip best, except for long
   // reductions with thousands of tiles, where 128 x 128 halves the LDS traffic (measured 5-9 %
@@ -645,11 +641,10 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_shifted: 16-bit types only");
   GemmConfig c = dtype == WC_F16 ? choose_shifted<half_t>(T_, P, K) : choose_shifted<bf16_t>(T_, P, K);
   // Runs of two and more pieces over more than 64 output channels, on problems that fill the chip
-  // with 128-row tiles: one operand tile per run.  WINOCONV_GEMM_ROWS=0 keeps the tile per piece,
-  // =2 takes the 128 x 128 tile of gemm_rows_kernel for every plan with runs (what the tests use
-  // to reach it with small shapes).
-  const char* rows_env = std::getenv("WINOCONV_GEMM_ROWS");
-  const int rows_mode = rows_env ? std::atoi(rows_env) : 1;
+  // with 128-row tiles: one operand tile per run.  wc_test_gemm_override(., 0) keeps the tile per
+  // piece, (., 2) takes the 128 x 128 tile of gemm_rows_kernel for every plan with runs (what the
+  // tests use to reach it with small shapes).
+  const int rows_mode = test_gemm_rows();
   bool rows = sh.n_run >= 2 && sh.n_run <= kRunExtra + 1 && rows_mode != 0 && (K > 32 || rows_mode == 2);
   if (rows) {
     GemmConfig r = dtype == WC_F16 ? choose_rows<half_t>(T_, P, K, rows_mode == 2) : choose_rows<bf16_t>(T_, P, K, rows_mode == 2);
@@ -672,9 +667,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_shifted: problem too large");
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
-  if (c.lds > 64 * 1024)
-    WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
   WC_CHECK_LAUNCH(rows ? "gemm_rows_kernel" : "gemm_kernel (shifted operand)");
   return WC_OK;
@@ -704,9 +697,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(Cp % c.bk == 0, "wc_batched_gemm: tile depth %d does not divide %d", c.bk, Cp);
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
-  if (c.lds > 64 * 1024)
-    WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
   WC_CHECK_LAUNCH("gemm_kernel");
   return WC_OK;

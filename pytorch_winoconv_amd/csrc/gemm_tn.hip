@@ -210,9 +210,7 @@ int launch_tn(GemmTnArgs g, int T_, void* stream) {
   WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_tn: problem too large");
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
-  if (lds > 64 * 1024)
-    WC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel<T, W, BK>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tn_kernel<T, W, BK>), lds)) return rc;
   hipLaunchKernelGGL((gemm_tn_kernel<T, W, BK>), dim3((unsigned)(g.per_xcd * kXcds)), dim3(256), lds, as_stream(stream), g);
   WC_CHECK_LAUNCH("gemm_tn_kernel");
   return WC_OK;

@@ -10,8 +10,11 @@
 //   y[o] = sum_k x[2o + k - pad] w[k] = sum_q sum_j x[2(o + j) + q - pad] w[2j + q].
 #include "wc_common.h"
 #include "wc_tables.h"
+#include <atomic>
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <unordered_set>
 
 namespace wc {
 
@@ -35,6 +38,26 @@ int fail(int code, const char* fmt, ...) {
   g_err = buf;
   return code;
 }
+
+// Kernels that need more than 64 KB of LDS must be told so once per device; the set remembers
+// which (device, kernel) pairs have been, so that launches after the first pay one lookup.
+int ensure_dynamic_lds(const void* fn, size_t bytes) {
+  if (bytes <= 64 * 1024) return WC_OK;
+  static std::mutex mu;
+  static std::unordered_set<uintptr_t> done;
+  int dev = 0;
+  WC_CHECK_HIP(hipGetDevice(&dev));
+  const uintptr_t key = reinterpret_cast<uintptr_t>(fn) * 64 + (uintptr_t)dev;
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count(key)) return WC_OK;
+  WC_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  done.insert(key);
+  return WC_OK;
+}
+
+std::atomic<int> g_gemm_config{-1}, g_gemm_rows{1};
+int test_gemm_config() { return g_gemm_config.load(std::memory_order_relaxed); }
+int test_gemm_rows() { return g_gemm_rows.load(std::memory_order_relaxed); }
 
 struct AxisPiece { int tap0, r; };
 
@@ -74,6 +97,14 @@ static int axis_pieces(int k, int stride, AxisPiece* out) {
 using namespace wc;
 
 extern "C" {
+
+int wc_test_gemm_override(int config, int rows_mode) {
+  WC_CHECK_ARG(config >= -1 && config < 16 && rows_mode >= 0 && rows_mode <= 2,
+               "wc_test_gemm_override: config %d, rows_mode %d", config, rows_mode);
+  g_gemm_config.store(config, std::memory_order_relaxed);
+  g_gemm_rows.store(rows_mode, std::memory_order_relaxed);
+  return WC_OK;
+}
 
 const char* wc_version(void) { return "winoconv-hip 0.1 (gfx950)"; }
 const char* wc_last_error(void) { return g_err.c_str(); }

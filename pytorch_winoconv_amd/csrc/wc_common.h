@@ -26,6 +26,13 @@ int fail(int code, const char* fmt, ...);
          return ::wc::fail(WC_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(e_)); \
   } while (0)
 
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per (device, kernel) for kernels above 64 KB of LDS
+int ensure_dynamic_lds(const void* fn, size_t bytes);
+// what wc_test_gemm_override last set: tile shape forced on wc_batched_gemm (-1: none) and the
+// choice between the two shifted-operand kernels (1: by size)
+int test_gemm_config();
+int test_gemm_rows();
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline long long ceil_div_ll(long long a, long long b) { return (a + b - 1) / b; }

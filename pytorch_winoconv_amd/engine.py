@@ -31,6 +31,32 @@ def _require_gpu(*tensors):
             raise TypeError("winoconv supports float32, float16 and bfloat16, got %s" % t.dtype)
 
 
+def check_operands(x, K, bias=None, U=None):
+    """Shapes and types the C ABI cannot see: the bias must hold K values of x's dtype, a transformed
+    filter must have x's dtype and device (its size is checked by check_u).  Raises before anything
+    is launched; the kernels would read a short bias out of bounds and a filter of another type as
+    garbage."""
+    if bias is not None:
+        if bias.dim() != 1 or bias.numel() != K:
+            raise ValueError("bias must be a 1-D tensor of %d values (one per output channel), got shape %r"
+                             % (K, tuple(bias.shape)))
+        if bias.dtype != x.dtype:
+            raise TypeError("bias is %s, the input is %s: they must share one dtype" % (bias.dtype, x.dtype))
+        if bias.device != x.device:
+            raise ValueError("bias is on %s, the input on %s" % (bias.device, x.device))
+    if U is not None:
+        if U.dtype != x.dtype:
+            raise TypeError("the transformed filter is %s, the input is %s: transform the filter in the input's dtype"
+                            % (U.dtype, x.dtype))
+        if U.device != x.device:
+            raise ValueError("the transformed filter is on %s, the input on %s" % (U.device, x.device))
+
+
+def misaligned(*tensors):
+    """True if one of the tensors does not start on a 16-byte boundary."""
+    return any(t is not None and t.data_ptr() % 16 != 0 for t in tensors)
+
+
 def _triple(v, nd, fill):
     if isinstance(v, int):
         v = (v,) * nd
@@ -287,6 +313,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
     without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses.
     `unfused=True` keeps thin 16-bit 3x3 layers on the three-kernel path (wc_conv_desc.unfused)."""
+    check_operands(x, int(w.shape[0]), bias, U)
     _require_gpu(x, w, bias, U)
     stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
@@ -298,9 +325,12 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
                                     stacked))
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
+    x_cl = channel_last(x)
+    # the one-kernel path of thin layers needs 16-byte aligned operands; a legal view can start anywhere
+    # (x[1:] of a channel-last tensor with 6 channels and 7 x 7 images is 4-byte aligned): three kernels then
+    unfused = bool(unfused) or misaligned(x_cl, U)
     desc, y_shape, nbytes, u_elems = _forward_setup(tuple(x.shape), tuple(w.shape), x.dtype, stride, padding, m,
                                                     chunk_images, whole_kernel, stacked, unfused)
-    x_cl = channel_last(x)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
     if bias is not None:

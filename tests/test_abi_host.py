@@ -141,6 +141,27 @@ def test_python_layer_refuses_cpu_tensors_and_bad_shapes():
         pkg.WinoConv2d(4, 4, 3, 1, 1)(x)
 
 
+def test_bias_and_cached_filter_are_checked_before_any_launch():
+    """The C ABI sees pointers only: a short bias would be read out of bounds and a transformed filter of
+    another dtype misread, so the host layer refuses both (torch's own conv2d raises for them too)."""
+    x = torch.randn(1, 4, 8, 8)
+    w = torch.randn(6, 4, 3, 3)
+    with pytest.raises(ValueError, match="bias must be a 1-D tensor of 6"):
+        engine.conv_forward(x, w, torch.randn(5))
+    with pytest.raises(ValueError, match="bias must be a 1-D tensor of 6"):
+        engine.conv_forward(x, w, torch.randn(6, 1))
+    with pytest.raises(TypeError, match="share one dtype"):
+        engine.conv_forward(x, w, torch.randn(6).half())
+    U16 = torch.zeros(16, 6, 32, dtype=torch.float16)
+    with pytest.raises(TypeError, match="transformed filter is torch.float16"):
+        engine.conv_forward(x, w, None, 1, 1, 2, U=U16)
+    xc, wc, out = torch.randn(1, 1, 8, 8, 4), torch.randn(1, 3, 3, 4, 6), torch.zeros(1, 1, 6, 6, 6)
+    with pytest.raises(ValueError, match="bias must be a 1-D tensor of 6"):
+        pkg.winograd_conv(xc, wc, out, bias=torch.randn(7))
+    with pytest.raises(TypeError, match="transformed filter is torch.float16"):
+        pkg.winograd_conv(xc, wc, out, U=U16)
+
+
 def test_bfloat16_is_a_storage_type():
     d = engine.make_desc((2, 8, 20, 20), (4, 8, 3, 3), torch.bfloat16, 1, 1, 2)
     assert d.dtype == _lib.WC_BF16 == 2 and engine.plan_conv(d).t_total == 16

@@ -22,10 +22,6 @@ CONFIGS = [
     ("metric F(4,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 4, H16),
     ("metric F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, H16),
     ("c1", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, F32),
-    ("c2 vgg 3->64 @224", (8, 3, 224, 224), (64, 3, 3, 3), 1, 1, 2, F32),
-    ("c2 vgg 64->64 @224 m4", (8, 64, 224, 224), (64, 64, 3, 3), 1, 1, 4, F32),
-    ("c2 vgg 128->256 @56", (8, 128, 56, 56), (256, 128, 3, 3), 1, 1, 2, F32),
-    ("c2 vgg 512->512 @14 m4", (8, 512, 14, 14), (512, 512, 3, 3), 1, 1, 4, F32),
     ("c3 64 @56", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 4, H16),
     ("c3 128 @28", (64, 128, 28, 28), (128, 128, 3, 3), 1, 1, 4, H16),
     ("c3 256 @14", (64, 256, 14, 14), (256, 256, 3, 3), 1, 1, 4, H16),
@@ -46,9 +42,20 @@ CONFIGS = [
     ("c5 3-D tile 2x4x4", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, H16),
 ]
 
+# c2: all 13 layers of the VGG-16 stack at N = 8 in fp32, each with both output tiles, F(2x2,3x3) and
+# F(4x4,3x3) (layers of equal shape get their own data: the seed is the layer number)
+VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56), (256, 256, 56),
+         (256, 512, 28), (512, 512, 28), (512, 512, 28), (512, 512, 14), (512, 512, 14), (512, 512, 14)]
+VGG_SEED = {}
+for _i, (_c, _k, _h) in enumerate(VGG16):
+    for _m in (2, 4):
+        _name = "c2 vgg %d: %d->%d @%d m%d" % (_i + 1, _c, _k, _h, _m)
+        VGG_SEED[_name] = _i
+        CONFIGS.append((_name, (8, _c, _h, _h), (_k, _c, 3, 3), 1, 1, _m, F32))
 
-def _data(xs, ws, dtype, dev):
-    g = torch.Generator().manual_seed(0)
+
+def _data(xs, ws, dtype, dev, seed=0):
+    g = torch.Generator().manual_seed(seed)
     fan = 1
     for v in ws[1:]:
         fan *= v
@@ -60,7 +67,7 @@ def _data(xs, ws, dtype, dev):
 @pytest.mark.parametrize("cfg", CONFIGS, ids=[c[0] for c in CONFIGS])
 def test_full_size_config(dev, cfg):
     name, xs, ws, stride, pad, m, dtype = cfg
-    x, w = _data(xs, ws, dtype, dev)
+    x, w = _data(xs, ws, dtype, dev, VGG_SEED.get(name, 0))
     xd, wd = x.to(dev), w.to(dev)
     stacked = False if name.endswith("piece by piece") else None
 
@@ -149,7 +156,7 @@ def test_stacked_plan_beyond_2g_elements_in_one_pass(dev):
     assert err <= 2e-2, err
 
 
-GRAD_CONFIGS = [c for c in CONFIGS if c[0] in ("metric F(4,3)", "metric F(2,3)", "c2 vgg 64->64 @224 m4", "c4 5x5 s1 tile 4",
+GRAD_CONFIGS = [c for c in CONFIGS if c[0] in ("metric F(4,3)", "metric F(2,3)", "c2 vgg 2: 64->64 @224 m4", "c4 5x5 s1 tile 4",
                                                "c4 7x7 s2", "c5 3-D", "c5 3-D tile 2x4x4")]
 
 

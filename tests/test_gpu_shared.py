@@ -117,11 +117,11 @@ def test_exact_on_small_integers(dev, case):
 
 
 @pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
-def test_one_operand_tile_per_run_is_exact_on_small_integers(dev, case, monkeypatch):
+def test_one_operand_tile_per_run_is_exact_on_small_integers(dev, case, gemm_override):
     """The product kernel that serves all pieces of a run from one tile of V (chosen by size; here
     forced, so that small shapes with partial tiles, one to five pieces per run and 3-D plane jumps
     reach it): same integer inputs as above, so the other order of its sums changes nothing."""
-    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+    gemm_override(rows_mode=2)
     test_exact_on_small_integers(dev, case)
 
 
@@ -219,8 +219,8 @@ def test_random_shapes(dev, case):
 
 
 @pytest.mark.parametrize("case", RANDOM[::2], ids=[str(i) for i in range(0, len(RANDOM), 2)])
-def test_random_shapes_with_one_operand_tile_per_run(dev, case, monkeypatch):
-    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+def test_random_shapes_with_one_operand_tile_per_run(dev, case, gemm_override):
+    gemm_override(rows_mode=2)
     test_random_shapes(dev, case)
 
 
@@ -234,7 +234,7 @@ STRIDE2 = [
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", STRIDE2)
-def test_stride_2_on_the_parity_phases(dev, dtype, case, monkeypatch):
+def test_stride_2_on_the_parity_phases(dev, dtype, case, gemm_override):
     """Stride 2 with a shared transformed input: the even and the odd samples of x are phases side
     by side in the rows of V, the pieces are pairs of a phase's taps.  Against fp64 convolution and
     against the CPU oracle's restatement (pieces with their own V) in the same storage type; once
@@ -255,7 +255,7 @@ def test_stride_2_on_the_parity_phases(dev, dtype, case, monkeypatch):
     assert _rel(y, yo.double()) <= (3e-3 if dtype == torch.float16 else 2e-2)
     U = engine.transform_filter(w.to(dev), xs, 2, pad, 2, stacked=2)
     assert torch.equal(engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 2, pad, 2, U=U, stacked=2), y)
-    monkeypatch.setenv("WINOCONV_GEMM_ROWS", "2")
+    gemm_override(rows_mode=2)
     y2 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 2, pad, 2, stacked=2)
     assert _rel(y2, ref) <= 2e-2 and _rel(y2, y.double().cpu()) <= (3e-3 if dtype == torch.float16 else 2e-2)
 

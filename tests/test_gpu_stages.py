@@ -182,12 +182,11 @@ def test_batched_gemm(dev, dtype, T, P, C, K):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_batched_gemm_long_reduction_tile(dev, dtype):
+def test_batched_gemm_long_reduction_tile(dev, dtype, gemm_override):
     """Cp >= 512 with many workgroups selects the 128 x 256 tile of eight wavefronts: checked
     against an fp64 product computed on the device, and bit for bit against the 256 x 128 tile
-    (forced through WINOCONV_GEMM_CONFIG), which adds the same products in the same order.
+    (forced through wc_test_gemm_override), which adds the same products in the same order.
     P = 2001 and K = 264 leave partial tiles on both axes."""
-    import os
     g = torch.Generator().manual_seed(5)
     T, P, C, K = 36, 2001, 512, 264
     V = torch.randn(T, P, C, generator=g).to(dtype).to(dev)
@@ -195,11 +194,8 @@ def test_batched_gemm_long_reduction_tile(dev, dtype):
     M = engine.batched_gemm(V, U)
     want = torch.bmm(V.double(), U.double().transpose(1, 2))
     assert _rel(M[:, :, :K], want) <= (2e-3 if dtype == torch.float16 else 8e-3)
-    os.environ["WINOCONV_GEMM_CONFIG"] = "0"
-    try:
-        M0 = engine.batched_gemm(V, U)
-    finally:
-        del os.environ["WINOCONV_GEMM_CONFIG"]
+    gemm_override(config=0)
+    M0 = engine.batched_gemm(V, U)
     assert torch.equal(M[:, :, :K], M0[:, :, :K])
 
 

@@ -192,3 +192,37 @@ def test_first_layers_against_fp64_and_three_kernel_path(dev, dtype, shape):
     assert torch.equal(engine.conv_forward(xd, wd, bd, 1, pad, 2, U=U), y)
     if dtype != torch.float32:
         assert not torch.equal(y3, y)            # other roundings (M stays in fp32): the fused kernel did run
+
+
+def test_misaligned_view_takes_the_three_kernel_path(dev):
+    """x[1:] of a channel-last fp16 tensor with 6 channels and 7 x 7 images starts 588 bytes into the
+    allocation: 4-byte aligned.  The one-kernel path needs 16-byte aligned operands, so the host layer
+    sends such a view through the three kernels, with the same result as for an aligned copy."""
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(3, 6, 7, 7, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
+    w = (torch.randn(8, 6, 3, 3, generator=g) * (2.0 / 54) ** 0.5).half().to(dev)
+    view = x[1:]
+    assert view.permute(0, 2, 3, 1).is_contiguous() and view.data_ptr() % 8 != 0
+    y = engine.conv_forward(view, w, None, 1, 1, 2)
+    y3 = engine.conv_forward(view.clone(memory_format=torch.channels_last), w, None, 1, 1, 2, unfused=True)
+    assert torch.equal(y, y3)
+    ref = F.conv2d(view.double().cpu(), w.double().cpu(), padding=1)
+    assert float((y.double().cpu() - ref).abs().max() / ref.abs().max()) <= 2e-2
+
+
+def test_fp16_input_transform_of_the_fused_kernel_at_large_magnitudes(dev):
+    """The fused fp16 kernel transforms the input with fp16 adds (the reference kernels' arithmetic type,
+    calculation_kernels.cu:786-806) where the three-kernel path adds in fp32 and rounds once.  With
+    inputs of magnitude 1e3..1e4 (sums of four stay below the fp16 maximum) the two agree to fp16
+    rounding of V, and both stay within the fp16 tolerance of the fp64 convolution."""
+    g = torch.Generator().manual_seed(22)
+    x = (torch.randn(2, 64, 20, 20, generator=g) * 3e3).clamp(-1.2e4, 1.2e4).half().to(dev)
+    w = (torch.randn(64, 64, 3, 3, generator=g) * (2.0 / 576) ** 0.5).half().to(dev)
+    y = engine.conv_forward(x, w, None, 1, 1, 2)
+    y3 = engine.conv_forward(x, w, None, 1, 1, 2, unfused=True)
+    ref = F.conv2d(x.double().cpu(), w.double().cpu(), padding=1)
+    scale = float(ref.abs().max())
+    assert torch.isfinite(y).all() and torch.isfinite(y3).all()
+    assert float((y.double().cpu() - ref).abs().max()) / scale <= 2e-2
+    assert float((y3.double().cpu() - ref).abs().max()) / scale <= 2e-2
+    assert float((y.double() - y3.double()).abs().max()) / scale <= 5e-3
