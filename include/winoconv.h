@@ -197,6 +197,21 @@ int wc_conv_forward(const wc_conv_desc* desc, const void* x,
                     const void* bias, void* y, void* workspace, size_t workspace_bytes,
                     void* stream);
 
+/* wc_conv_forward without a workspace argument.  No counterpart in the reference; it is for callers
+ * that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  U, V and M live in a buffer of WC_STATIC_SCRATCH_BYTES inside the
+ * library's device image (each GPU the library runs on holds its own copy until the process ends),
+ * and the batch is processed in as many chunks of images as it takes for them to fit.  Returns
+ * WC_ERR_WORKSPACE, before anything is launched, if U plus the V and M of a single image exceed the
+ * buffer.  Allocates nothing and frees nothing.  The first call on a device looks up the buffer's
+ * address (make it outside graph capture).  All calls on one GPU share the buffer: calls that
+ * overlap in time on one GPU (two streams, two host threads) race; nothing in it needs to start at
+ * zero, a call only reads what it has written.  Same results as wc_conv_forward, bit for bit. */
+#define WC_STATIC_SCRATCH_BYTES (64u * 1024u * 1024u)
+int wc_conv_forward_static(const wc_conv_desc* desc, const void* x,
+                           const void* w, const int64_t w_strides[5], const void* U_cached,
+                           const void* bias, void* y, void* stream);
+
 /* ---- weight gradient -------------------------------------------------------------------------- */
 /* No counterpart in the reference: it never implemented a backward pass (only a pointer-assign
  * helper exists for one, src/back/utils.cu:15-24; include/split_functions_grad.h:3-6 is empty).

@@ -15,6 +15,7 @@ CSRC = os.path.join(_HERE, "csrc")
 WC_F32, WC_F16, WC_BF16 = 0, 1, 2
 WC_OK, WC_ERR_BAD_ARG, WC_ERR_UNSUPPORTED, WC_ERR_WORKSPACE, WC_ERR_HIP = 0, -1, -2, -3, -4
 WC_MAX_PIECES = 64
+WC_STATIC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
 
@@ -60,6 +61,7 @@ SIGNATURES = {
     "wc_conv_workspace_bytes": (_i, [_desc_p, ctypes.POINTER(_sz)]),
     "wc_conv_u_elems": (_i, [_desc_p, ctypes.POINTER(_sz)]),
     "wc_conv_forward": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "wc_conv_forward_static": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _vp, _vp]),
     "wc_conv_backward_weight_workspace_bytes": (_i, [_desc_p, ctypes.POINTER(_sz)]),
     "wc_conv_backward_weight": (_i, [_desc_p, _vp, _vp, _vp, _i64_5, _vp, _sz, _vp]),
 }

@@ -10,9 +10,37 @@
 // intermediates V and M (each written once and read once).
 #include "wc_common.h"
 
+#include <mutex>
+
 using namespace wc;
 
+// Scratch of wc_conv_forward_static: lives in the library's device image, one copy per GPU at that
+// GPU's own address, held until the process ends.  Host code never uses this name as an address:
+// static_scratch() asks the runtime for the device address once per device and hands that out.
+static __device__ __align__(256) unsigned char scratch[WC_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];      // device address of `scratch` on each GPU, null until first asked
+std::mutex g_scratch_mu;
+
+// Device address of `scratch` on the current device.
+int static_scratch(void** out) {
+  int dev = 0;
+  WC_CHECK_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(WC_ERR_UNSUPPORTED, "wc_conv_forward_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    WC_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr || (reinterpret_cast<uintptr_t>(ptr) & 255) != 0)
+      return fail(WC_ERR_HIP, "wc_conv_forward_static: bad address %p for the static scratch", ptr);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return WC_OK;
+}
 
 struct Layout {
   wc_plan plan;
@@ -137,6 +165,40 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
     if (rc) return rc;
   }
   return WC_OK;
+}
+
+int wc_conv_forward_static(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
+                           const void* U_cached, const void* bias, void* y, void* stream) {
+  WC_CHECK_ARG(d != nullptr, "wc_conv_forward_static: null descriptor");
+  // the largest chunk of images whose V and M fit beside U; the caller's own chunk if that is smaller
+  wc_conv_desc dd = *d;
+  dd.chunk_images = 1;
+  Layout L;
+  int rc = make_layout(&dd, &L);
+  if (rc) return rc;
+  const size_t cap = WC_STATIC_SCRATCH_BYTES;
+  if (L.need() > cap)
+    return fail(WC_ERR_WORKSPACE, "wc_conv_forward_static: one image needs %zu bytes of scratch, the static buffer "
+                "holds %zu; use wc_conv_forward with a caller-provided workspace", L.need(), cap);
+  if (!L.thin) {
+    // v_bytes carries a fixed tail for plans that share one transformed input; the rest grows with the chunk
+    Layout L2;
+    dd.chunk_images = d->N >= 2 ? 2 : 1;
+    rc = make_layout(&dd, &L2);
+    if (rc) return rc;
+    const size_t per_image = dd.chunk_images == 2 ? L2.need() - L.need() + 512 : 0;   // rounding of V and M to 256 each
+    long long fit = per_image ? 1 + (long long)((cap - L.need()) / per_image) : 1;
+    if (fit > d->N) fit = d->N;
+    if (d->chunk_images > 0 && d->chunk_images < fit) fit = d->chunk_images;
+    dd.chunk_images = (int)fit;
+    rc = make_layout(&dd, &L);
+    if (rc) return rc;
+    if (L.need() > cap) return fail(WC_ERR_WORKSPACE, "wc_conv_forward_static: chunk of %d images needs %zu bytes", dd.chunk_images, L.need());
+  }
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  return wc_conv_forward(&dd, x, w, w_strides, U_cached, bias, y, ws, cap, stream);
 }
 
 }  // extern "C"

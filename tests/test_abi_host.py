@@ -162,6 +162,20 @@ def test_bias_and_cached_filter_are_checked_before_any_launch():
         pkg.winograd_conv(xc, wc, out, U=U16)
 
 
+def test_static_scratch_entry_point_refuses_oversized_problems_before_any_gpu_call():
+    """One image of this layer needs 116 MB of V and M, the static buffer holds 64 MiB: the size check comes
+    before the first HIP call, so it can be seen without a GPU (the pointers are never touched)."""
+    lib = _lib.load()
+    desc = engine.make_desc((1, 256, 224, 224), (256, 256, 3, 3), torch.float16, 1, 1, 4)
+    fake = ctypes.c_void_p(4096)
+    strides = (ctypes.c_int64 * 5)(2304, 9, 0, 3, 1)
+    rc = lib.wc_conv_forward_static(ctypes.byref(desc), fake, fake, strides, None, None, fake, None)
+    assert rc == _lib.WC_ERR_WORKSPACE and b"static buffer" in lib.wc_last_error()
+    assert _lib.WC_STATIC_SCRATCH_BYTES == 64 << 20
+    header = open(os.path.join(ROOT, "include", "winoconv.h")).read()
+    assert "#define WC_STATIC_SCRATCH_BYTES (64u * 1024u * 1024u)" in header
+
+
 def test_bfloat16_is_a_storage_type():
     d = engine.make_desc((2, 8, 20, 20), (4, 8, 3, 3), torch.bfloat16, 1, 1, 2)
     assert d.dtype == _lib.WC_BF16 == 2 and engine.plan_conv(d).t_total == 16
