@@ -11,8 +11,8 @@ copied, channel-last (NHWC) in HBM before the timed region starts.
 A step is one pass of the whole path over the batch: filter transform, input transform,
 batched GEMM, output transform - the same C-ABI calls, in the same order and on the same
 stream, that wc_conv_forward makes for a one-chunk batch - with a HIP event between the
-stages so that each kernel's duration is measured inside the timed region.  Exactly K steps
-are timed between two device synchronisations.
+stages of every fourth step (--event-every) so that each kernel's duration is measured inside
+the timed region.  Exactly K steps are timed between two device synchronisations.
 
 Prints ONE JSON line.  `value` is effective TFLOP/s = direct-convolution FLOPs
 (2*N*K*C*oH*oW*9) / time per step.  `roofline` describes the batched GEMM (the dominant
@@ -278,10 +278,14 @@ def main():
     ap.add_argument("--prewarm", type=float, default=0.5, metavar="SECONDS",
                     help="run untimed steps for this long before the warm-up steps (clocks settle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--gemm-config", type=int, default=-1, metavar="I",
+                    help="force tile shape I of the batched GEMM through the library's test hook (-1: its own choice)")
     ap.add_argument("--suite", action="store_true",
                     help="also time every other benchmark configuration (adds a 'suite' list)")
-    ap.add_argument("--event-every", type=int, default=1, metavar="N",
-                    help="record the per-stage HIP events on every N-th timed step")
+    ap.add_argument("--event-every", type=int, default=4, metavar="N",
+                    help="record the per-stage HIP events on every N-th timed step (an event record between two "
+                         "kernels keeps the second from starting under the tail of the first: about 13 us per "
+                         "step with events, measured; 1 = every step)")
     ap.add_argument("--suite-only", default=None, metavar="TEXT",
                     help="with --suite: only the configurations whose name contains TEXT")
     ap.add_argument("--backward", action="store_true",
@@ -301,6 +305,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     lib = _lib.load()
+    if args.gemm_config >= 0:
+        _lib.check(lib.wc_test_gemm_override(args.gemm_config, 1))
     dev = torch.device("cuda:0")
     dtype = torch.float16
 
@@ -355,10 +361,11 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # Stage durations come from HIP events inside the timed region, on every step by default: they
-    # then agree with the profiler's kernel durations (120.6 against 120.4 us for the GEMM on one
-    # box).  The event records cost about 3 % of a step, and launching the four stages one by one
-    # another 3 % against the one-call entry point, which is timed separately below.
+    # Stage durations come from HIP events inside the timed region, on every fourth step by default
+    # (--event-every): they agree with the profiler's kernel durations (120.6 against 120.4 us for
+    # the GEMM on one box).  A step with event records takes about 13 us longer than one without
+    # (0.252 against 0.239 ms measured with events on every step / on none), because each record
+    # sits between two kernels; the steps without records run the same four C-ABI calls.
     sampled = [i % args.event_every == 0 for i in range(args.steps)]
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] if s else None for s in sampled]
     t0 = time.perf_counter()
