@@ -234,6 +234,41 @@ def run_backward(steps=20):
     return out
 
 
+def run_host_overhead(calls=300):
+    """Host side of a small layer (c1: fp32, N=1, C=K=64, 56x56, F(2,3): four kernels of about 5 us): us per
+    call of conv_forward through the compiled host layer (the pybind11 module MakePytorchBackend) and through
+    the ctypes binding of the same C ABI.  `enqueue_us`: the loop of calls alone, before the device has been
+    waited for (what the host spends per call); `wall_us`: the same loop including the final synchronisation."""
+    import torch
+    from pytorch_winoconv_amd import engine
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, 64, 56, 56, generator=g).to(dev).contiguous(memory_format=torch.channels_last)
+    w = (torch.randn(64, 64, 3, 3, generator=g) * (2.0 / 576) ** 0.5).to(dev)
+    out = {}
+    for name, use_ext in (("compiled", True), ("ctypes", False)):
+        if use_ext and engine._ext is None:
+            continue
+        engine.USE_EXT = use_ext
+        try:
+            for _ in range(20):
+                engine.conv_forward(x, w, None, 1, 1, 2)
+            best_q = best_w = float("inf")
+            for _ in range(5):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    engine.conv_forward(x, w, None, 1, 1, 2)
+                t1 = time.perf_counter()
+                torch.cuda.synchronize()
+                t2 = time.perf_counter()
+                best_q, best_w = min(best_q, (t1 - t0) / calls * 1e6), min(best_w, (t2 - t0) / calls * 1e6)
+            out[name] = {"enqueue_us": round(best_q, 1), "wall_us": round(best_w, 1)}
+        finally:
+            engine.USE_EXT = engine._ext is not None
+    return out
+
+
 def run_split_concat(steps=20):
     """Tile split / concat (bit-exact copies) at the metric layer's shape: us per call and HBM GB/s
     of the algorithmic bytes (input once + tiles once; tiles once + output once)."""
@@ -292,6 +327,8 @@ def main():
                     help="also time the weight and input gradients of the metric layer")
     ap.add_argument("--split-concat", action="store_true",
                     help="also time the tile split / concat kernels at the metric layer's shape")
+    ap.add_argument("--host-overhead", action="store_true",
+                    help="also time the host side of a small layer (c1) through the compiled host layer and through ctypes")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -447,6 +484,8 @@ def main():
         result["backward_us"] = run_backward()
     if args.split_concat:
         result["split_concat"] = run_split_concat()
+    if args.host_overhead:
+        result["host_overhead_c1"] = run_host_overhead()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

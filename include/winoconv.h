@@ -133,6 +133,13 @@ int wc_plan_dwm(int kD, int kH, int kW, int* num_split,
 /* General plan of a convolution (stride 1 or 2; tile 2 with F(2,r) pieces, or tile 4 with
  * F(4,r) pieces in 2-D). */
 int wc_plan_conv(const wc_conv_desc* desc, wc_plan* plan);
+/* Fills in what a caller leaves open.  desc->stacked == -1 on entry: replaced by the form of the plan
+ * (0, 1 or 2, see wc_conv_desc.stacked) that measured fastest on MI355X for this dtype, kernel, stride and
+ * channel count.  desc->m == 4 with stacked == 2 (a tile that plan does not have): replaced by 3 where the
+ * three-tap pieces on F(3,3) apply (fp16, 2-D, stride 1, at least 3 taps per axis and 5 on one), else by 2;
+ * the caller reads the tile that will really be used back from desc->m.  No counterpart in the reference,
+ * which has one form only (src/base_conv_launchers.cu:282-399).  Every other function wants stacked >= 0. */
+int wc_conv_auto(wc_conv_desc* desc);
 /* Output extent and tile grid: replaces the shape arithmetic of DWM<T>
  * (src/winograd_conv.cpp:71-90) and of dwm2d_/dwm3d_ (dwm.py:56-61,118-121). */
 int wc_conv_out_dims(const wc_conv_desc* desc, int out[3], int grid[3]);

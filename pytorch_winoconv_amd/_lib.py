@@ -47,6 +47,7 @@ SIGNATURES = {
     "wc_test_gemm_override": (_i, [_i, _i]),
     "wc_plan_dwm": (_i, [_i, _i, _i, c_int_p] + [c_int_p] * 8),
     "wc_plan_conv": (_i, [_desc_p, _plan_p]),
+    "wc_conv_auto": (_i, [_desc_p]),
     "wc_conv_out_dims": (_i, [_desc_p, c_int_p, c_int_p]),
     "wc_padded_channels": (_i, [_i]),
     "wc_padded_channels8": (_i, [_i]),
@@ -69,14 +70,31 @@ SIGNATURES = {
 _lib = None
 
 
+def _ext_make_args():
+    """Paths the Makefile's `ext` target needs (torch, Python and pybind11 headers, the module suffix)."""
+    import sysconfig
+    import pybind11
+    import torch
+    return ["TORCH_DIR=%s" % os.path.dirname(torch.__file__), "PY_INC=%s" % sysconfig.get_paths()["include"],
+            "PYBIND_INC=%s" % pybind11.get_include(), "EXT_SUFFIX=%s" % sysconfig.get_config_var("EXT_SUFFIX")]
+
+
+def ext_path():
+    import sysconfig
+    return os.path.join(_HERE, "MakePytorchBackend" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
 def build(jobs=8, verbose=False):
-    """Compile every HIP source for gfx950 into libwinoconv_hip.so (always recompiles)."""
-    subprocess.run(["make", "-C", CSRC, "clean"], check=True,
-                   stdout=None if verbose else subprocess.DEVNULL)
-    subprocess.run(["make", "-C", CSRC, "-j%d" % jobs], check=True,
-                   stdout=None if verbose else subprocess.DEVNULL)
+    """Compile every HIP source for gfx950 into libwinoconv_hip.so (hipcc) and the host layer, the
+    pybind11 module MakePytorchBackend (g++), always from scratch."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.run(["make", "-C", CSRC, "clean"] + _ext_make_args(), check=True, stdout=out)
+    subprocess.run(["make", "-C", CSRC, "-j%d" % jobs], check=True, stdout=out)
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("build finished without producing %s" % LIB_PATH)
+    subprocess.run(["make", "-C", CSRC, "ext"] + _ext_make_args(), check=True, stdout=out)
+    if not os.path.exists(ext_path()):
+        raise RuntimeError("build finished without producing %s" % ext_path())
     return LIB_PATH
 
 

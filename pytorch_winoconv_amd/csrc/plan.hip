@@ -287,6 +287,72 @@ int wc_plan_conv(const wc_conv_desc* d, wc_plan* plan) {
   return WC_OK;
 }
 
+// Which form of a DWM plan measured fastest on MI355X (wc_conv_auto, stacked == -1):
+//  * 16-bit: pieces added by the batched GEMM (2-D 1.15-1.3x for 5x5 and 7x7 kernels, 3-D 1.05-1.4x: fewer
+//    bytes moved); stride-1 kernels of 4 to 10 taps over at most 256 input channels (3-D: 4 to 8 taps over at
+//    most 128, or 4 taps over at most 256) get the two-tap pieces that share one transformed input (against
+//    stacked F(2,r) pieces 1.15-3x in 2-D at 128 and 256 channels, equal at 512; 1.5-2x in 3-D); where the
+//    caller accepts tile 4 (fp16, 2-D, 5 to 10 taps, at least 3 on the other axis, at most 256 channels) the
+//    shared tile is F(3,3) with three-tap pieces (1.4-1.8x faster than stacked F(4,r) pieces).  At stride 2
+//    the shared-input plan works on the parity phases of x and pays where every phase has four taps (2-D 7x7
+//    and 8x8 kernels, at most 256 channels: 1.2-1.75x) or, in 3-D, two or four (at most 128 channels:
+//    1.65-2.5x); kernels with three taps per phase are 1.8x slower that way and keep their stacked pieces.
+//  * fp32 (product bound by the MFMA rate, to which stacking adds zero taps): only 2-D plans of two to four
+//    pieces are stacked (5x5: 1.1-1.15x; 7x7 with nine pieces: 0.9-1.0x).
+static int auto_stacked(const wc_conv_desc* d) {
+  const int nd = d->ndim;
+  if (d->whole_kernel || (nd == 3 && d->m != 2)) return 0;
+  const int* ks = d->kernel + (3 - nd);
+  int kmax = 0, kmin = 99;
+  for (int a = 0; a < nd; ++a) { kmax = ks[a] > kmax ? ks[a] : kmax; kmin = ks[a] < kmin ? ks[a] : kmin; }
+  if (d->dtype != WC_F32) {
+    if (d->stride == 2) {
+      bool all4 = true, all24 = true;
+      for (int a = 0; a < nd; ++a) {
+        const int t = (ks[a] + 1) / 2;
+        all4 = all4 && t == 4;
+        all24 = all24 && (t == 2 || t == 4);
+      }
+      if (nd == 2 && all4 && d->C <= 256) return 2;
+      if (nd == 3 && all24 && kmax >= 4 && d->C <= 128) return 2;
+    }
+    if (d->stride == 1) {
+      const int cp = wc_padded_channels(d->C);
+      const bool tile3 = d->dtype == WC_F16 && nd == 2 && d->m == 4 && kmin >= 3 && kmax >= 5 && kmax <= 10 && cp <= 256;
+      const bool tile2 = nd == 2 ? (kmax >= 4 && kmax <= 10 && cp <= 256)
+                                 : ((kmax >= 4 && kmax <= 8 && cp <= 128) || (kmax == 4 && cp <= 256));
+      if (tile3 || tile2) return 2;
+    }
+    return 1;
+  }
+  if (nd != 2) return 0;
+  int n = 1;
+  for (int a = 0; a < nd; ++a) {
+    int sum = 0;
+    for (int q = 0; q < (d->stride == 2 ? 2 : 1); ++q) {
+      const int t = d->stride == 2 ? (ks[a] + 1 - q) / 2 : ks[a];
+      if (t > 0) sum += t == 4 ? 2 : (t + 2) / 3;
+    }
+    n *= sum;
+  }
+  return n > 1 && n <= 4 ? 1 : 0;
+}
+
+int wc_conv_auto(wc_conv_desc* d) {
+  WC_CHECK_ARG(d != nullptr, "wc_conv_auto: null descriptor");
+  WC_CHECK_ARG(d->ndim == 2 || d->ndim == 3, "ndim must be 2 or 3, got %d", d->ndim);
+  WC_CHECK_ARG(d->stacked >= -1 && d->stacked <= 2, "stacked must be -1 (choose), 0, 1 or 2");
+  if (d->stacked == -1) d->stacked = auto_stacked(d);
+  if (d->stacked == 2 && d->m == 4) {
+    // the shared-input plan exists for output tiles 2 and 3: tile 3 (F(3,3): fp16 error 3e-3 of the output
+    // range, between F(2,r) and F(4,r); too coarse for bf16) where its three-tap pieces apply, else 2
+    const int kh = d->kernel[1], kw = d->kernel[2];
+    const bool tile3 = d->ndim == 2 && d->stride == 1 && d->dtype == WC_F16 && (kh < kw ? kh : kw) >= 3 && (kh > kw ? kh : kw) >= 5;
+    d->m = tile3 ? 3 : 2;
+  }
+  return WC_OK;
+}
+
 int wc_conv_out_dims(const wc_conv_desc* d, int out[3], int grid[3]) {
   int rc = check_desc(d);
   if (rc) return rc;

@@ -10,6 +10,15 @@ import torch
 from . import _lib
 from ._lib import ConvDesc, Plan, check
 
+# The compiled host layer (csrc/host/make_pytorch_backend.cpp, built by build()): conv_forward goes through it
+# when it is there - same C ABI, a few microseconds of C++ per call instead of some twenty of Python.  Without
+# it (a host with hipcc's output but no C++ build of the module) the ctypes path below does the same work.
+try:
+    from . import MakePytorchBackend as _ext
+except ImportError:
+    _ext = None
+USE_EXT = _ext is not None
+
 _DTYPES = {torch.float32: _lib.WC_F32, torch.float16: _lib.WC_F16, torch.bfloat16: _lib.WC_BF16}
 
 
@@ -94,13 +103,11 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.dtype = _DTYPES[dtype]
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
-    d.stacked = 2 if stacked == 2 else int(bool(stacked))
-    if d.stacked == 2 and d.m == 4:
-        # the shared-input plan exists for output tiles 2 and 3: a caller who asked for tile 4 gets 3 where
-        # _stack picks that plan for its speed (fp16, 2-D, at least 3 taps per axis and 5 on one; F(3,3):
-        # fp16 error 3e-3 of the output range, between F(2,r) and F(4,r); too coarse for bf16), else 2
-        ks = d.kernel[1:]
-        d.m = 3 if (nd == 2 and d.stride == 1 and dtype == torch.float16 and min(ks) >= 3 and max(ks) >= 5) else 2
+    d.stacked = -1 if stacked is None else 2 if stacked == 2 else int(bool(stacked))
+    # what is left open is filled in by the library: the form of the plan if `stacked` is None, and the tile
+    # 3 or 2 where a caller asked for tile 4 and gets the shared-input plan, which has no such tile (d.m then
+    # tells the tile really used)
+    check(_lib.load().wc_conv_auto(ctypes.byref(d)))
     d.unfused = int(bool(unfused))
     return d
 
@@ -213,7 +220,7 @@ def output_transform(desc, plan, M, bias, n_images):
 
 # ---------------------------------------------------------------- whole convolution
 def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
-    """`stacked=None` picks what measured faster on MI355X: pieces summed by the batched GEMM for
+    """`stacked=None` picks what measured faster on MI355X (the rule itself lives in the library, wc_conv_auto): pieces summed by the batched GEMM for
     16-bit plans (2-D: 1.15-1.3x for 5x5 and 7x7 kernels; 3-D: 1.05-1.4x; fewer bytes moved); for
     fp32, whose product is bound by the MFMA rate and to which stacking adds zero taps, only 2-D
     plans of up to four pieces (5x5: 1.1-1.15x; 7x7, nine pieces: 0.9-1.0x).  16-bit stride-1
@@ -237,35 +244,18 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     faster than stacked F(2,r) pieces at N=4, 16x28x28."""
     if stacked is not None:
         return 2 if stacked == 2 else bool(stacked)
-    if whole_kernel or (nd == 3 and m != 2):
-        return False
+    if w_shape is None:
+        return dtype != torch.float32 and not (whole_kernel or (nd == 3 and m != 2))
     if isinstance(stride, (tuple, list)):
         stride = stride[0]
-    if dtype != torch.float32:
-        if stride == 2 and w_shape is not None:
-            taps = [(int(k) + 1) // 2 for k in w_shape[2:]]      # per parity phase
-            if nd == 2 and all(t == 4 for t in taps) and int(w_shape[1]) <= 256:
-                return 2
-            if nd == 3 and all(t in (2, 4) for t in taps) and max(int(k) for k in w_shape[2:]) >= 4 and int(w_shape[1]) <= 128:
-                return 2
-        if stride == 1 and w_shape is not None:
-            ks = [int(k) for k in w_shape[2:]]
-            cp = (int(w_shape[1]) + 31) // 32 * 32
-            tile3 = dtype == torch.float16 and nd == 2 and m == 4 and min(ks) >= 3 and 5 <= max(ks) <= 10 and cp <= 256
-            if nd == 2:
-                tile2 = 4 <= max(ks) <= 10 and cp <= 256
-            else:
-                tile2 = (4 <= max(ks) <= 8 and cp <= 128) or (max(ks) == 4 and cp <= 256)
-            if tile3 or tile2:
-                return 2
-        return True
-    if w_shape is None or nd != 2:
-        return False
-    n = 1
-    for k in w_shape[2:]:
-        taps = [(int(k) + 1 - q) // 2 for q in range(2)] if stride == 2 else [int(k)]
-        n *= sum((t + 2) // 3 if t != 4 else 2 for t in taps if t > 0)
-    return 1 < n <= 4
+    d = ConvDesc()
+    d.ndim = nd
+    d.N, d.C, d.K = 1, int(w_shape[1]), int(w_shape[0])
+    d.kernel[:] = ((1,) if nd == 2 else ()) + tuple(int(v) for v in w_shape[2:])
+    d.stride, d.m, d.dtype = int(stride), int(m), _DTYPES[dtype]
+    d.whole_kernel, d.stacked = int(bool(whole_kernel)), -1
+    check(_lib.load().wc_conv_auto(ctypes.byref(d)))
+    return 2 if d.stacked == 2 else bool(d.stacked)
 
 
 def thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
@@ -313,6 +303,9 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
     without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses.
     `unfused=True` keeps thin 16-bit 3x3 layers on the three-kernel path (wc_conv_desc.unfused)."""
+    if USE_EXT:
+        return _ext.conv_forward(x, w, bias, stride, padding, m, U, chunk_images, bool(whole_kernel), stacked,
+                                 bool(unfused))
     check_operands(x, int(w.shape[0]), bias, U)
     _require_gpu(x, w, bias, U)
     stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)

@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # the tests load what is built; only a tree in which nothing has been built yet is built here
+    from pytorch_winoconv_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
 
 
 @pytest.fixture(scope="session")
@@ -31,3 +35,14 @@ def gemm_override():
         _lib.check(lib.wc_test_gemm_override(config, rows_mode))
     yield force
     _lib.check(lib.wc_test_gemm_override(-1, 1))
+
+
+@pytest.fixture(params=["compiled", "ctypes"])
+def host_layer(request, monkeypatch):
+    """Runs a test once through the compiled host layer (the pybind11 module MakePytorchBackend) and once
+    through the ctypes binding of the same C ABI."""
+    from pytorch_winoconv_amd import engine
+    if request.param == "compiled" and engine._ext is None:
+        pytest.fail("the compiled host layer MakePytorchBackend is not built (pytorch_winoconv_amd.build())")
+    monkeypatch.setattr(engine, "USE_EXT", request.param == "compiled")
+    return request.param
