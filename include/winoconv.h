@@ -12,7 +12,7 @@
  * which device (and what the test hook wc_test_gemm_override last set).
  *
  * Data layouts (row-major, innermost last).  "Channel-last" means NHWC / NDHWC.
- *   x   (N, D, H, W, C)        D = 1 for 2-D problems
+ *   x   (N, D, H, W, C)        D = 1 for 2-D problems (or channel-first, see wc_conv_desc.x_layout)
  *   w   any strided (K, C, kD, kH, kW) view: element strides are passed in
  *   y   (N, oD, oH, oW, K)
  *   U   (T, K,  Cp)            transformed filter, Cp = wc_padded_channels(C)
@@ -106,6 +106,13 @@ typedef struct {
                     *      32, a multiple of 4 in 33..64 or 97..128), at most 512 output channels (256 with
                     *      128 input channels);
                     * 1: always filter transform -> input transform -> batched GEMM -> output transform. */
+  int x_layout;    /* 0: x is channel-last (N, D, H, W, C); 1: x is channel-first contiguous (N, C, D, H, W), the layout
+                    *    torch tensors have by default.  Single-piece 2-D plans at stride 1 (kernels of at most 3 taps
+                    *    per axis) then read x as it is inside the input transform; every other plan copies it to
+                    *    channel-last scratch first (wc_conv_forward: the workspace grows by the size of x).  The
+                    *    reference always runs that copy, as a torch pass of its own (dwm.py:129-133). */
+  int y_layout;    /* the same for y: 1 = channel-first contiguous (N, K, oD, oH, oW); wc_conv_forward then writes the
+                    *    output transform's channel-last result to scratch and copies it (dwm.py:143-144). */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */
@@ -166,13 +173,20 @@ int wc_wino_concat2d(const void* tiles, void* y, int B, int oH, int oW, int K, i
 int wc_wino_concat3d(const void* tiles, void* y, int B, int oD, int oH, int oW, int K, int m,
                      int elem_size, void* stream);
 
+/* Bit-exact copy between channel-first (n, C, S) and channel-last (n, S, C) memory, S = [D] H W positions;
+ * to_channel_last = 1 for the first direction.  Replaces the permute passes of the reference's Python callers
+ * (dwm.py:129-133,143-144; Split_and_Concat.py:25,47,64,81).  elem_size is 2 or 4 bytes. */
+int wc_layout_copy(const void* src, void* dst, int n_images, int channels, long long spatial,
+                   int to_channel_last, int elem_size, void* stream);
+
 /* ---- pipeline stages ---------------------------------------------------------------------- */
 /* U = (G x G x G) g for every piece.  Replaces wNorm2WinoTransform + wNorm2WinoCalculation
  * (src/split_kernel.cu:14-53, src/calculation_kernels.cu:2-761) and matrix_conv.py:150-153.
  * w_strides: element strides of w for (K, C, kD, kH, kW). */
 int wc_filter_transform(const wc_conv_desc* desc, const wc_plan* plan,
                         const void* w, const int64_t w_strides[5], void* U, void* stream);
-/* V = (BT x BT x BT) d for `n_images` images starting at x.  Replaces
+/* V = (BT x BT x BT) d for `n_images` images starting at x (channel-first x, desc->x_layout = 1, only for the
+ * plans named there: WC_ERR_UNSUPPORTED otherwise).  Replaces
  * inputNorm2WinoTransform + inputNorm2WinoCalculation (src/split_kernel.cu:60-120,
  * src/calculation_kernels.cu:763-1522) and matrix_conv.py:158-203. */
 int wc_input_transform(const wc_conv_desc* desc, const wc_plan* plan,

@@ -34,7 +34,7 @@ class ConvDesc(ctypes.Structure):
                 ("in_", ctypes.c_int * 3), ("kernel", ctypes.c_int * 3), ("pad", ctypes.c_int * 3),
                 ("stride", ctypes.c_int), ("m", ctypes.c_int), ("dtype", ctypes.c_int),
                 ("chunk_images", ctypes.c_int), ("whole_kernel", ctypes.c_int), ("stacked", ctypes.c_int),
-                ("unfused", ctypes.c_int)]
+                ("unfused", ctypes.c_int), ("x_layout", ctypes.c_int), ("y_layout", ctypes.c_int)]
 
 
 # name -> (restype, argtypes); every symbol include/winoconv.h declares
@@ -55,6 +55,7 @@ SIGNATURES = {
     "wc_wino_split3d": (_i, [_vp, _vp] + [_i] * 13 + [_vp]),
     "wc_wino_concat2d": (_i, [_vp, _vp] + [_i] * 6 + [_vp]),
     "wc_wino_concat3d": (_i, [_vp, _vp] + [_i] * 7 + [_vp]),
+    "wc_layout_copy": (_i, [_vp, _vp, _i, _i, ctypes.c_longlong, _i, _i, _vp]),
     "wc_filter_transform": (_i, [_desc_p, _plan_p, _vp, _i64_5, _vp, _vp]),
     "wc_input_transform": (_i, [_desc_p, _plan_p, _vp, _i, _vp, _vp]),
     "wc_batched_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),

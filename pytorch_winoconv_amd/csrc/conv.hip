@@ -53,7 +53,9 @@ struct Layout {
   size_t es;
   size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
   bool thin;                          // the one-kernel path runs: V and M are not needed
-  size_t need() const { return thin ? u_bytes : u_bytes + v_bytes + m_bytes; }
+  bool x_direct;                      // channel-first x is read by the input transform itself
+  size_t xcl_bytes, ycl_bytes;        // channel-last scratch copies of a chunk of x / of y (0 if not needed)
+  size_t need() const { return (thin ? u_bytes : u_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
 };
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -91,6 +93,14 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   L->v_bytes = round256((size_t)T * (Pc + (L->shared ? L->shift.tail : 0)) * L->vrow * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
   L->thin = !d->unfused && thin_conv_fits(d, &L->plan);
+  // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
+  // through a channel-last copy of one chunk (the one-kernel path: of the whole batch)
+  L->x_direct = d->x_layout == 1 && !L->thin && input_transform_nchw_fits(d, &L->plan);
+  const size_t images = L->thin ? d->N : chunk;
+  const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L->es;
+  const size_t y_image = (size_t)L->out[0] * L->out[1] * L->out[2] * d->K * L->es;
+  L->xcl_bytes = d->x_layout == 1 && !L->x_direct ? round256(images * x_image) : 0;
+  L->ycl_bytes = d->y_layout == 1 ? round256(images * y_image) : 0;
   return WC_OK;
 }
 
@@ -135,34 +145,52 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   void* Uws = ws;
   void* V = ws + L.u_bytes;
   void* M = ws + L.u_bytes + L.v_bytes;
+  unsigned char* tail = ws + (L.thin ? L.u_bytes : L.u_bytes + L.v_bytes + L.m_bytes);
+  void* Xcl = tail;                       // channel-last copies of channel-first tensors, one chunk each
+  void* Ycl = tail + L.xcl_bytes;
   const void* U = U_cached;
-  if (L.thin) {
-    // thin 16-bit F(2x2, 3x3) layers: one kernel, no V and M
-    if (!U) {
-      rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
-      if (rc) return rc;
-      U = Uws;
-    }
-    return thin_conv_forward(d, &L.plan, x, U, bias, y, stream);
-  }
   if (!U) {
     rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
     if (rc) return rc;
     U = Uws;
   }
-  const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L.es;
-  const size_t y_image = (size_t)L.out[0] * L.out[1] * L.out[2] * d->K * L.es;
-  for (int b0 = 0; b0 < d->N; b0 += L.chunk) {
-    const int n = (d->N - b0 < L.chunk) ? d->N - b0 : L.chunk;
-    const long long P = L.tiles_per_image * n;
-    WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
-    rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);
-    if (rc) return rc;
-    rc = L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
-                  : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
-    if (rc) return rc;
-    rc = wc_output_transform(d, &L.plan, M, bias, n, static_cast<unsigned char*>(y) + b0 * y_image, stream);
-    if (rc) return rc;
+  wc_conv_desc dcl = *d;                  // the stages behind a scratch copy see channel-last tensors
+  dcl.x_layout = L.x_direct ? 1 : 0;
+  dcl.y_layout = 0;
+  const long long in_pos = (long long)d->in[0] * d->in[1] * d->in[2];
+  const long long out_pos = (long long)L.out[0] * L.out[1] * L.out[2];
+  const size_t x_image = (size_t)in_pos * d->C * L.es;
+  const size_t y_image = (size_t)out_pos * d->K * L.es;
+  const int step = L.thin ? d->N : L.chunk;
+  for (int b0 = 0; b0 < d->N; b0 += step) {
+    const int n = (d->N - b0 < step) ? d->N - b0 : step;
+    const void* xin = static_cast<const unsigned char*>(x) + b0 * x_image;
+    void* yout = static_cast<unsigned char*>(y) + b0 * y_image;
+    if (L.xcl_bytes) {
+      rc = transpose_images(xin, Xcl, n, d->C, in_pos, (int)L.es, stream);
+      if (rc) return rc;
+      xin = Xcl;
+    }
+    void* ydst = L.ycl_bytes ? Ycl : yout;
+    if (L.thin) {
+      // thin F(2x2, 3x3) layers: one kernel, no V and M
+      rc = thin_conv_forward(&dcl, &L.plan, xin, U, bias, ydst, stream);
+      if (rc) return rc;
+    } else {
+      const long long P = L.tiles_per_image * n;
+      WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
+      rc = wc_input_transform(&dcl, &L.plan, xin, n, V, stream);
+      if (rc) return rc;
+      rc = L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
+                    : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+      if (rc) return rc;
+      rc = wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream);
+      if (rc) return rc;
+    }
+    if (L.ycl_bytes) {
+      rc = transpose_images(Ycl, yout, n, out_pos, d->K, (int)L.es, stream);
+      if (rc) return rc;
+    }
   }
   return WC_OK;
 }

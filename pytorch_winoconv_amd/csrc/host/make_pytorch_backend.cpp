@@ -259,12 +259,13 @@ std::vector<int> ints_of(py::object v, int nd, const char* what) {
 }
 
 // Winograd / DWM convolution of an NC[D]HW tensor with a (K, C, [kD,] kH, kW) filter; returns an NC[D]HW
-// tensor whose memory is channel-last.  A channel-last input is used without a copy, any other layout is
-// permuted once.  The compiled form of the Python callers' common path (dwm.py:5-40, matrix_conv.py:70-135
+// tensor whose memory is channel-last (or plain contiguous with channels_first_out).  A channel-last input is
+// used without a copy and a contiguous channel-first one is handed to the library as it is
+// (wc_conv_desc.x_layout); any other layout is made contiguous first.  The compiled form of the Python callers' common path (dwm.py:5-40, matrix_conv.py:70-135
 // of the reference end in the same call).
 at::Tensor conv_forward(at::Tensor x, at::Tensor w, std::optional<at::Tensor> bias, py::object stride, py::object padding,
                         int m, std::optional<at::Tensor> U, int chunk_images, bool whole_kernel, py::object stacked,
-                        bool unfused) {
+                        bool unfused, bool channels_first_out) {
   const int nd = (int)x.dim() - 2;
   if ((nd != 2 && nd != 3) || w.dim() != nd + 2)
     throw std::invalid_argument("expected 4-D or 5-D input and matching filter, got " + shape_str(x.sizes()) + " and " + shape_str(w.sizes()));
@@ -317,18 +318,24 @@ at::Tensor conv_forward(at::Tensor x, at::Tensor w, std::optional<at::Tensor> bi
   check(wc_conv_auto(&d));
   int out[3], grid[3];
   check(wc_conv_out_dims(&d, out, grid));
-  std::vector<int64_t> ys{x.size(0)};
+  std::vector<int64_t> ys{x.size(0)};                      // channel-last shape of y
   for (int a = 3 - nd; a < 3; ++a) ys.push_back(out[a]);
   ys.push_back(K);
   std::vector<int64_t> to_cl{0}, to_cf{0, nd + 1};
   for (int a = 0; a < nd; ++a) { to_cl.push_back(2 + a); to_cf.push_back(1 + a); }
   to_cl.push_back(1);
-  at::Tensor y = at::empty(ys, x.options());
-  if (x.size(0) == 0) return y.permute(to_cf);
-  at::Tensor x_cl = x.permute(to_cl);
-  if (!x_cl.is_contiguous()) x_cl = x_cl.contiguous();
+  std::vector<int64_t> ys_cf{ys[0], K};
+  for (int a = 0; a < nd; ++a) ys_cf.push_back(ys[1 + a]);
+  at::Tensor y = at::empty(channels_first_out ? ys_cf : ys, x.options());
+  if (x.size(0) == 0) return channels_first_out ? y : y.permute(to_cf);
+  at::Tensor x_mem = x.permute(to_cl);
+  if (!x_mem.is_contiguous()) {                            // not channel-last memory: channel-first, read as it is
+    x_mem = x.is_contiguous() ? x : x.contiguous();
+    d.x_layout = 1;
+  }
+  d.y_layout = channels_first_out;
   auto misaligned = [](const at::Tensor& t) { return (reinterpret_cast<uintptr_t>(t.data_ptr()) & 15) != 0; };
-  d.unfused = unfused || misaligned(x_cl) || (U && U->defined() && misaligned(*U));
+  d.unfused = unfused || misaligned(x_mem) || (U && U->defined() && misaligned(*U));
   if (U && U->defined()) {
     size_t ue = 0;
     check(wc_conv_u_elems(&d, &ue));
@@ -345,10 +352,10 @@ at::Tensor conv_forward(at::Tensor x, at::Tensor w, std::optional<at::Tensor> bi
   void* stream = stream_of(x);
   {
     py::gil_scoped_release nogil;
-    check(wc_conv_forward(&d, x_cl.data_ptr(), w.data_ptr(), s, U && U->defined() ? U->data_ptr() : nullptr,
+    check(wc_conv_forward(&d, x_mem.data_ptr(), w.data_ptr(), s, U && U->defined() ? U->data_ptr() : nullptr,
                           bc.defined() ? bc.data_ptr() : nullptr, y.data_ptr(), ws.data_ptr(), bytes, stream));
   }
-  return y.permute(to_cf);
+  return channels_first_out ? y : y.permute(to_cf);
 }
 
 // The reference's native entry point (pybind/extern.hpp:7-9): VALID convolution.  The four scratch tensors
@@ -386,6 +393,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("split_and_concat", &split_and_concat);
   m.def("conv_forward", &conv_forward, py::arg("x"), py::arg("w"), py::arg("bias") = py::none(), py::arg("stride") = 1,
         py::arg("padding") = 0, py::arg("m") = 2, py::arg("U") = py::none(), py::arg("chunk_images") = 0,
-        py::arg("whole_kernel") = false, py::arg("stacked") = py::none(), py::arg("unfused") = false);
+        py::arg("whole_kernel") = false, py::arg("stacked") = py::none(), py::arg("unfused") = false,
+        py::arg("channels_first_out") = false);
   m.def("version", []() { return std::string(wc_version()); });
 }

@@ -12,6 +12,12 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
   int rc = wc_conv_out_dims(d, out, grid);
   if (rc) return rc;
   WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_input_transform: bad plan");
+  if (d->x_layout == 1) {
+    if (!input_transform_nchw_fits(d, plan))
+      return fail(WC_ERR_UNSUPPORTED, "wc_input_transform: channel-first x is read directly by single-piece 2-D plans at "
+                  "stride 1 only; copy it with wc_layout_copy, or let wc_conv_forward do so");
+    return input_transform_nchw(d, plan, x, n_images, V, stream);
+  }
   const int Cp = wc_padded_channels(d->C);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
   const bool flat = plan->m[0] == 1;

@@ -165,6 +165,8 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
   WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
+  WC_CHECK_ARG((d->x_layout == 0 || d->x_layout == 1) && (d->y_layout == 0 || d->y_layout == 1),
+               "x_layout and y_layout must be 0 (channel-last) or 1 (channel-first)");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
     return fail(WC_ERR_UNSUPPORTED, "stacked plans are built for DWM plans with output tile 2, or 4 in 2-D");
   if (d->stacked == 2 && d->m != 2 && !(d->m == 3 && d->stride == 1))

@@ -119,6 +119,13 @@ inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream);
 
+// Input transform of single-piece 2-D plans at stride 1 that reads channel-first x (input_transform_2d_nchw.hip):
+// whether the plan is in its range, and the launch.
+bool input_transform_nchw_fits(const wc_conv_desc* d, const wc_plan* plan);
+int input_transform_nchw(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V, void* stream);
+// src (n, R, Q) -> dst (n, Q, R), elements of 2 or 4 bytes (layout_copy.hip)
+int transpose_images(const void* src, void* dst, long long n, long long R, long long Q, int elem_size, void* stream);
+
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;
 

@@ -76,7 +76,7 @@ def _triple(v, nd, fill):
 
 
 def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False, stacked=False,
-              unfused=False):
+              unfused=False, x_layout=0, y_layout=0):
     """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter.  `whole_kernel`: one
     F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces.  `stacked`: the
     DWM pieces share one tile and are added by the batched GEMM instead of by the output transform
@@ -109,6 +109,7 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     # tells the tile really used)
     check(_lib.load().wc_conv_auto(ctypes.byref(d)))
     d.unfused = int(bool(unfused))
+    d.x_layout, d.y_layout = int(x_layout), int(y_layout)     # 1: channel-first contiguous memory (wc_conv_desc.x_layout)
     return d
 
 
@@ -298,14 +299,17 @@ def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, s
 
 
 def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False,
-                 stacked=None, unfused=False):
+                 stacked=None, unfused=False, channels_first_out=False):
     """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
-    is channel-last (torch.channels_last / channels_last_3d); a channel-last input is used
-    without a copy, any other layout is permuted once.  `stacked`: see make_desc; None chooses.
+    is channel-last (torch.channels_last / channels_last_3d), or, with `channels_first_out`, plain
+    contiguous.  A channel-last input is used without a copy; a contiguous (channel-first) one is
+    handed to the library as it is (wc_conv_desc.x_layout: small single-piece plans read it inside the
+    input transform, the others copy it to channel-last scratch with the library's own kernel); any
+    other layout is made contiguous first.  `stacked`: see make_desc; None chooses.
     `unfused=True` keeps thin 16-bit 3x3 layers on the three-kernel path (wc_conv_desc.unfused)."""
     if USE_EXT:
         return _ext.conv_forward(x, w, bias, stride, padding, m, U, chunk_images, bool(whole_kernel), stacked,
-                                 bool(unfused))
+                                 bool(unfused), bool(channels_first_out))
     check_operands(x, int(w.shape[0]), bias, U)
     _require_gpu(x, w, bias, U)
     stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)
@@ -318,36 +322,51 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
                                     stacked))
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
-    x_cl = channel_last(x)
+    # channel-last memory is used as it is, and so is contiguous channel-first memory (x_layout = 1)
+    nd = x.dim() - 2
+    v = x.permute((0,) + tuple(range(2, 2 + nd)) + (1,))
+    x_layout = 0
+    if v.is_contiguous():
+        x_mem = v
+    else:
+        x_mem = x if x.is_contiguous() else x.contiguous()
+        x_layout = 1
+    y_layout = int(bool(channels_first_out))
     # the one-kernel path of thin layers needs 16-byte aligned operands; a legal view can start anywhere
     # (x[1:] of a channel-last tensor with 6 channels and 7 x 7 images is 4-byte aligned): three kernels then
-    unfused = bool(unfused) or misaligned(x_cl, U)
+    unfused = bool(unfused) or misaligned(x_mem, U)
     desc, y_shape, nbytes, u_elems = _forward_setup(tuple(x.shape), tuple(w.shape), x.dtype, stride, padding, m,
-                                                    chunk_images, whole_kernel, stacked, unfused)
+                                                    chunk_images, whole_kernel, stacked, unfused, x_layout, y_layout)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-    y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
+    if y_layout:
+        y = torch.empty([y_shape[0], y_shape[-1]] + y_shape[1:-1], dtype=x.dtype, device=x.device)
+    else:
+        y = torch.empty(y_shape, dtype=x.dtype, device=x.device)
     if bias is not None:
         bias = bias.contiguous()
     if U is not None and (not U.is_contiguous() or U.numel() != u_elems):
         check_u(desc, U)                                  # raises with the sizes in the message
-    check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_cl), _ptr(w), _w_strides(w), _ptr(U),
+    check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_mem), _ptr(w), _w_strides(w), _ptr(U),
                               _ptr(bias), _ptr(y), _ptr(ws), nbytes, _stream(x)))
-    return channel_first_view(y)
+    return y if y_layout else channel_first_view(y)
 
 
 _SETUPS = {}
 
 
-def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused=False):
+def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused=False,
+                   x_layout=0, y_layout=0):
     """Descriptor, output shape (channel-last), workspace bytes and size of U for one problem.  Kept
     per problem: for small layers (a few tens of microseconds on the GPU) rebuilding them on every
     call costs as much host time as the launches themselves."""
     key = (x_shape, w_shape, dtype, stride if isinstance(stride, int) else tuple(stride),
-           padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked, unfused)
+           padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked, unfused,
+           x_layout, y_layout)
     hit = _SETUPS.get(key)
     if hit is None:
         lib = _lib.load()
-        desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused)
+        desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused,
+                         x_layout, y_layout)
         out, _ = out_dims(desc)
         nbytes, ue = ctypes.c_size_t(), ctypes.c_size_t()
         check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
