@@ -269,6 +269,52 @@ def run_host_overhead(calls=300):
     return out
 
 
+def run_layouts(steps=50):
+    """ms per layer with the input in channel-last memory (used as it is), in channel-first contiguous memory
+    handed to the library (read inside the input transform, or copied by the library's kernel), and in
+    channel-first memory permuted by a torch pass first (what the reference does: dwm.py:129-133); then the
+    first again with a channel-first output."""
+    import torch
+    from pytorch_winoconv_amd import engine
+    dev = torch.device("cuda:0")
+    shapes = [("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 2, torch.float32),
+              ("c3 fp16 N64 C64 56x56 F(2,3) one kernel", (64, 64, 56, 56), (64, 64, 3, 3), 2, torch.float16),
+              ("c3 fp16 N64 C128 28x28 F(4,3)", (64, 128, 28, 28), (128, 128, 3, 3), 4, torch.float16),
+              ("c3 fp16 N64 C256 14x14 F(4,3)", (64, 256, 14, 14), (256, 256, 3, 3), 4, torch.float16),
+              ("c3 fp16 N64 C512 7x7 F(4,3)", (64, 512, 7, 7), (512, 512, 3, 3), 4, torch.float16),
+              ("metric fp16 N64 C256 56x56 F(4,3)", (64, 256, 56, 56), (256, 256, 3, 3), 4, torch.float16),
+              ("c2 vgg fp32 N8 64->64 224x224 F(4,3)", (8, 64, 224, 224), (64, 64, 3, 3), 4, torch.float32)]
+    out = []
+    for name, xs, ws, m, dtype in shapes:
+        g = torch.Generator().manual_seed(0)
+        x_cf = torch.randn(*xs, generator=g).to(dtype).to(dev)
+        x_cl = x_cf.contiguous(memory_format=torch.channels_last)
+        w = (torch.randn(*ws, generator=g) * (2.0 / (ws[1] * 9)) ** 0.5).to(dtype).to(dev)
+        calls = {
+            "channel_last_in": lambda: engine.conv_forward(x_cl, w, None, 1, 1, m),
+            "channel_first_in": lambda: engine.conv_forward(x_cf, w, None, 1, 1, m),
+            "channel_first_in_torch_permute": lambda: engine.conv_forward(x_cf.contiguous(memory_format=torch.channels_last), w, None, 1, 1, m),
+            "channel_first_in_and_out": lambda: engine.conv_forward(x_cf, w, None, 1, 1, m, channels_first_out=True),
+            "channel_first_in_and_out_torch_permutes": lambda: engine.conv_forward(
+                x_cf.contiguous(memory_format=torch.channels_last), w, None, 1, 1, m).contiguous(),
+        }
+        row = {"config": name}
+        for what, fn in calls.items():
+            for _ in range(5):
+                fn()
+            best = float("inf")
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                torch.cuda.synchronize()
+                best = min(best, (time.perf_counter() - t0) / steps * 1e3)
+            row[what] = round(best, 4)
+        out.append(row)
+    return out
+
+
 def run_split_concat(steps=20):
     """Tile split / concat (bit-exact copies) at the metric layer's shape: us per call and HBM GB/s
     of the algorithmic bytes (input once + tiles once; tiles once + output once)."""
@@ -329,6 +375,8 @@ def main():
                     help="also time the tile split / concat kernels at the metric layer's shape")
     ap.add_argument("--host-overhead", action="store_true",
                     help="also time the host side of a small layer (c1) through the compiled host layer and through ctypes")
+    ap.add_argument("--layouts", action="store_true",
+                    help="also time small and large layers with channel-last and channel-first tensors")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -484,6 +532,8 @@ def main():
         result["backward_us"] = run_backward()
     if args.split_concat:
         result["split_concat"] = run_split_concat()
+    if args.layouts:
+        result["layouts_ms"] = run_layouts()
     if args.host_overhead:
         result["host_overhead_c1"] = run_host_overhead()
     if not args.no_cpu:

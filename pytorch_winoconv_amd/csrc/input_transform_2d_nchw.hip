@@ -6,7 +6,7 @@
 // inside the transform.  A workgroup owns one row of tiles (all of it, or a block of neighbouring
 // tiles when the image is wide) and 32 words of channels (64 channels of a 16-bit type as channel
 // pairs, 32 channels of fp32).  Phase 1: lanes run along W, where channel-first memory is
-// contiguous - the window rows of a tile row are one contiguous run per channel - and put the
+// contiguous (16-byte loads where the row pitch allows, all loads of a pass in flight together), and put the
 // patch into LDS as [row][column][word], the word index innermost with a row pitch of 33 words,
 // which is free of bank conflicts for the column-wise writes of this phase and the word-wise
 // reads of the next.  Phase 2: a thread takes one tile and one word of channels, reads its window
@@ -35,7 +35,9 @@ struct InNchwArgs {
   int n_blocks, per_xcd;
 };
 
-template <typename T, int K1, int K2, bool PAIR>
+// CE: image columns per global load (the 16-, 4- or 2/4-byte form: the row pitch W must be a multiple of CE and
+// x aligned to the load size)
+template <typename T, int K1, int K2, int CE>
 __global__ __launch_bounds__(256) void input_transform_nchw_kernel(InNchwArgs a) {
   constexpr int A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
   constexpr int m1 = Mats<K1>::m, m2 = Mats<K2>::m;
@@ -60,50 +62,65 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(InNchwArgs a)
   const int tid = threadIdx.x;
 
   // ---- phase 1: patch (A1 rows x PW columns x 32 words) from channel-first memory into LDS
-  if constexpr (sizeof(T) == 2 && PAIR) {
-    // image columns in aligned pairs: one 4-byte load per channel, two words out
-    const int xs = x0 & ~1;
-    const int NP = (x0 + PW - xs + 1) >> 1;
-    const int total = kNchwWords * A1 * NP;
-    for (int it = tid; it < total; it += 256) {
-      const int pq = it % NP;
-      const int r = (it / NP) % A1;
-      const int w = it / (NP * A1);
-      const int ic = xs + 2 * pq, yy = y0 + r;
-      const int c = c0 + 2 * w;
-      const bool in_img = (unsigned)yy < (unsigned)a.H && ic >= 0 && ic + 1 < a.W;   // W is even, so is ic
-      unsigned lo = 0, hi = 0;
-      if (in_img) {
-        const T* p = x + (b * a.C + c) * plane + (long long)yy * a.W + ic;
-        if (c < a.C) lo = *reinterpret_cast<const unsigned*>(p);
-        if (c + 1 < a.C) hi = *reinterpret_cast<const unsigned*>(p + plane);
+  // positions outside the image are zero words: whole rows, then the columns left and right of the image
+  const int nl = max(0, -x0), nr = max(0, x0 + PW - a.W);
+  static_for<0, A1>([&](auto r_) {
+    constexpr int r = decltype(r_)::value;
+    if ((unsigned)(y0 + r) >= (unsigned)a.H) {
+      for (int i = tid; i < PW * kNchwWords; i += 256) lds_words[(r * PW + (i >> 5)) * kNchwPitch + (i & 31)] = 0;
+    } else {
+      for (int i = tid; i < (nl + nr) * kNchwWords; i += 256) {
+        const int k = i >> 5;
+        const int j = k < nl ? k : PW - nr + (k - nl);
+        lds_words[(r * PW + j) * kNchwPitch + (i & 31)] = 0;
       }
-      const int j0 = ic - x0;
-      if (j0 >= 0 && j0 < PW) lds_words[(r * PW + j0) * kNchwPitch + w] = (lo & 0xffffu) | (hi << 16);
-      if (j0 + 1 >= 0 && j0 + 1 < PW) lds_words[(r * PW + j0 + 1) * kNchwPitch + w] = (lo >> 16) | (hi & 0xffff0000u);
     }
-  } else {
-    const int total = kNchwWords * A1 * PW;
-    for (int it = tid; it < total; it += 256) {
-      const int j = it % PW;
-      const int r = (it / PW) % A1;
-      const int w = it / (PW * A1);
-      const int ic = x0 + j, yy = y0 + r;
-      const int c = c0 + VEC * w;
-      const bool in_img = (unsigned)yy < (unsigned)a.H && (unsigned)ic < (unsigned)a.W;
-      unsigned word = 0;
-      if (in_img) {
-        const T* p = x + (b * a.C + c) * plane + (long long)yy * a.W + ic;
-        if constexpr (sizeof(T) == 2) {
-          unsigned lo = 0, hi = 0;
-          if (c < a.C) lo = *reinterpret_cast<const unsigned short*>(p);
-          if (c + 1 < a.C) hi = *reinterpret_cast<const unsigned short*>(p + plane);
-          word = lo | (hi << 16);
-        } else {
-          if (c < a.C) word = *reinterpret_cast<const unsigned*>(p);
+  });
+  // the image part: lanes along W in chunks of CE columns, LPR lanes per row of the patch, the rows of
+  // 256 / LPR words of channels per pass; all loads of a pass are requested before the first is used
+  constexpr int LPR = 64 / CE;                       // lanes per patch row: 64 columns
+  constexpr int WPP = 256 / LPR;                     // words of channels per pass
+  using Raw = Pack<T, CE>;
+  const int lane_q = tid % LPR, lane_w = tid / LPR;
+  const int q_first = max(0, x0) / CE;               // first chunk with a column of the patch
+  const int col_end = min(a.W, x0 + PW);             // one past the last image column of the patch
+  for (int w = lane_w; w < kNchwWords; w += WPP) {
+    const int c = c0 + VEC * w;
+    for (int qq = q_first + lane_q; qq * CE < col_end; qq += LPR) {
+      const int ic0 = qq * CE;
+      Raw lo[A1], hi[A1];
+      static_for<0, A1>([&](auto r_) {
+        constexpr int r = decltype(r_)::value;
+        const int yy = y0 + r;
+        lo[r] = Raw{};
+        hi[r] = Raw{};
+        if ((unsigned)yy < (unsigned)a.H) {
+          const T* p = x + (b * a.C + c) * plane + (long long)yy * a.W + ic0;
+          if (c < a.C) lo[r] = *reinterpret_cast<const Raw*>(p);
+          if constexpr (VEC == 2) {
+            if (c + 1 < a.C) hi[r] = *reinterpret_cast<const Raw*>(p + plane);
+          }
         }
-      }
-      lds_words[(r * PW + j) * kNchwPitch + w] = word;
+      });
+      static_for<0, A1>([&](auto r_) {
+        constexpr int r = decltype(r_)::value;
+        if ((unsigned)(y0 + r) < (unsigned)a.H) {
+#pragma unroll
+          for (int i = 0; i < CE; ++i) {
+            const int j = ic0 + i - x0;
+            if (j >= 0 && j < PW) {
+              unsigned word;
+              if constexpr (VEC == 2) {
+                const Pack<T, 2> pr{{lo[r].v[i], hi[r].v[i]}};
+                word = __builtin_bit_cast(unsigned, pr);
+              } else {
+                word = __builtin_bit_cast(unsigned, lo[r].v[i]);
+              }
+              lds_words[(r * PW + j) * kNchwPitch + w] = word;
+            }
+          }
+        }
+      });
     }
   }
   __syncthreads();
@@ -143,9 +160,9 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(InNchwArgs a)
 
 using InNchwKernel = void (*)(InNchwArgs);
 
-template <typename T, bool PAIR>
+template <typename T, int CE>
 static InNchwKernel pick_nchw(int k1, int k2) {
-#define WC_CASE(a, b) if (k1 == a && k2 == b) return &input_transform_nchw_kernel<T, a, b, PAIR>;
+#define WC_CASE(a, b) if (k1 == a && k2 == b) return &input_transform_nchw_kernel<T, a, b, CE>;
   WC_CASE(KIND_21, KIND_21) WC_CASE(KIND_21, KIND_22) WC_CASE(KIND_21, KIND_23)
   WC_CASE(KIND_22, KIND_21) WC_CASE(KIND_22, KIND_22) WC_CASE(KIND_22, KIND_23)
   WC_CASE(KIND_23, KIND_21) WC_CASE(KIND_23, KIND_22) WC_CASE(KIND_23, KIND_23)
@@ -160,7 +177,10 @@ bool input_transform_nchw_fits(const wc_conv_desc* d, const wc_plan* plan) {
   if (d->ndim != 2 || plan->n_pieces != 1 || plan->tap_step != 1 || d->whole_kernel || d->stacked == 2) return false;
   if (plan->m[0] != 1 || plan->m[1] != plan->m[2] || (plan->m[1] != 2 && plan->m[1] != 4)) return false;
   const wc_piece& pc = plan->piece[0];
-  return pc.r[1] >= 1 && pc.r[1] <= 3 && pc.r[2] >= 1 && pc.r[2] <= 3;
+  if (!(pc.r[1] >= 1 && pc.r[1] <= 3 && pc.r[2] >= 1 && pc.r[2] <= 3)) return false;
+  // the lanes of the loading phase run along W: images narrower than 16 columns leave most of them idle, and the
+  // copy to channel-last memory followed by the channel-last kernel measured faster (N=64, 512 channels, 7x7)
+  return d->in[2] >= 16;
 }
 
 int input_transform_nchw(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V, void* stream) {
@@ -192,11 +212,16 @@ int input_transform_nchw(const wc_conv_desc* d, const wc_plan* plan, const void*
   WC_CHECK_ARG(blocks < (1ll << 30), "input_transform_nchw: problem too large");
   a.n_blocks = (int)blocks;
   a.per_xcd = ceil_div((int)blocks, kXcds);
-  const bool pair = es == 2 && d->in[2] % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0;
+  // columns per load: 16-byte loads where the row pitch and the base allow them, else 4-byte, else single elements
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+  const int W = d->in[2];
+  int ce = 1;
+  if (W % (16 / es) == 0 && (addr & 15) == 0) ce = 16 / es;
+  else if (es == 2 && W % 2 == 0 && (addr & 3) == 0) ce = 2;
   InNchwKernel fn = dispatch_dtype(d->dtype, [&](auto t) -> InNchwKernel {
     using T = decltype(t);
-    if constexpr (sizeof(T) == 2) return pair ? pick_nchw<T, true>(k1, k2) : pick_nchw<T, false>(k1, k2);
-    else return pick_nchw<T, false>(k1, k2);
+    if constexpr (sizeof(T) == 2) return ce == 8 ? pick_nchw<T, 8>(k1, k2) : ce == 2 ? pick_nchw<T, 2>(k1, k2) : pick_nchw<T, 1>(k1, k2);
+    else return ce == 4 ? pick_nchw<T, 4>(k1, k2) : pick_nchw<T, 1>(k1, k2);
   });
   if (!fn) return fail(WC_ERR_UNSUPPORTED, "channel-first input transform for kinds (%d, %d) not built", k1, k2);
   const size_t lds = (size_t)A1 * a.PW * kNchwPitch * 4;

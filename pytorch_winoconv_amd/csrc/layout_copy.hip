@@ -43,6 +43,38 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   }
 }
 
+// The same for 2-byte elements with both extents even and 4-byte aligned tensors: every global access moves a
+// pair of elements (a wavefront reads and writes 256 contiguous bytes per tile row instead of 128).  The tile
+// sits in LDS as [r][q] with a pitch of 66 elements: the pair-wise writes along q are consecutive words, and
+// the reads of one column q for two consecutive rows land in 32 different banks across the 32 row pairs.
+__global__ __launch_bounds__(256) void transpose_pairs_kernel(TransposeArgs a) {
+  __shared__ unsigned short tile[64 * 66];
+  const long long blk = blockIdx.x;
+  const int tq = (int)(blk % a.tiles_q);
+  const long long rest = blk / a.tiles_q;
+  const int tr = (int)(rest % a.tiles_r);
+  const long long n = rest / a.tiles_r;
+  const long long r0 = (long long)tr * 64, q0 = (long long)tq * 64;
+  const unsigned short* src = static_cast<const unsigned short*>(a.src) + n * a.R * a.Q;
+  unsigned short* dst = static_cast<unsigned short*>(a.dst) + n * a.R * a.Q;
+  const int lx = threadIdx.x & 31, ly = threadIdx.x >> 5;      // 32 pairs per row, 8 rows per pass
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = ly + 8 * i;
+    if (r0 + r < a.R && q0 + 2 * lx < a.Q)
+      *reinterpret_cast<unsigned*>(&tile[r * 66 + 2 * lx]) = *reinterpret_cast<const unsigned*>(src + (r0 + r) * a.Q + q0 + 2 * lx);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int qq = ly + 8 * i;
+    if (q0 + qq < a.Q && r0 + 2 * lx < a.R) {
+      const unsigned v = (unsigned)tile[(2 * lx) * 66 + qq] | ((unsigned)tile[(2 * lx + 1) * 66 + qq] << 16);
+      *reinterpret_cast<unsigned*>(dst + (q0 + qq) * a.R + r0 + 2 * lx) = v;
+    }
+  }
+}
+
 // src (n, R, Q) -> dst (n, Q, R), elements of 2 or 4 bytes
 int transpose_images(const void* src, void* dst, long long n, long long R, long long Q, int elem_size, void* stream) {
   WC_CHECK_ARG(src && dst && n > 0 && R > 0 && Q > 0, "layout copy: null pointer or empty tensor");
@@ -52,7 +84,11 @@ int transpose_images(const void* src, void* dst, long long n, long long R, long 
   a.tiles_r = (int)ceil_div_ll(R, 64); a.tiles_q = (int)ceil_div_ll(Q, 64);
   a.n_blocks = n * a.tiles_r * a.tiles_q;
   WC_CHECK_ARG(a.n_blocks < (1ll << 31), "layout copy: problem too large");
-  if (elem_size == 2)
+  const bool pairs = elem_size == 2 && R % 2 == 0 && Q % 2 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3) == 0;
+  if (pairs)
+    hipLaunchKernelGGL(transpose_pairs_kernel, dim3((unsigned)a.n_blocks), dim3(256), 0, as_stream(stream), a);
+  else if (elem_size == 2)
     hipLaunchKernelGGL(transpose_kernel<unsigned short>, dim3((unsigned)a.n_blocks), dim3(256), 0, as_stream(stream), a);
   else
     hipLaunchKernelGGL(transpose_kernel<unsigned>, dim3((unsigned)a.n_blocks), dim3(256), 0, as_stream(stream), a);

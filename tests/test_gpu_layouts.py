@@ -44,12 +44,13 @@ def test_layout_copy_is_a_bit_exact_permute(dev, es, shape):
 # single-piece 2-D plans at stride 1: every tile pair the kernel is built for, even and odd widths (4-byte and
 # 2-byte loads), channel counts that are no multiple of the block, tile rows cut into blocks (wide image)
 DIRECT = [
-    # x shape, w shape, pad, m
-    ((2, 8, 9, 11), (12, 8, 3, 3), 1, 2), ((2, 8, 9, 12), (12, 8, 3, 3), 1, 4), ((1, 3, 10, 10), (5, 3, 3, 3), 0, 2),
-    ((2, 70, 13, 14), (4, 70, 3, 3), 1, 4), ((1, 33, 7, 7), (4, 33, 3, 3), 1, 4), ((1, 5, 6, 200), (4, 5, 3, 3), 1, 2),
-    ((1, 5, 9, 131), (4, 5, 3, 3), 1, 4), ((2, 6, 8, 10), (4, 6, 1, 1), 0, 2), ((2, 6, 8, 10), (4, 6, 2, 3), (1, 0), 2),
-    ((2, 6, 8, 10), (4, 6, 3, 1), (0, 1), 4), ((1, 6, 11, 10), (4, 6, 2, 2), 1, 4), ((1, 6, 11, 10), (4, 6, 1, 2), 0, 4),
-    ((1, 6, 11, 10), (4, 6, 3, 2), 2, 2), ((1, 6, 11, 9), (4, 6, 2, 1), 0, 4), ((1, 6, 11, 10), (4, 6, 1, 3), 1, 2),
+    # x shape, w shape, pad, m   (images at least 16 columns wide: narrower ones take the copy, see below)
+    ((2, 8, 9, 19), (12, 8, 3, 3), 1, 2), ((2, 8, 9, 20), (12, 8, 3, 3), 1, 4), ((1, 3, 10, 18), (5, 3, 3, 3), 0, 2),
+    ((2, 70, 13, 22), (4, 70, 3, 3), 1, 4), ((1, 33, 7, 17), (4, 33, 3, 3), 1, 4), ((1, 5, 6, 200), (4, 5, 3, 3), 1, 2),
+    ((1, 5, 9, 131), (4, 5, 3, 3), 1, 4), ((2, 6, 8, 24), (4, 6, 1, 1), 0, 2), ((2, 6, 8, 16), (4, 6, 2, 3), (1, 0), 2),
+    ((2, 6, 8, 18), (4, 6, 3, 1), (0, 1), 4), ((1, 6, 11, 18), (4, 6, 2, 2), 1, 4), ((1, 6, 11, 26), (4, 6, 1, 2), 0, 4),
+    ((1, 6, 11, 32), (4, 6, 3, 2), 2, 2), ((1, 6, 11, 17), (4, 6, 2, 1), 0, 4), ((1, 6, 11, 40), (4, 6, 1, 3), 1, 2),
+    ((2, 40, 9, 56), (4, 40, 3, 3), 1, 4), ((1, 20, 5, 64), (4, 20, 3, 3), 1, 2),
 ]
 
 
@@ -84,15 +85,18 @@ def test_input_transform_reads_channel_first_memory(dev, dtype, case):
 
 
 def test_stage_refuses_channel_first_memory_for_other_plans(dev):
-    d = engine.make_desc((1, 8, 12, 12), (8, 8, 5, 5), torch.float16, 1, 2, 2, x_layout=1)
-    x = torch.zeros(1, 8, 12, 12, dtype=torch.float16, device=dev)
-    with pytest.raises(NotImplementedError, match="wc_layout_copy"):
-        engine.input_transform(d, engine.plan_conv(d), x)
+    """DWM plans, and images narrower than 16 columns (the copy and the channel-last kernel are faster there)."""
+    for xs, ws, pad in (((1, 8, 12, 20), (8, 8, 5, 5), 2), ((1, 8, 12, 12), (8, 8, 3, 3), 1)):
+        d = engine.make_desc(xs, ws, torch.float16, 1, pad, 2, x_layout=1)
+        x = torch.zeros(*xs, dtype=torch.float16, device=dev)
+        with pytest.raises(NotImplementedError, match="wc_layout_copy"):
+            engine.input_transform(d, engine.plan_conv(d), x)
 
 
 FORWARD = [
     # x shape, w shape, stride, pad, m: single piece (read directly), DWM pieces, stride 2, thin layers, 3-D
-    ((3, 20, 15, 14), (24, 20, 3, 3), 1, 1, 4), ((3, 20, 15, 13), (24, 20, 3, 3), 1, 1, 2), ((2, 20, 15, 14), (24, 20, 5, 5), 1, 2, 2),
+    ((3, 20, 15, 24), (24, 20, 3, 3), 1, 1, 4), ((3, 20, 15, 13), (24, 20, 3, 3), 1, 1, 2), ((2, 20, 15, 14), (24, 20, 5, 5), 1, 2, 2),
+    ((2, 36, 9, 33), (24, 36, 3, 3), 1, 1, 2),
     ((2, 20, 15, 14), (24, 20, 7, 7), 1, 3, 4), ((2, 20, 21, 20), (24, 20, 7, 7), 2, 3, 2), ((2, 20, 15, 14), (24, 20, 3, 3), 2, 1, 2),
     ((2, 64, 12, 12), (64, 64, 3, 3), 1, 1, 2), ((2, 3, 20, 20), (16, 3, 3, 3), 1, 1, 2), ((2, 12, 6, 9, 10), (8, 12, 3, 3, 3), 1, 1, 2),
     ((1, 12, 6, 9, 10), (8, 12, 5, 4, 3), 1, 1, 2),
