@@ -33,10 +33,10 @@ sys.path.insert(0, ROOT)
 N, C, K, H, W, R, PAD, M_TILE = 64, 256, 256, 56, 56, 3, 1, 4
 MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
 HBM_PEAK_GB_S = 8000.0              # MI355X published HBM3E bandwidth
-# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116734 KiB, x2.00 by the copy
+# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116740 KiB, x2.00 by the copy
 # probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
-# profiles/conv3x3_f16_n64_c256_56x56_all_kernels.md.
-GEMM_HBM_TRAFFIC_BYTES = int((116835 * 2.0 + 225792 * 1.0) * 1024)
+# profiles/mfma_utilisation_shipped_gemms.md.
+GEMM_HBM_TRAFFIC_BYTES = int((116740 * 2.0 + 225792 * 1.0) * 1024)
 
 
 def synthetic(n):
