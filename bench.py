@@ -192,7 +192,7 @@ def run_suite(steps=10, only=None):
             ms = fl = msc = 0.0
             for c, k, hw in VGG16:
                 # like the modules: tile 2 where wc_conv_forward has a fused kernel for it (the 3-channel first layer)
-                tile = 2 if engine.thin_layer(torch.float32 if dt == "f32" else torch.float16, 2, c, k, (3, 3), stride) else m
+                tile = 2 if engine.thin_preferred(torch.float32 if dt == "f32" else torch.float16, 2, c, k, (3, 3), stride) else m
                 a, b, c_ = one((8, c, hw, hw), (k, c, 3, 3), stride, pad, tile, dt)
                 ms, fl, msc = ms + a, fl + b, msc + c_
         else:

@@ -104,7 +104,9 @@ typedef struct {
                     *    - at most 4 input channels (any dtype, at most 512 output channels): first layers, or
                     *    - fp16 / bf16 data and input channels that pad to 32, 64 or 128 (an even number up to
                     *      32, a multiple of 4 in 33..64 or 97..128), at most 512 output channels (256 with
-                    *      128 input channels);
+                    *      128 input channels), or
+                    *    - fp32 data, an even number of at most 64 input channels, at most 512 output channels (256
+                    *      above 32 input channels): the products on fp32 MFMA;
                     * 1: always filter transform -> input transform -> batched GEMM -> output transform. */
   int x_layout;    /* 0: x is channel-last (N, D, H, W, C); 1: x is channel-first contiguous (N, C, D, H, W), the layout
                     *    torch tensors have by default.  Single-piece 2-D plans at stride 1 (kernels of at most 3 taps

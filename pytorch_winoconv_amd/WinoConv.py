@@ -102,7 +102,7 @@ class _WinoConvNd(nn.Module):
                                           (dtype == torch.float16 and self.in_channels < 8)):
             return 2
         # thin 16-bit 3x3 layers run as one fused F(2,3) kernel; the cached U must be of that tile
-        if self.output_block is None and engine.thin_layer(dtype, self.nd, self.in_channels, self.out_channels,
+        if self.output_block is None and engine.thin_preferred(dtype, self.nd, self.in_channels, self.out_channels,
                                                             self.kernel_size, self.stride):
             return 2
         return self._tile()

@@ -10,6 +10,7 @@
 // intermediates V and M (each written once and read once).
 #include "wc_common.h"
 
+#include <cstdlib>
 #include <mutex>
 
 using namespace wc;
@@ -59,6 +60,14 @@ struct Layout {
 };
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+// WINOCONV_LOG=1 in the environment (read once, at the first call): wc_conv_forward prints the plan it runs to
+// stderr - silent otherwise (the reference prints from inside its launchers on every call:
+// src/winograd_conv.cpp:106).
+bool log_enabled() {
+  static const bool on = [] { const char* e = std::getenv("WINOCONV_LOG"); return e && e[0] == '1'; }();
+  return on;
+}
 
 int make_layout(const wc_conv_desc* d, Layout* L) {
   int rc = wc_plan_conv(d, &L->plan);
@@ -141,6 +150,21 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0)
     return fail(WC_ERR_WORKSPACE, "wc_conv_forward: workspace must be 256-byte aligned");
 
+  if (log_enabled()) {
+    static const char* const dt[] = {"f32", "f16", "bf16"};
+    std::fprintf(stderr, "winoconv: %dD %s N=%d C=%d K=%d in=%dx%dx%d kernel=%dx%dx%d stride=%d pad=%d,%d,%d | tile m=%d,%d,%d "
+                 "pieces=%d T=%d stacked=%d%s | %s | chunk=%d images, tiles/image=%lld, workspace=%zu B (U %zu, V %zu, M %zu, "
+                 "x copy %zu, y copy %zu) | x %s, y %s, filter %s\n",
+                 d->ndim, dt[d->dtype], d->N, d->C, d->K, d->in[0], d->in[1], d->in[2], d->kernel[0], d->kernel[1], d->kernel[2],
+                 d->stride, d->pad[0], d->pad[1], d->pad[2], L.plan.m[0], L.plan.m[1], L.plan.m[2], L.plan.n_pieces, L.plan.t_total,
+                 d->stacked, d->whole_kernel ? " whole-kernel tile" : "",
+                 L.thin ? "one fused kernel" : (L.shared ? "input transform, shifted batched GEMM, output transform"
+                                                         : "input transform, batched GEMM, output transform"),
+                 L.thin ? d->N : L.chunk, L.tiles_per_image, need, L.u_bytes, L.thin ? (size_t)0 : L.v_bytes,
+                 L.thin ? (size_t)0 : L.m_bytes, L.xcl_bytes, L.ycl_bytes,
+                 d->x_layout ? (L.x_direct ? "channel-first, read by the input transform" : "channel-first, copied") : "channel-last",
+                 d->y_layout ? "channel-first, copied" : "channel-last", U_cached ? "transformed by the caller" : "transformed here");
+  }
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   void* Uws = ws;
   void* V = ws + L.u_bytes;

@@ -45,6 +45,17 @@ template <> struct Mfma16<bf16_t> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
 };
+// fp32: a lane's 16-byte fragment holds four consecutive channels and feeds four v_mfma_f32_16x16x4_f32, each
+// of which pairs channel e of the four lane groups' fragments (both operands are cut the same way, so every
+// channel of a 16-channel step meets its partner exactly once).
+template <> struct Mfma16<float> {
+  using Frag = floatx4;
+  __device__ static __forceinline__ floatx4 run(Frag a, Frag b, floatx4 c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+  }
+};
 
 // The accumulator scheme below is written for these matrices.
 static_assert(Mats<KIND_23>::at(0, 0) == 1 && Mats<KIND_23>::at(0, 1) == 1 && Mats<KIND_23>::at(0, 2) == 1 &&
@@ -143,17 +154,18 @@ static_assert(Mats<KIND_23>::bt(0, 0) == 1 && Mats<KIND_23>::bt(0, 2) == -1 && M
               Mats<KIND_23>::bt(3, 1) == 1 && Mats<KIND_23>::bt(3, 3) == -1, "B^T of F(2,3)");
 
 template <typename T, int CP>
-__global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
+__global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
   // Up to 64 channels a wavefront holds U of all 16 elements (4 wavefronts).  With 128 that is twice
   // the register file, so SPLIT: 8 wavefronts, the upper four take the element rows 2 and 3 and hand
   // their share of the output tile to the lower four through LDS.
-  constexpr bool SPLIT = CP > 64;
+  constexpr bool SPLIT = CP * sizeof(T) > 128;       // 128 channels of a 16-bit type, 64 of fp32
+  constexpr int EPF = 16 / sizeof(T);                // channels per 16-byte fragment
   constexpr int NT = SPLIT ? 512 : 256;
   constexpr int NROW = SPLIT ? 2 : 4;     // element rows per wavefront
   constexpr int VEC = kThinTiles * CP / NT;   // channels per thread in the transform
   constexpr int CVECS = CP / VEC;
-  constexpr int KS = CP / 32;             // MFMA steps along the channels
-  constexpr int PITCH = CP * 2 + 16;      // bytes per (element, tile) row in LDS; the pad spreads 16 rows over all banks
+  constexpr int KS = CP / (4 * EPF);      // fragment steps along the channels (four lane groups x EPF channels each)
+  constexpr int PITCH = CP * sizeof(T) + 16;   // bytes per (element, tile) row in LDS; the pad spreads 16 rows over all banks
   constexpr int BUF = 16 * kThinTiles * PITCH;
   using MF = Mfma16<T>;
   using Frag = typename MF::Frag;
@@ -209,13 +221,13 @@ __global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_pe
   Frag u[NROW * 4][KS];
   {
     const int ko = kbase + (lane & 15);
-    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + 8 * (lane >> 4) +
+    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + EPF * (lane >> 4) +
                  (long long)row0i * 4 * a.K * CP;
     static_for<0, NROW * 4>([&](auto t_) {
       constexpr int t = decltype(t_)::value;
       static_for<0, KS>([&](auto s_) {
         constexpr int s = decltype(s_)::value;
-        u[t][s] = *reinterpret_cast<const Frag*>(U + (long long)t * a.K * CP + s * 32);
+        u[t][s] = *reinterpret_cast<const Frag*>(U + (long long)t * a.K * CP + s * 4 * EPF);
       });
     });
   }
@@ -236,7 +248,7 @@ __global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_pe
         bt23<4, 1>(t2, d);
 #pragma unroll
         for (int e = 0; e < 16; ++e)
-          *reinterpret_cast<half2v*>(vdst + e * (kThinTiles * PITCH / 2) + 2 * h) = d[e];
+          *reinterpret_cast<half2v*>(vdst + e * (kThinTiles * PITCH / (int)sizeof(T)) + 2 * h) = d[e];
       } else {
         typedef float float2v __attribute__((ext_vector_type(2)));
         float2v d[16], t2[16];
@@ -248,7 +260,7 @@ __global__ __launch_bounds__(CP > 64 ? 512 : 256) __attribute__((amdgpu_waves_pe
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const float o[2] = {d[e][0], d[e][1]};
-          store_pack<T, 2>(vdst + e * (kThinTiles * PITCH / 2) + 2 * h, o);
+          store_pack<T, 2>(vdst + e * (kThinTiles * PITCH / (int)sizeof(T)) + 2 * h, o);
         }
       }
     });
@@ -444,8 +456,8 @@ int launch_tiny(ThinArgs a, int k_groups, void* stream) {
 
 template <typename T, int CP>
 int launch_thin(ThinArgs a, int k_groups, void* stream) {
-  constexpr bool split = CP > 64;
-  constexpr int lds = 2 * 16 * kThinTiles * (CP * 2 + 16) + (split ? 4 * 4 * 64 * 16 : 0);
+  constexpr bool split = CP * sizeof(T) > 128;
+  constexpr int lds = 2 * 16 * kThinTiles * (CP * (int)sizeof(T) + 16) + (split ? 4 * 4 * 64 * 16 : 0);
   // workgroups that stay resident (registers and LDS): two per CU, one of the eight-wavefront form;
   // shared among the groups of output channels, in whole multiples of the 8 XCDs
   int wgs = std::min(a.n_blocks, std::max(kXcds, (split ? 256 : 512) / k_groups / kXcds * kXcds));
@@ -470,8 +482,12 @@ bool thin_conv_fits(const wc_conv_desc* d, const wc_plan* plan) {
   if (wc_conv_out_dims(d, out, grid) != WC_OK) return false;
   if ((long long)d->N * out[1] * out[2] * d->K * es >= (1ll << 31)) return false;      // and into y
   if (d->C <= 4) return d->K <= 8 * kThinK;          // tiny_conv3x3_kernel, any storage type
-  if (d->dtype == WC_F32) return false;
   const int Cp = wc_padded_channels(d->C);
+  if (d->dtype == WC_F32) {
+    // fp32: U of 32 channels fits four wavefronts, of 64 channels eight (the products run on fp32 MFMA)
+    if (Cp > 64 || d->C % 2 != 0) return false;
+    return d->K <= (Cp == 64 ? 4 : 8) * kThinK;
+  }
   if (Cp > 128 || (Cp == 96) || d->C % (Cp == 32 ? 2 : 4) != 0) return false;
   return d->K <= (Cp == 128 ? 4 : 8) * kThinK;   // measured: no gain beyond (K = 512 at 128 channels: 0.97x)
 }
@@ -511,7 +527,7 @@ int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x,
       if (Cp == 128) return launch_thin<T, 128>(a, k_groups, stream);
       return Cp == 64 ? launch_thin<T, 64>(a, k_groups, stream) : launch_thin<T, 32>(a, k_groups, stream);
     } else {
-      return fail(WC_ERR_UNSUPPORTED, "thin_conv_forward: 16-bit types only");
+      return Cp == 64 ? launch_thin<T, 64>(a, k_groups, stream) : launch_thin<T, 32>(a, k_groups, stream);
     }
   });
 }

@@ -113,6 +113,14 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     return d
 
 
+def effective_tile(x_shape, w_shape, dtype, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
+    """The output tile conv_forward really uses for this problem and the plan form it picks: (m, stacked).  A
+    caller who asks for tile 4 gets 3 or 2 where the plan whose pieces share one transformed input is chosen
+    (that plan has no tile 4), and the accuracy is that of the smaller tile."""
+    d = make_desc(x_shape, w_shape, dtype, stride, padding, m, 0, whole_kernel, stacked)
+    return d.m, d.stacked
+
+
 def plan_conv(desc):
     plan = Plan()
     check(_lib.load().wc_plan_conv(ctypes.byref(desc), ctypes.byref(plan)))
@@ -261,21 +269,35 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
 
 def thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
     """True for the layers wc_conv_forward runs as one fused F(2x2, 3x3) kernel (wc_conv_desc.unfused):
-    2-D, 3x3, stride 1 and either at most 4 input channels (any type, at most 512 output channels) or
+    2-D, 3x3, stride 1 and either at most 4 input channels (any type, at most 512 output channels), or
     fp16 / bf16 with input channels padded to 32, 64 or 128 (an even number up to 32, a multiple of 4 in
-    33..64 and 97..128) and at most 512 output channels (256 with 128 input channels).  Callers that
-    cache U use it to transform the filter with tile 2."""
+    33..64 and 97..128) and at most 512 output channels (256 with 128 input channels), or fp32 with an
+    even number of at most 64 input channels and at most 512 output channels (256 above 32 input
+    channels).  Callers that cache U use it to transform the filter with tile 2."""
     if nd != 2 or tuple(kernel) != (3, 3):
         return False
     if (stride if isinstance(stride, int) else max(stride)) != 1:
         return False
     if in_channels <= 4:
         return out_channels <= 512
-    if dtype == torch.float32:
-        return False
     cp = (in_channels + 31) // 32 * 32
+    if dtype == torch.float32:
+        return cp <= 64 and in_channels % 2 == 0 and out_channels <= (256 if cp == 64 else 512)
     return (cp in (32, 64, 128) and in_channels % (2 if cp == 32 else 4) == 0
             and out_channels <= (256 if cp == 128 else 512))
+
+
+def thin_preferred(dtype, nd, in_channels, out_channels, kernel, stride):
+    """True where the fused F(2x2, 3x3) kernel also beats the three-kernel path with tile 4, so that a caller
+    free to choose the tile should take 2: every 16-bit layer the kernel takes (1.25-1.7x), first layers, and in
+    fp32 (where the products run on the eight times slower fp32 MFMA and F(4,3) needs 2.25x fewer of them) layers
+    with at most 32 input channels or at most 64 output channels (N=8, 64 -> 64 at 224x224: 194 against 227 us;
+    64 -> 128 at 112x112: 110 against 90 us, so tile 4 there)."""
+    if not thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
+        return False
+    if dtype != torch.float32 or in_channels <= 4:
+        return True
+    return in_channels <= 32 or out_channels <= 64
 
 
 def check_u(desc, U):

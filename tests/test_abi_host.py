@@ -176,6 +176,19 @@ def test_static_scratch_entry_point_refuses_oversized_problems_before_any_gpu_ca
     assert "#define WC_STATIC_SCRATCH_BYTES (64u * 1024u * 1024u)" in header
 
 
+def test_effective_tile_tells_what_a_request_for_tile_4_becomes():
+    """The plan whose pieces share one transformed input has tiles 2 and 3 only: fp16 callers who ask for 4 get 3
+    where the three-tap pieces apply (kernels of 5..10 taps), bf16 callers and 4x4 kernels get 2; plain 3x3
+    layers keep 4.  The choice is made by the library (wc_conv_auto) and reported back."""
+    et = engine.effective_tile
+    assert et((2, 8, 20, 21), (4, 8, 7, 7), torch.float16, 1, 3, 4) == (3, 2)
+    assert et((2, 8, 20, 21), (4, 8, 7, 7), torch.bfloat16, 1, 3, 4) == (2, 2)
+    assert et((2, 8, 20, 21), (4, 8, 4, 4), torch.float16, 1, 1, 4) == (2, 2)
+    assert et((2, 8, 20, 21), (4, 8, 3, 3), torch.float16, 1, 1, 4)[0] == 4
+    assert et((2, 8, 20, 21), (4, 8, 7, 7), torch.float32, 1, 3, 4) == (4, 0)
+    assert et((2, 8, 20, 21), (4, 8, 7, 7), torch.float16, 1, 3, 4, stacked=True) == (4, 1)
+
+
 def test_bfloat16_is_a_storage_type():
     d = engine.make_desc((2, 8, 20, 20), (4, 8, 3, 3), torch.bfloat16, 1, 1, 2)
     assert d.dtype == _lib.WC_BF16 == 2 and engine.plan_conv(d).t_total == 16
@@ -367,7 +380,8 @@ def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
     import pytorch_winoconv_amd as pkg
     from pytorch_winoconv_amd import engine
     assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float16) == 2
-    assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float32) == 4
+    assert pkg.WinoConv2d(64, 64, 3, padding=1)._tile_for(torch.float32) == 2       # fp32: fused where it beats F(4,3)
+    assert pkg.WinoConv2d(64, 128, 3, padding=1)._tile_for(torch.float32) == 4 and pkg.WinoConv2d(32, 256, 3, padding=1)._tile_for(torch.float32) == 2
     assert pkg.WinoConv2d(64, 64, 3, padding=1, output_block=4)._tile_for(torch.float16) == 4
     assert pkg.WinoConv2d(64, 1024, 3, padding=1)._tile_for(torch.float16) == 4     # too many output channels
     assert pkg.WinoConv2d(96, 64, 3, padding=1)._tile_for(torch.float16) == 4       # no kernel for channels padded to 96
@@ -382,7 +396,12 @@ def test_modules_pick_tile_2_for_layers_the_fused_kernel_takes():
     assert t(torch.float16, 2, 30, 8, (3, 3), 1) and not t(torch.float16, 2, 7, 8, (3, 3), 1)    # 2 channels per thread
     assert t(torch.float16, 2, 3, 64, (3, 3), 1) and t(torch.float32, 2, 3, 64, (3, 3), 1) and t(torch.float32, 2, 1, 512, (3, 3), 1)   # first layers
     assert not t(torch.float32, 2, 5, 64, (3, 3), 1) and not t(torch.float32, 2, 3, 600, (3, 3), 1)
-    assert not t(torch.float16, 3, 64, 64, (3, 3), 1) and not t(torch.float32, 2, 64, 64, (3, 3), 1)
+    assert not t(torch.float16, 3, 64, 64, (3, 3), 1)
+    assert t(torch.float32, 2, 64, 256, (3, 3), 1) and not t(torch.float32, 2, 64, 257, (3, 3), 1)      # fp32: up to 64 channels
+    assert t(torch.float32, 2, 32, 512, (3, 3), 1) and not t(torch.float32, 2, 66, 64, (3, 3), 1) and not t(torch.float32, 2, 33, 64, (3, 3), 1)
+    tp = engine.thin_preferred
+    assert tp(torch.float32, 2, 64, 64, (3, 3), 1) and not tp(torch.float32, 2, 64, 128, (3, 3), 1) and tp(torch.float32, 2, 32, 512, (3, 3), 1)
+    assert tp(torch.float16, 2, 128, 256, (3, 3), 1) and tp(torch.float32, 2, 3, 64, (3, 3), 1)
 
 
 def test_product_generator_equals_oracle_generator():

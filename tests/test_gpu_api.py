@@ -239,3 +239,24 @@ def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked):
         got = y.clone()
         want = pkg.engine.conv_forward(x_cl.permute(0, 3, 1, 2), w, None, 1, pad, m, stacked=stacked)   # eager, own buffers
         assert torch.equal(got.permute(0, 3, 1, 2), want), i
+
+
+def test_plan_dump_with_winoconv_log(dev):
+    """WINOCONV_LOG=1 makes wc_conv_forward print the plan it runs (one line per call, to stderr); without it
+    the library prints nothing.  The variable is read once per process, so each case is a process of its own."""
+    import os
+    import subprocess
+    import sys
+    code = ("import torch, pytorch_winoconv_amd as p; x = torch.randn(2, 8, 20, 21, device='cuda').half(); "
+            "w = torch.randn(4, 8, 7, 7, device='cuda').half(); p.engine.conv_forward(x, w, None, 1, 3, 4); "
+            "torch.cuda.synchronize()")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for flag, expect in (("1", True), ("0", False)):
+        env = dict(os.environ, WINOCONV_LOG=flag, PYTHONPATH=root)
+        r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr
+        lines = [ln for ln in r.stderr.splitlines() if ln.startswith("winoconv:")]
+        assert bool(lines) == expect
+        if expect:
+            assert "tile m=1,3,3" in lines[0] and "pieces=9" in lines[0] and "stacked=2" in lines[0]
+            assert "shifted batched GEMM" in lines[0] and "channel-first, copied" in lines[0]

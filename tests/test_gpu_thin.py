@@ -115,7 +115,8 @@ def test_tile_request_and_cached_filter(dev, dtype):
     ((2, 64, 9, 9), (520, 64, 3, 3), 1, torch.float16),      # more than 512 output channels
     ((2, 64, 12, 12), (8, 64, 3, 3), 2, torch.float16),      # stride 2
     ((2, 64, 12, 12), (8, 64, 5, 5), 1, torch.float16),      # DWM plan
-    ((2, 64, 9, 9), (8, 64, 3, 3), 1, torch.float32),       # fp32 with more than 4 channels
+    ((2, 96, 9, 9), (8, 96, 3, 3), 1, torch.float32),       # fp32 with more than 64 channels
+    ((2, 64, 9, 9), (300, 64, 3, 3), 1, torch.float32),     # fp32, 64 channels, more than 256 output channels
     ((2, 64, 5, 9, 9), (8, 64, 3, 3, 3), 1, torch.float16),  # 3-D
 ])
 def test_outside_the_range_nothing_changes(dev, case):
@@ -226,3 +227,37 @@ def test_fp16_input_transform_of_the_fused_kernel_at_large_magnitudes(dev):
     assert float((y.double().cpu() - ref).abs().max()) / scale <= 2e-2
     assert float((y3.double().cpu() - ref).abs().max()) / scale <= 2e-2
     assert float((y.double() - y3.double()).abs().max()) / scale <= 5e-3
+
+
+FP32_SHAPES = [s for s in SHAPES if s[1] <= 64 and s[1] % 2 == 0 and s[2] <= 256] + [
+    (1, 64, 64, 56, 56, 1),      # the single-layer configuration of the benchmark suite
+    (2, 32, 400, 10, 12, 1),     # 32 channels: up to 512 output channels
+    (3, 50, 256, 14, 9, 1),
+]
+
+
+@pytest.mark.parametrize("shape", FP32_SHAPES)
+def test_fp32_layers_of_at_most_64_channels(dev, shape):
+    """fp32 with at most 64 input channels runs the same one kernel on v_mfma_f32_16x16x4_f32 (U of 32 channels in
+    four wavefronts' registers, of 64 channels in eight).  Exact on small integers; on normal inputs within the fp32
+    tolerance of the fp64 convolution and of the oracle, and as close to fp64 as the three-kernel path."""
+    N, C, K, H, W, pad = shape
+    assert engine.thin_layer(torch.float32, 2, C, K, (3, 3), 1)
+    g = torch.Generator().manual_seed(11)
+    xi = torch.randint(-3, 4, (N, C, H, W), generator=g).double()
+    wi = 4.0 * torch.randint(-2, 3, (K, C, 3, 3), generator=g).double()
+    bi = torch.randint(-8, 9, (K,), generator=g).double()
+    yi = engine.conv_forward(xi.float().to(dev), wi.float().to(dev), bi.float().to(dev), 1, pad, 2)
+    assert torch.equal(yi.cpu(), F.conv2d(xi, wi, bi, padding=pad).float())
+    x = torch.randn(N, C, H, W, generator=g)
+    w = torch.randn(K, C, 3, 3, generator=g) * (2.0 / (9 * C)) ** 0.5
+    b = torch.randn(K, generator=g)
+    ref = F.conv2d(x.double(), w.double(), b.double(), padding=pad)
+    xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
+    y = engine.conv_forward(xd, wd, bd, 1, pad, 2)
+    y3 = engine.conv_forward(xd, wd, bd, 1, pad, 2, unfused=True)
+    assert _rel(y, ref) <= 1e-3 and _rel(y, ow.dwm_conv(x, w, b, 1, pad, 2, "fp32")) <= 1e-5
+    assert _rel(y, ref) <= 1.5 * _rel(y3, ref) + 1e-6
+    assert not torch.equal(y, y3)                # other order of the sums: the fused kernel did run
+    U = engine.transform_filter(wd, x.shape, 1, pad, 2)
+    assert torch.equal(engine.conv_forward(xd, wd, bd, 1, pad, 2, U=U), y)
