@@ -97,7 +97,8 @@ SUITE = [
     # c3, 64 and 128 channels: the default is the fused F(2,3) kernel; the three-kernel F(4,3) line stands beside it.
     # c4: the 16-bit default adds the DWM pieces in the batched GEMM; at stride 1 the pieces share one
     # transformed input (tile 3 / F(3,3) with the reference's three-tap pieces where the caller asks for tile 4,
-    # tile 2 / F(2,2) with two-tap pieces where it asks for 2; 7x7 at stride 2: F(2,2) on the parity phases of x),
+    # tile 2 / F(2,2) with two-tap pieces where it asks for 2; 7x7 at stride 2: F(2,2) on the parity phases of x;
+    # 3x3 at stride 2: the direct form, the product reading x itself, with the Winograd plans beside it),
     # else each has its own ("stacked"); two lines with
     # the reference's structure (pieces added after their output transforms) stand beside them.
     ("c1 fp32 N1 C64 56x56 F(2,3)", (1, 64, 56, 56), (64, 64, 3, 3), 1, 1, 2, "f32"),
@@ -117,8 +118,10 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 2, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-stacked"),
-    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
-    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 4, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 direct form (the default)", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16-nodirect"),
+    ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 4, "f16-nodirect"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 direct form", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-direct"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM shared input F(2,2) on the parity phases", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-stacked"),
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-stacked"),
@@ -151,6 +154,7 @@ def run_suite(steps=10, only=None):
         # other DWM plans are stacked)
         stacked = False if dt.endswith("-pieces") else True if dt.endswith("-stacked") else None
         unfused = dt.endswith("-unfused")                          # thin layers: keep the three-kernel path
+        direct = False if dt.endswith("-nodirect") else True if dt.endswith("-direct") else None
         g = torch.Generator().manual_seed(0)
         fan = 1
         for v in ws[1:]:
@@ -159,7 +163,7 @@ def run_suite(steps=10, only=None):
         x = x.contiguous(memory_format=torch.channels_last if len(xs) == 4 else torch.channels_last_3d)
         w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype).to(dev)
         for _ in range(2):
-            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused)
+            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
         # best of three rounds: a single round now and then includes a stall of tens of milliseconds
         # (the caching allocator returning memory between configurations of very different sizes)
         ms = float("inf")
@@ -167,17 +171,17 @@ def run_suite(steps=10, only=None):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
-                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused)
+                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
             torch.cuda.synchronize()
             ms = min(ms, (time.perf_counter() - t0) / steps * 1e3)
-        U = engine.transform_filter(w, xs, stride, pad, m, stacked=stacked)
-        engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused)
+        U = engine.transform_filter(w, xs, stride, pad, m, stacked=stacked, direct=direct)
+        engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused, direct=direct)
         msc = float("inf")
         for _ in range(3):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
-                engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused)
+                engine.conv_forward(x, w, None, stride, pad, m, U=U, stacked=stacked, unfused=unfused, direct=direct)
             torch.cuda.synchronize()
             msc = min(msc, (time.perf_counter() - t0) / steps * 1e3)
         flops = 2.0 * xs[0] * ws[0] * ws[1]

@@ -115,6 +115,14 @@ typedef struct {
                     *    reference always runs that copy, as a torch pass of its own (dwm.py:129-133). */
   int y_layout;    /* the same for y: 1 = channel-first contiguous (N, K, oD, oH, oW); wc_conv_forward then writes the
                     *    output transform's channel-last result to scratch and copies it (dwm.py:143-144). */
+  int direct;      /* 1: the direct form, the degenerate end of the split: pieces of one tap on the trivial tile F(1,1),
+                    *    for which there is nothing to transform, so the batched product reads the pixels of x as its V
+                    *    operand, walks the taps along its reduction axis and writes y; no V or M in memory, U is the
+                    *    filter as (K, kH, kW, C).  2-D, fp16 / bf16, C a multiple of 32, K a multiple of 8; m, stacked
+                    *    and whole_kernel are ignored.  wc_conv_auto chooses it for stride 2, which the reference does
+                    *    not implement (src/winograd_conv.cpp:122-126) and where Winograd tiles on the parity phases
+                    *    save few or no multiplications.  wc_conv_forward, wc_filter_transform, wc_conv_workspace_bytes
+                    *    and wc_conv_u_elems honour it; the other stage functions do not apply. */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */
@@ -143,10 +151,11 @@ int wc_plan_dwm(int kD, int kH, int kW, int* num_split,
  * F(4,r) pieces in 2-D). */
 int wc_plan_conv(const wc_conv_desc* desc, wc_plan* plan);
 /* Fills in what a caller leaves open.  desc->stacked == -1 on entry: replaced by the form of the plan
- * (0, 1 or 2, see wc_conv_desc.stacked) that measured fastest on MI355X for this dtype, kernel, stride and
- * channel count.  desc->m == 4 with stacked == 2 (a tile that plan does not have): replaced by 3 where the
+ * (0, 1 or 2, see wc_conv_desc.stacked; or desc->direct = 1 with stacked = 0) that measured fastest on MI355X
+ * for this dtype, kernel, stride and channel count.  desc->m == 4 with stacked == 2 (a tile that plan does not have): replaced by 3 where the
  * three-tap pieces on F(3,3) apply (fp16, 2-D, stride 1, at least 3 taps per axis and 5 on one), else by 2;
- * the caller reads the tile that will really be used back from desc->m.  No counterpart in the reference,
+ * desc->direct == -1 on entry: the direct form is never chosen (and the field comes back 0).
+ * The caller reads the tile that will really be used back from desc->m.  No counterpart in the reference,
  * which has one form only (src/base_conv_launchers.cu:282-399).  Every other function wants stacked >= 0. */
 int wc_conv_auto(wc_conv_desc* desc);
 /* Output extent and tile grid: replaces the shape arithmetic of DWM<T>

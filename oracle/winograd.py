@@ -265,3 +265,28 @@ def matrix_conv(x, w, m=2, discipline="fp32"):
                      *[mm[0] for mm in mats], Mm.to(mt)).to(st)                # matrix_conv.py:207-211
     y = tl.wino_concat(Y.numpy(), od, m)                                       # matrix_conv.py:134
     return torch.from_numpy(y)
+
+
+def direct_conv(x, w, bias=None, stride=1, padding=0, discipline="fp32"):
+    """The degenerate end of the split: every piece is ONE tap on the trivial tile F(1,1), for which A^T, G and B^T
+    are 1, so y[b, k, oy, ox] = sum over taps (ky, kx) and channels of x[b, c, stride oy + ky - pad, stride ox + kx - pad]
+    w[k, c, ky, kx] with nothing transformed: the products are added tap by tap (ky outermost, the order the engine's
+    product walks its reduction axis) in the arithmetic type of the discipline, the bias is added to the sum, and the
+    result is rounded once to the storage type.  2-D.  The reference has no such form and no stride 2 at all
+    (src/winograd_conv.cpp:122-126); the definition of the convolution itself (torch's conv2d in fp64) pins it."""
+    mt, st = _MATH[discipline], _STORE[discipline]
+    B, C, H, W = x.shape
+    K, _, kh, kw = w.shape
+    ph, pw = (padding, padding) if isinstance(padding, int) else tuple(padding)
+    oH, oW = out_dims((H, W), (kh, kw), (ph, pw), stride)
+    xp = torch.zeros(B, C, H + 2 * ph + stride, W + 2 * pw + stride, dtype=mt)
+    xp[:, :, ph:ph + H, pw:pw + W] = x.to(st).to(mt)
+    wm = w.to(st).to(mt)
+    acc = torch.zeros(B, K, oH, oW, dtype=mt)
+    for ky in range(kh):
+        for kx in range(kw):
+            win = xp[:, :, ky:ky + stride * (oH - 1) + 1:stride, kx:kx + stride * (oW - 1) + 1:stride]
+            acc += torch.einsum("bchw,kc->bkhw", win, wm[:, :, ky, kx])
+    if bias is not None:
+        acc += bias.to(st).to(mt).view(1, K, 1, 1)
+    return acc.to(st)

@@ -34,7 +34,8 @@ class ConvDesc(ctypes.Structure):
                 ("in_", ctypes.c_int * 3), ("kernel", ctypes.c_int * 3), ("pad", ctypes.c_int * 3),
                 ("stride", ctypes.c_int), ("m", ctypes.c_int), ("dtype", ctypes.c_int),
                 ("chunk_images", ctypes.c_int), ("whole_kernel", ctypes.c_int), ("stacked", ctypes.c_int),
-                ("unfused", ctypes.c_int), ("x_layout", ctypes.c_int), ("y_layout", ctypes.c_int)]
+                ("unfused", ctypes.c_int), ("x_layout", ctypes.c_int), ("y_layout", ctypes.c_int),
+                ("direct", ctypes.c_int)]
 
 
 # name -> (restype, argtypes); every symbol include/winoconv.h declares

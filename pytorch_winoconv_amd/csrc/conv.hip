@@ -54,9 +54,10 @@ struct Layout {
   size_t es;
   size_t u_bytes, v_bytes, m_bytes;   // each rounded up to 256
   bool thin;                          // the one-kernel path runs: V and M are not needed
+  bool direct;                        // the direct form: the product reads x itself, V and M are not needed
   bool x_direct;                      // channel-first x is read by the input transform itself
   size_t xcl_bytes, ycl_bytes;        // channel-last scratch copies of a chunk of x / of y (0 if not needed)
-  size_t need() const { return (thin ? u_bytes : u_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
+  size_t need() const { return (thin || direct ? u_bytes : u_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
 };
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -69,7 +70,17 @@ bool log_enabled() {
   return on;
 }
 
-int make_layout(const wc_conv_desc* d, Layout* L) {
+int make_layout(const wc_conv_desc* d_in, Layout* L) {
+  WC_CHECK_ARG(d_in != nullptr, "null descriptor");
+  // the direct form has no tiles: its shapes are those of the plain plan with the same kernel, stride and padding
+  wc_conv_desc plain = *d_in;
+  L->direct = d_in->direct == 1;
+  if (L->direct) {
+    if (!direct_conv_fits(d_in))
+      return fail(WC_ERR_UNSUPPORTED, "direct form: 2-D, fp16 / bf16, input channels a multiple of 32, output channels a multiple of 8");
+    plain.direct = 0; plain.stacked = 0; plain.m = 2; plain.whole_kernel = 0; plain.unfused = 1;
+  }
+  const wc_conv_desc* d = &plain;
   int rc = wc_plan_conv(d, &L->plan);
   if (rc) return rc;
   rc = wc_conv_out_dims(d, L->out, L->grid);
@@ -98,14 +109,15 @@ int make_layout(const wc_conv_desc* d, Layout* L) {
   const long long Pc = L->tiles_per_image * chunk;
   if (T * Pc * (long long)(L->Cp > L->ldm ? L->Cp : L->ldm) >= (1ll << 40))
     return fail(WC_ERR_UNSUPPORTED, "chunk of %d images is too large", chunk);
-  L->u_bytes = round256((size_t)T * d->K * L->Cp * L->es);
+  L->u_bytes = L->direct ? round256((size_t)d->K * d->kernel[1] * d->kernel[2] * d->C * L->es)
+                         : round256((size_t)T * d->K * L->Cp * L->es);
   L->v_bytes = round256((size_t)T * (Pc + (L->shared ? L->shift.tail : 0)) * L->vrow * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
-  L->thin = !d->unfused && thin_conv_fits(d, &L->plan);
+  L->thin = !L->direct && !d->unfused && thin_conv_fits(d, &L->plan);
   // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
   // through a channel-last copy of one chunk (the one-kernel path: of the whole batch)
-  L->x_direct = d->x_layout == 1 && !L->thin && input_transform_nchw_fits(d, &L->plan);
-  const size_t images = L->thin ? d->N : chunk;
+  L->x_direct = d->x_layout == 1 && !L->thin && !L->direct && input_transform_nchw_fits(d, &L->plan);
+  const size_t images = L->thin || L->direct ? d->N : chunk;
   const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L->es;
   const size_t y_image = (size_t)L->out[0] * L->out[1] * L->out[2] * d->K * L->es;
   L->xcl_bytes = d->x_layout == 1 && !L->x_direct ? round256(images * x_image) : 0;
@@ -131,7 +143,7 @@ int wc_conv_u_elems(const wc_conv_desc* d, size_t* elems) {
   Layout L;
   int rc = make_layout(d, &L);
   if (rc) return rc;
-  *elems = (size_t)L.plan.t_total * d->K * L.Cp;
+  *elems = L.direct ? (size_t)d->K * d->kernel[1] * d->kernel[2] * d->C : (size_t)L.plan.t_total * d->K * L.Cp;
   return WC_OK;
 }
 
@@ -169,7 +181,7 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   void* Uws = ws;
   void* V = ws + L.u_bytes;
   void* M = ws + L.u_bytes + L.v_bytes;
-  unsigned char* tail = ws + (L.thin ? L.u_bytes : L.u_bytes + L.v_bytes + L.m_bytes);
+  unsigned char* tail = ws + (L.thin || L.direct ? L.u_bytes : L.u_bytes + L.v_bytes + L.m_bytes);
   void* Xcl = tail;                       // channel-last copies of channel-first tensors, one chunk each
   void* Ycl = tail + L.xcl_bytes;
   const void* U = U_cached;
@@ -185,7 +197,7 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   const long long out_pos = (long long)L.out[0] * L.out[1] * L.out[2];
   const size_t x_image = (size_t)in_pos * d->C * L.es;
   const size_t y_image = (size_t)out_pos * d->K * L.es;
-  const int step = L.thin ? d->N : L.chunk;
+  const int step = L.thin || L.direct ? d->N : L.chunk;
   for (int b0 = 0; b0 < d->N; b0 += step) {
     const int n = (d->N - b0 < step) ? d->N - b0 : step;
     const void* xin = static_cast<const unsigned char*>(x) + b0 * x_image;
@@ -196,7 +208,10 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
       xin = Xcl;
     }
     void* ydst = L.ycl_bytes ? Ycl : yout;
-    if (L.thin) {
+    if (L.direct) {
+      rc = direct_conv(&dcl, xin, n, U, bias, ydst, stream);
+      if (rc) return rc;
+    } else if (L.thin) {
       // thin F(2x2, 3x3) layers: one kernel, no V and M
       rc = thin_conv_forward(&dcl, &L.plan, xin, U, bias, ydst, stream);
       if (rc) return rc;

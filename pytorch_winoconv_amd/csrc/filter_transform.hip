@@ -191,6 +191,11 @@ using namespace wc;
 extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const void* w,
                                    const int64_t w_strides[5], void* U, void* stream) {
   WC_CHECK_ARG(d && plan && w && w_strides && U, "wc_filter_transform: null pointer");
+  if (d->direct == 1) {
+    // the direct form has nothing to transform: U is the filter with taps outermost, channels innermost
+    if (!direct_conv_fits(d)) return fail(WC_ERR_UNSUPPORTED, "wc_filter_transform: problem outside the direct form's range");
+    return direct_filter(d, w, w_strides, U, stream);
+  }
   int out[3], grid[3];
   int rc = wc_conv_out_dims(d, out, grid);   // validates the descriptor
   if (rc) return rc;

@@ -76,6 +76,12 @@ struct GemmArgs {
   // the same plans for gemm_rows_kernel: pieces per run, runs in all, and what the first row of
   // a run moves by from one run to the next / beyond that from one plane to the next (rows of V)
   int n_run, total_runs, run_rows, plane_extra;
+  // direct form (gemm_kernel<..., DIRECT>): the rows of the V operand are the pixels of x itself, row p of the product
+  // is output pixel (b, oy, ox) and starts at input pixel (stride oy - pad_h, stride ox - pad_w); the reduction walks
+  // the taps (kx fastest: the next pixel, then the next image row) with cblocks reduction blocks per tap; taps that
+  // fall outside the image contribute zeros; `bias` (K values, may be null) is added before the result is rounded
+  int H, W, oH, oW, conv_stride, pad_h, pad_w, kw, cblocks;
+  const void* bias;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -87,8 +93,9 @@ typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte g
 // is conflict-free for 128-byte and for 256-byte wide bank sets alike.
 __device__ __forceinline__ int swizzle(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
 
-template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false>
+template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false, bool DIRECT = false>
 __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
+  static_assert(!DIRECT || SHIFT, "the direct form walks the taps like the shifted operand");
   using MF = Mfma<T>;
   constexpr int NT = 64 * NWP * NWK;               // threads: NWP x NWK wavefronts
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
@@ -119,12 +126,22 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   const int lrow = tid / CPR, lpart = tid % CPR;
   const T* gptr[NLOAD];
   int loff[NLOAD];
+  int iy0[DIRECT ? BM / RPP : 1], ix0[DIRECT ? BM / RPP : 1];   // first input pixel of each V row this thread loads
 #pragma unroll
   for (int i = 0; i < NLOAD; ++i) {
     const int row = lrow + i * RPP;                // row of the stacked [X ; W] tile
     if (row < BM) {
       const int p = min(p0 + row, g.P - 1);
-      gptr[i] = Vt + (long long)p * (SHIFT ? g.ldv : g.Cp) + lpart * EPC;
+      if constexpr (DIRECT) {
+        const int per = g.oH * g.oW;
+        const int b = p / per, rem = p - b * per;
+        const int oy = rem / g.oW, ox = rem - oy * g.oW;
+        iy0[i] = oy * g.conv_stride - g.pad_h;
+        ix0[i] = ox * g.conv_stride - g.pad_w;
+        gptr[i] = Vt + (((long long)b * g.H + iy0[i]) * g.W + ix0[i]) * g.ldv + lpart * EPC;
+      } else {
+        gptr[i] = Vt + (long long)p * (SHIFT ? g.ldv : g.Cp) + lpart * EPC;
+      }
     } else {
       const int k = min(k0 + row - BM, g.K - 1);
       gptr[i] = Ut + (long long)k * g.Cp + lpart * EPC;
@@ -134,10 +151,27 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
 
   Chunk16 regs[NLOAD];
   // `vshift`: what the V operand has jumped by at reduction block kt (rows i < BM / RPP are V's)
+  int tap_y = 0, tap_x = 0, tap_cb = 0;             // direct form: the tap and channel block of the next load
   auto gload = [&](int kt, long long vshift) {
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i)
+    for (int i = 0; i < NLOAD; ++i) {
+      if constexpr (DIRECT) {
+        if (i < BM / RPP) {
+          const int j = i < BM / RPP ? i : 0;
+          const bool inside = (unsigned)(iy0[j] + tap_y) < (unsigned)g.H && (unsigned)(ix0[j] + tap_x) < (unsigned)g.W;
+          regs[i] = Chunk16{0u, 0u, 0u, 0u};
+          if (inside) regs[i] = *reinterpret_cast<const Chunk16*>(gptr[i] + kt * BK + vshift);
+          continue;
+        }
+      }
       regs[i] = *reinterpret_cast<const Chunk16*>(gptr[i] + kt * BK + (SHIFT && i < BM / RPP ? vshift : 0));
+    }
+    if constexpr (DIRECT) {
+      if (++tap_cb == g.cblocks) {
+        tap_cb = 0;
+        if (++tap_x == g.kw) { tap_x = 0; ++tap_y; }
+      }
+    }
   };
   auto lstore = [&](int buf) {
 #pragma unroll
@@ -231,8 +265,17 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           Pack<T, 4> o;
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (DIRECT) {
+            if (g.bias) {
+              const int kb = k0 + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i0 + ii][j][4 * q + e]);
+              for (int e = 0; e < 4; ++e)
+                if (kb + e < g.K) bv[e] = static_cast<float>(static_cast<const T*>(g.bias)[kb + e]);
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i0 + ii][j][4 * q + e] + bv[e]);
           *reinterpret_cast<Pack<T, 4>*>(cs + (wp * EI * 32 + ii * 32 + l32) * CS + wk * WN * 32 + j * 32 + 8 * q + 4 * lhi) = o;
         }
     __syncthreads();
@@ -258,14 +301,14 @@ struct GemmConfig {
   int threads;
 };
 
-template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false>
+template <typename T, int WM, int WN, int BK, int NWP = 2, int NWK = 2, bool SHIFT = false, bool DIRECT = false>
 static GemmConfig make_config() {
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BM = 32 * NWP * WM, BN = 32 * NWK * WN;
   constexpr int EI = sizeof(T) == 4 ? 1 : (NWP * NWK == 4 ? WM : WM / 2);
   constexpr size_t stages = (size_t)2 * (BM + BN) * BK * sizeof(T);
   constexpr size_t out_tile = (size_t)32 * NWP * EI * (BN + EPC) * sizeof(T);
-  return GemmConfig{&gemm_kernel<T, WM, WN, BK, NWP, NWK, SHIFT>, BM, BN, BK,
+  return GemmConfig{&gemm_kernel<T, WM, WN, BK, NWP, NWK, SHIFT, DIRECT>, BM, BN, BK,
                     stages > out_tile ? stages : out_tile, 64 * NWP * NWK};
 }
 
@@ -659,6 +702,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   g.jump = (long long)(sh.run_rows - sh.n_run) * Cp;     // on to the same tile one grid row further
   g.plane_runs = sh.n_runs;
   g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
+  g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
   g.n_run = sh.n_run; g.total_runs = sh.n_planes * sh.n_runs;
   g.run_rows = sh.run_rows; g.plane_extra = sh.plane_rows - sh.n_runs * sh.run_rows;
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
@@ -670,6 +714,64 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
   WC_CHECK_LAUNCH(rows ? "gemm_rows_kernel" : "gemm_kernel (shifted operand)");
+  return WC_OK;
+}
+
+// Tiles of the direct form, chosen like those of the shifted operand.
+template <typename T>
+static GemmConfig choose_direct(int P, int K) {
+  auto blocks = [&](const GemmConfig& c) { return (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn); };
+  switch (test_gemm_config()) {                       // wc_test_gemm_override: a tile shape forced by a test
+    case 0: return make_config<T, 2, 2, 32, 4, 2, true, true>();
+    case 1: return make_config<T, 2, 2, 32, 2, 2, true, true>();
+    case 2: return make_config<T, 4, 1, 32, 2, 2, true, true>();
+    case 3: return make_config<T, 1, 1, 32, 2, 2, true, true>();
+    case 4: return make_config<T, 4, 2, 32, 2, 2, true, true>();   // 256 x 128, four wavefronts
+    default: break;
+  }
+  // Measured on MI355X (fp16, stride 2): the largest tile that still gives every compute unit a workgroup
+  // wins: 256 x 128 over 128 x 128 by 15-25 % at 392 workgroups (N=32, C=K=128, 112x112: 54.9 against
+  // 63.7 us; C=K=256, 56x56: 93.5 against 115 us), and loses by 40 % at 196.  Four wavefronts of 128 x 64
+  // beat eight of 64 x 64 for the large tile (54.9 against 73.0 us): half the LDS reads per MFMA.
+  if (K > 64) {
+    GemmConfig big = make_config<T, 4, 2, 32, 2, 2, true, true>();   // 256 x 128, four wavefronts
+    if (blocks(big) >= kCus) return big;
+    GemmConfig mid = make_config<T, 2, 2, 32, 2, 2, true, true>();   // 128 x 128
+    if (blocks(mid) >= kCus) return mid;
+  }
+  return make_config<T, 1, 1, 32, 2, 2, true, true>();               // 64 x 64
+}
+
+// y (N, oH, oW, K) = direct convolution of x (N, H, W, C) with U (K, kh kw C): the batched product with the
+// pixels of x as its V operand (no transform, no intermediate in memory); 16-bit types, C a multiple of 32,
+// K a multiple of 8.
+int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,
+                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream) {
+  WC_CHECK_ARG(x && U && y, "gemm_direct_conv: null pointer");
+  WC_CHECK_ARG(C > 0 && C % 32 == 0 && K > 0 && K % 8 == 0, "gemm_direct_conv: C %d (multiple of 32), K %d (multiple of 8)", C, K);
+  if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "gemm_direct_conv: 16-bit types only");
+  const long long P = (long long)N * oH * oW;
+  WC_CHECK_ARG(P > 0 && P < (1ll << 31) && (long long)kh * kw * C < (1ll << 24), "gemm_direct_conv: problem too large");
+  GemmConfig c = dtype == WC_F16 ? choose_direct<half_t>((int)P, K) : choose_direct<bf16_t>((int)P, K);
+  GemmArgs g;
+  g.V = x; g.U = U; g.M = y; g.bias = bias;
+  g.P = (int)P; g.K = K; g.ldm = K;
+  g.Cp = kh * kw * C;                                    // reduction length = row length of U
+  g.ldv = C;
+  g.run_blocks = kw * C / c.bk;                          // one run: the taps of one kernel row, neighbouring pixels
+  g.jump = (long long)(W - kw) * C;                      // on to the same column one image row further
+  g.plane_runs = kh + 1; g.jump2 = 0;                    // one plane: never left
+  g.n_run = kw; g.total_runs = kh; g.run_rows = W; g.plane_extra = 0;
+  g.H = H; g.W = W; g.oH = oH; g.oW = oW; g.conv_stride = stride; g.pad_h = pad_h; g.pad_w = pad_w;
+  g.kw = kw; g.cblocks = C / c.bk;
+  g.sV = 0; g.sU = 0; g.sM = 0;
+  g.tiles_p = ceil_div((int)P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 1;
+  const long long blocks = (long long)g.tiles_p * g.tiles_k;
+  g.n_blocks = (int)blocks;
+  g.per_xcd = ceil_div((int)blocks, kXcds);
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
+  hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
+  WC_CHECK_LAUNCH("gemm_kernel (direct form)");
   return WC_OK;
 }
 
@@ -691,6 +793,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.sV = (long long)P * Cp; g.sU = (long long)K * Cp; g.sM = (long long)P * ldm;
   g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
   g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
+  g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

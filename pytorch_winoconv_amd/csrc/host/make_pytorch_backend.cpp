@@ -265,7 +265,7 @@ std::vector<int> ints_of(py::object v, int nd, const char* what) {
 // of the reference end in the same call).
 at::Tensor conv_forward(at::Tensor x, at::Tensor w, std::optional<at::Tensor> bias, py::object stride, py::object padding,
                         int m, std::optional<at::Tensor> U, int chunk_images, bool whole_kernel, py::object stacked,
-                        bool unfused, bool channels_first_out) {
+                        bool unfused, bool channels_first_out, py::object direct) {
   const int nd = (int)x.dim() - 2;
   if ((nd != 2 && nd != 3) || w.dim() != nd + 2)
     throw std::invalid_argument("expected 4-D or 5-D input and matching filter, got " + shape_str(x.sizes()) + " and " + shape_str(w.sizes()));
@@ -315,6 +315,7 @@ at::Tensor conv_forward(at::Tensor x, at::Tensor w, std::optional<at::Tensor> bi
   d.chunk_images = chunk_images;
   d.whole_kernel = whole_kernel;
   d.stacked = stacked.is_none() ? -1 : (py::isinstance<py::bool_>(stacked) ? (int)stacked.cast<bool>() : stacked.cast<int>());
+  d.direct = direct.is_none() ? 0 : (direct.cast<bool>() ? 1 : -1);      // None: the library may choose it
   check(wc_conv_auto(&d));
   int out[3], grid[3];
   check(wc_conv_out_dims(&d, out, grid));
@@ -394,6 +395,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("conv_forward", &conv_forward, py::arg("x"), py::arg("w"), py::arg("bias") = py::none(), py::arg("stride") = 1,
         py::arg("padding") = 0, py::arg("m") = 2, py::arg("U") = py::none(), py::arg("chunk_images") = 0,
         py::arg("whole_kernel") = false, py::arg("stacked") = py::none(), py::arg("unfused") = false,
-        py::arg("channels_first_out") = false);
+        py::arg("channels_first_out") = false, py::arg("direct") = py::none());
   m.def("version", []() { return std::string(wc_version()); });
 }

@@ -165,6 +165,7 @@ static int check_desc(const wc_conv_desc* d) {
   WC_CHECK_ARG(d->chunk_images >= 0, "chunk_images must be >= 0");
   WC_CHECK_ARG(d->whole_kernel == 0 || d->whole_kernel == 1, "whole_kernel must be 0 or 1");
   WC_CHECK_ARG(d->stacked >= 0 && d->stacked <= 2, "stacked must be 0, 1 or 2");
+  WC_CHECK_ARG(d->direct == 0 || d->direct == 1, "direct must be 0 or 1");
   WC_CHECK_ARG((d->x_layout == 0 || d->x_layout == 1) && (d->y_layout == 0 || d->y_layout == 1),
                "x_layout and y_layout must be 0 (channel-last) or 1 (channel-first)");
   if (d->stacked && (d->whole_kernel || (d->ndim == 3 && d->m != 2)))
@@ -340,11 +341,29 @@ static int auto_stacked(const wc_conv_desc* d) {
   return n > 1 && n <= 4 ? 1 : 0;
 }
 
+// Stride 2 in 16-bit: where the direct form measured faster than the parity-phase Winograd plans on MI355X
+// (fp16, filter conversion included on both sides).  It wins while the reduction kh kw C is short: 3x3 at
+// N=32, C=K=128, 112x112 runs 63 us against 128 (F(4,r)) and 164 (F(2,r)); C=K=256, 56x56 107 against 160;
+// 4x4 103 against 144; 5x5 at C=128 145 against 154.  Longer reductions favour the plans, whose saving in
+// multiplications grows with the kernel: 6x6 at C=128 200 against 182 us, 5x5 at C=256 257 against 194, 3x3 at
+// C=512 (14x14 images) 91 against 66.  With 64 output channels or fewer the direct form runs 64 x 64 tiles
+// only, which loses for kernels beyond 5x5 (7x7, C=K=64, 224x224: 387 against 371 us).
+static bool direct_preferred(const wc_conv_desc* d) {
+  const int taps = d->kernel[1] * d->kernel[2];
+  return (long long)taps * d->C <= 3200 && (d->K > 64 || taps <= 25);
+}
+
 int wc_conv_auto(wc_conv_desc* d) {
   WC_CHECK_ARG(d != nullptr, "wc_conv_auto: null descriptor");
   WC_CHECK_ARG(d->ndim == 2 || d->ndim == 3, "ndim must be 2 or 3, got %d", d->ndim);
   WC_CHECK_ARG(d->stacked >= -1 && d->stacked <= 2, "stacked must be -1 (choose), 0, 1 or 2");
-  if (d->stacked == -1) d->stacked = auto_stacked(d);
+  WC_CHECK_ARG(d->direct >= -1 && d->direct <= 1, "direct must be -1 (never), 0 (may be chosen) or 1");
+  const bool never_direct = d->direct == -1;
+  if (never_direct) d->direct = 0;
+  if (d->stacked == -1) {
+    if (d->stride == 2 && !d->direct && !never_direct && direct_conv_fits(d) && direct_preferred(d)) d->direct = 1;
+    d->stacked = d->direct ? 0 : auto_stacked(d);
+  }
   if (d->stacked == 2 && d->m == 4) {
     // the shared-input plan exists for output tiles 2 and 3: tile 3 (F(3,3): fp16 error 3e-3 of the output
     // range, between F(2,r) and F(4,r); too coarse for bf16) where its three-tap pieces apply, else 2

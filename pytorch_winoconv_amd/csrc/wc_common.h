@@ -126,8 +126,17 @@ int input_transform_nchw(const wc_conv_desc* d, const wc_plan* plan, const void*
 // src (n, R, Q) -> dst (n, Q, R), elements of 2 or 4 bytes (layout_copy.hip)
 int transpose_images(const void* src, void* dst, long long n, long long R, long long Q, int elem_size, void* stream);
 
+// Direct form (wc_conv_desc.direct; direct_conv.hip, gemm.hip): whether a problem is in its range, the copy of the
+// filter to U (K, kh, kw, C), and the product that reads x itself.
+bool direct_conv_fits(const wc_conv_desc* d);
+int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
+int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y, void* stream);
+int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,
+                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream);
+
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;
+constexpr int kCus = 256;                  // compute units of an MI355X
 
 // Maps the hardware workgroup id to a logical one so that each XCD owns one contiguous
 // range of logical ids (neighbouring tiles then share that XCD's L2).  `per_xcd` is

@@ -76,7 +76,7 @@ def _triple(v, nd, fill):
 
 
 def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0, whole_kernel=False, stacked=False,
-              unfused=False, x_layout=0, y_layout=0):
+              unfused=False, x_layout=0, y_layout=0, direct=None):
     """Descriptor for an NC[D]HW input and a (K, C, [kD,] kH, kW) filter.  `whole_kernel`: one
     F(2,k) tile per axis for a k x k kernel, k = 4..7, instead of the DWM pieces.  `stacked`: the
     DWM pieces share one tile and are added by the batched GEMM instead of by the output transform
@@ -104,6 +104,9 @@ def make_desc(x_shape, w_shape, dtype, stride=1, padding=0, m=2, chunk_images=0,
     d.chunk_images = int(chunk_images)
     d.whole_kernel = int(bool(whole_kernel))
     d.stacked = -1 if stacked is None else 2 if stacked == 2 else int(bool(stacked))
+    # the direct form (wc_conv_desc.direct): True asks for it, False rules it out, None leaves it to the library,
+    # which takes it for 16-bit stride-2 layers when `stacked` is left open too
+    d.direct = 1 if direct else (-1 if direct is False else 0)
     # what is left open is filled in by the library: the form of the plan if `stacked` is None, and the tile
     # 3 or 2 where a caller asked for tile 4 and gets the shared-input plan, which has no such tile (d.m then
     # tells the tile really used)
@@ -262,7 +265,7 @@ def _stack(stacked, dtype, nd, whole_kernel, w_shape=None, stride=1, m=2):
     d.N, d.C, d.K = 1, int(w_shape[1]), int(w_shape[0])
     d.kernel[:] = ((1,) if nd == 2 else ()) + tuple(int(v) for v in w_shape[2:])
     d.stride, d.m, d.dtype = int(stride), int(m), _DTYPES[dtype]
-    d.whole_kernel, d.stacked = int(bool(whole_kernel)), -1
+    d.whole_kernel, d.stacked, d.direct = int(bool(whole_kernel)), -1, -1     # the Winograd / DWM form, the direct one aside
     check(_lib.load().wc_conv_auto(ctypes.byref(d)))
     return 2 if d.stacked == 2 else bool(d.stacked)
 
@@ -312,16 +315,20 @@ def check_u(desc, U):
                          "(transform_filter must be called with the same options)" % (U.numel(), n.value))
 
 
-def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None):
+def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, stacked=None, direct=None):
     """Transformed filter U for later calls of conv_forward(..., U=U) with the same options."""
     _require_gpu(w)
-    stacked = _stack(stacked, w.dtype, len(x_shape) - 2, whole_kernel, w.shape, stride, m)
-    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked)
+    desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked, direct=direct)
+    if desc.direct:
+        U = torch.empty(desc.K, desc.kernel[1], desc.kernel[2], desc.C, dtype=w.dtype, device=w.device)
+        plan = Plan()
+        check(_lib.load().wc_filter_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(w), _w_strides(w), _ptr(U), _stream(w)))
+        return U
     return filter_transform(desc, plan_conv(desc), w)
 
 
 def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False,
-                 stacked=None, unfused=False, channels_first_out=False):
+                 stacked=None, unfused=False, channels_first_out=False, direct=None):
     """Winograd / DWM convolution of an NC[D]HW tensor.  Returns an NC[D]HW tensor whose memory
     is channel-last (torch.channels_last / channels_last_3d), or, with `channels_first_out`, plain
     contiguous.  A channel-last input is used without a copy; a contiguous (channel-first) one is
@@ -331,17 +338,16 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     `unfused=True` keeps thin 16-bit 3x3 layers on the three-kernel path (wc_conv_desc.unfused)."""
     if USE_EXT:
         return _ext.conv_forward(x, w, bias, stride, padding, m, U, chunk_images, bool(whole_kernel), stacked,
-                                 bool(unfused), bool(channels_first_out))
+                                 bool(unfused), bool(channels_first_out), direct)
     check_operands(x, int(w.shape[0]), bias, U)
     _require_gpu(x, w, bias, U)
-    stacked = _stack(stacked, x.dtype, x.dim() - 2, whole_kernel, w.shape, stride, m)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("input, filter and bias must share one dtype")
     lib = _lib.load()
     if x.shape[0] == 0:
         # empty batch: the shape arithmetic is checked on one image, nothing is launched
         out, _ = out_dims(make_desc((1,) + tuple(x.shape[1:]), w.shape, x.dtype, stride, padding, m, 0, whole_kernel,
-                                    stacked))
+                                    stacked, direct=direct))
         osp = out[1:] if x.dim() == 4 else out
         return channel_first_view(torch.empty([0] + osp + [w.shape[0]], dtype=x.dtype, device=x.device))
     # channel-last memory is used as it is, and so is contiguous channel-first memory (x_layout = 1)
@@ -358,7 +364,7 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     # (x[1:] of a channel-last tensor with 6 channels and 7 x 7 images is 4-byte aligned): three kernels then
     unfused = bool(unfused) or misaligned(x_mem, U)
     desc, y_shape, nbytes, u_elems = _forward_setup(tuple(x.shape), tuple(w.shape), x.dtype, stride, padding, m,
-                                                    chunk_images, whole_kernel, stacked, unfused, x_layout, y_layout)
+                                                    chunk_images, whole_kernel, stacked, unfused, x_layout, y_layout, direct)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     if y_layout:
         y = torch.empty([y_shape[0], y_shape[-1]] + y_shape[1:-1], dtype=x.dtype, device=x.device)
@@ -377,18 +383,18 @@ _SETUPS = {}
 
 
 def _forward_setup(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused=False,
-                   x_layout=0, y_layout=0):
+                   x_layout=0, y_layout=0, direct=None):
     """Descriptor, output shape (channel-last), workspace bytes and size of U for one problem.  Kept
     per problem: for small layers (a few tens of microseconds on the GPU) rebuilding them on every
     call costs as much host time as the launches themselves."""
     key = (x_shape, w_shape, dtype, stride if isinstance(stride, int) else tuple(stride),
            padding if isinstance(padding, int) else tuple(padding), m, chunk_images, whole_kernel, stacked, unfused,
-           x_layout, y_layout)
+           x_layout, y_layout, direct)
     hit = _SETUPS.get(key)
     if hit is None:
         lib = _lib.load()
         desc = make_desc(x_shape, w_shape, dtype, stride, padding, m, chunk_images, whole_kernel, stacked, unfused,
-                         x_layout, y_layout)
+                         x_layout, y_layout, direct)
         out, _ = out_dims(desc)
         nbytes, ue = ctypes.c_size_t(), ctypes.c_size_t()
         check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))

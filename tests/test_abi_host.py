@@ -451,3 +451,14 @@ def test_module_tables_equal_oracle_tables():
         assert np.allclose(pkg.matrix_conv.A[key], AT, atol=1e-16, rtol=0)
         assert np.allclose(pkg.matrix_conv.G[key], G, atol=1e-16, rtol=0)
         assert np.allclose(pkg.matrix_conv.B[key], BT, atol=1e-16, rtol=0)
+
+
+@pytest.mark.parametrize("C,K,k,chosen", [
+    (128, 128, 3, 1), (256, 256, 3, 1), (128, 128, 4, 1), (128, 128, 5, 1), (64, 64, 3, 1), (32, 64, 5, 1), (64, 128, 7, 1),
+    (512, 512, 3, 0), (256, 256, 5, 0), (128, 128, 6, 0), (128, 128, 7, 0), (64, 64, 7, 0), (32, 8, 7, 0)])
+def test_the_library_chooses_the_direct_form_for_short_reductions(C, K, k, chosen):
+    """kh kw C <= 3200, and kernels of at most 25 taps when K <= 64: the side of the measured crossover each
+    stride-2 layer of the sweep behind the rule fell on."""
+    d = engine.make_desc((2, C, 28, 28), (K, C, k, k), torch.float16, 2, k // 2, 2, stacked=None)
+    assert d.direct == chosen
+    assert engine.make_desc((2, C, 28, 28), (K, C, k, k), torch.bfloat16, 2, k // 2, 2, stacked=None).direct == chosen

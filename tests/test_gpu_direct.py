@@ -1,0 +1,112 @@
+"""The direct form (wc_conv_desc.direct): pieces of one tap on the tile F(1,1), i.e. the batched product reading the
+pixels of x itself with the taps along its reduction axis.  The library chooses it for 16-bit stride-2 layers (which
+the reference does not implement: src/winograd_conv.cpp:122-126) whose reduction kh kw C is short, where it measured
+faster than the parity-phase Winograd plans; on request it runs any 2-D kernel and stride.
+
+Pinned bit for bit on small integers (every product and sum exact), against fp64 torch convolution and the oracle on
+normal data, and against the Winograd / DWM plans of the same engine."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import winograd as ow
+from pytorch_winoconv_amd import engine
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # x shape, w shape, stride, pad
+    ((2, 32, 12, 13), (8, 32, 3, 3), 2, 1), ((3, 64, 21, 20), (24, 64, 3, 3), 2, 1), ((1, 32, 9, 9), (16, 32, 3, 3), 2, 0),
+    ((2, 32, 15, 14), (8, 32, 7, 7), 2, 3), ((1, 96, 17, 19), (40, 96, 5, 5), 2, 2), ((2, 32, 10, 11), (8, 32, 4, 6), 2, (1, 2)),
+    ((1, 128, 30, 30), (136, 128, 3, 3), 2, 1), ((2, 32, 8, 9), (8, 32, 1, 1), 2, 0), ((2, 32, 9, 10), (72, 32, 2, 2), 2, 0),
+    ((5, 64, 33, 31), (64, 64, 3, 3), 2, 1), ((1, 32, 7, 7), (8, 32, 7, 7), 2, 3), ((2, 32, 10, 10), (8, 32, 3, 3), 2, 3),
+    ((40, 32, 28, 28), (32, 32, 3, 3), 2, 1),     # enough output pixels for the largest tile
+    # stride 1 on request
+    ((2, 32, 9, 11), (8, 32, 3, 3), 1, 1), ((1, 64, 12, 12), (16, 64, 5, 5), 1, 2), ((1, 32, 8, 8), (8, 32, 1, 3), 1, (0, 1)),
+]
+
+
+def _rel(a, b):
+    return float((a.double().cpu() - b.double().cpu()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES)
+def test_exact_on_small_integers(dev, dtype, case, host_layer):
+    xs, ws, stride, pad = case
+    g = torch.Generator().manual_seed(1)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = torch.randint(-2, 3, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    ref = F.conv2d(x, w, b, stride=stride, padding=pad)
+    assert float(ref.abs().max()) < (2048 if dtype == torch.float16 else 256) * 8      # representable after the one rounding
+    y = engine.conv_forward(x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev), stride, pad, 2, direct=True)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert torch.equal(y.cpu(), ref.float().to(dtype))
+    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, stride, pad, "fp16" if dtype == torch.float16 else "bf16"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES)
+def test_against_fp64_the_oracle_and_the_winograd_plans(dev, dtype, case):
+    xs, ws, stride, pad = case
+    g = torch.Generator().manual_seed(2)
+    fan = ws[1] * ws[2] * ws[3]
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), b.double(), stride=stride, padding=pad)
+    xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
+    y = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=True)
+    tol = 2e-3 if dtype == torch.float16 else 1.2e-2            # one rounding of an fp32 sum
+    assert _rel(y, ref) <= tol
+    assert _rel(y, ow.direct_conv(x, w, b, stride, pad, "fp16" if dtype == torch.float16 else "bf16")) <= tol
+    yw = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=False)          # the Winograd / DWM plan
+    assert _rel(yw, ref) <= 2e-2 and _rel(y, yw.cpu()) <= 2e-2
+    # the library's own choice is one of the two; at stride 1 it is never the direct form
+    chosen = engine.make_desc(xs, ws, dtype, stride, pad, 2, stacked=None).direct
+    assert stride == 2 or chosen == 0
+    ya = engine.conv_forward(xd, wd, bd, stride, pad, 2)
+    assert torch.equal(ya, y if chosen else yw)
+    # cached filter, no bias, channel-first in and out, one image per pass
+    U = engine.transform_filter(wd, xs, stride, pad, 2, direct=True)
+    assert tuple(U.shape) == (ws[0], ws[2], ws[3], ws[1])
+    assert torch.equal(U, wd.permute(0, 2, 3, 1).contiguous())
+    assert torch.equal(engine.conv_forward(xd, wd, bd, stride, pad, 2, U=U, direct=True), y)
+    assert _rel(engine.conv_forward(xd, wd, None, stride, pad, 2, direct=True), F.conv2d(x.double(), w.double(), None, stride=stride, padding=pad)) <= tol
+    xcl = xd.contiguous(memory_format=torch.channels_last)
+    ycf = engine.conv_forward(xcl, wd, bd, stride, pad, 2, direct=True, channels_first_out=True, chunk_images=1)
+    assert ycf.is_contiguous() and torch.equal(ycf, y)
+
+
+def test_outside_its_range_the_direct_form_is_refused_or_not_chosen(dev):
+    x = torch.randn(2, 20, 12, 12, device=dev).half()
+    w = torch.randn(8, 20, 3, 3, device=dev).half()
+    with pytest.raises(NotImplementedError, match="direct form"):
+        engine.conv_forward(x, w, None, 2, 1, 2, direct=True)                   # 20 channels: no multiple of 32
+    assert engine.make_desc(x.shape, w.shape, torch.float16, 2, 1, 2, stacked=None).direct == 0
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None).direct == 1
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 1, 1, 2, stacked=None).direct == 0      # stride 1
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float32, 2, 1, 2, stacked=None).direct == 0      # fp32
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None, direct=False).direct == 0
+    assert engine.make_desc((2, 32, 12, 12), (12, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None).direct == 0     # K no multiple of 8
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=True).direct == 0      # an explicit plan form
+
+
+def test_c4_stride_2_layers_at_full_size(dev):
+    """N=32, 128 channels, 112x112, 3x3 and 7x7 at stride 2, the library's choice (direct for 3x3, the parity-phase
+    plan for 7x7) and the direct form on request: the last image against fp64 on the CPU, and a permuted batch
+    gives the permuted output bit for bit."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(32, 128, 112, 112, generator=g).half()
+    xd = x.to(dev).contiguous(memory_format=torch.channels_last)
+    for k, pad in ((3, 1), (7, 3)):
+        w = (torch.randn(128, 128, k, k, generator=g) * (2.0 / (128 * k * k)) ** 0.5).half()
+        assert engine.make_desc(x.shape, w.shape, torch.float16, 2, pad, 2, stacked=None).direct == (1 if k == 3 else 0)
+        ref = F.conv2d(x[31:].double(), w.double(), stride=2, padding=pad)
+        perm = torch.randperm(32, generator=g).to(dev)
+        xp = xd[perm].contiguous(memory_format=torch.channels_last)
+        for direct, tol in ((None, 2e-3 if k == 3 else 1e-2), (True, 2e-3)):
+            y = engine.conv_forward(xd, w.to(dev), None, 2, pad, 2, direct=direct)
+            assert _rel(y[31:], ref) <= tol
+            assert torch.equal(engine.conv_forward(xp, w.to(dev), None, 2, pad, 2, direct=direct), y[perm])
