@@ -229,6 +229,26 @@ int wc_conv_forward(const wc_conv_desc* desc, const void* x,
                     const void* bias, void* y, void* workspace, size_t workspace_bytes,
                     void* stream);
 
+/* wc_conv_forward with the time every stage took on the device: a pair of events around each stage on `stream`,
+ * read after the stream has been waited for, so the call returns when the convolution is done (opt-in: it
+ * serialises the host with the device).  Replaces the perf_counter / synchronize pairs the reference puts
+ * around its phases (dwm.py:44-106).  stage_ms[s] is the sum over the image chunks; stages that did not run
+ * read 0.  The one-kernel forms (thin layers, the direct form) count as WC_STAGE_PRODUCT.  Same results
+ * as wc_conv_forward, bit for bit. */
+enum {
+  WC_STAGE_FILTER = 0,      /* filter transform (0 with U_cached) */
+  WC_STAGE_LAYOUT_IN = 1,   /* channel-first x copied to channel-last scratch */
+  WC_STAGE_INPUT = 2,       /* input transform */
+  WC_STAGE_PRODUCT = 3,     /* batched GEMM, or the one fused kernel */
+  WC_STAGE_OUTPUT = 4,      /* output transform */
+  WC_STAGE_LAYOUT_OUT = 5,  /* channel-last scratch copied to channel-first y */
+  WC_N_STAGES = 6
+};
+int wc_conv_forward_timed(const wc_conv_desc* desc, const void* x,
+                          const void* w, const int64_t w_strides[5], const void* U_cached,
+                          const void* bias, void* y, void* workspace, size_t workspace_bytes,
+                          void* stream, float stage_ms[WC_N_STAGES]);
+
 /* wc_conv_forward without a workspace argument.  No counterpart in the reference; it is for callers
  * that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  U, V and M live in a buffer of WC_STATIC_SCRATCH_BYTES inside the

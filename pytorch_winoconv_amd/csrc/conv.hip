@@ -12,6 +12,7 @@
 
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 using namespace wc;
 
@@ -125,6 +126,46 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   return WC_OK;
 }
 
+// Opt-in timing of the stages of one call: a pair of events around every stage on the caller's stream, read
+// after one synchronisation at the end (the reference times its phases with perf_counter and device-wide
+// synchronisations around each: dwm.py:44-106).
+struct StageTimer {
+  struct Span { int stage; hipEvent_t t0, t1; };
+  std::vector<Span> spans;
+  hipStream_t stream;
+  bool on;
+  StageTimer(bool enabled, void* s) : stream(as_stream(s)), on(enabled) {}
+  ~StageTimer() {
+    for (Span& sp : spans) { (void)hipEventDestroy(sp.t0); (void)hipEventDestroy(sp.t1); }
+  }
+  template <typename F>
+  int run(int stage, F&& f) {
+    if (!on) return f();
+    Span sp; sp.stage = stage;
+    if (hipEventCreate(&sp.t0) != hipSuccess) return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipEventCreate failed");
+    if (hipEventCreate(&sp.t1) != hipSuccess) { (void)hipEventDestroy(sp.t0); return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipEventCreate failed"); }
+    spans.push_back(sp);
+    if (hipEventRecord(sp.t0, stream) != hipSuccess) return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipEventRecord failed");
+    const int rc = f();
+    if (hipEventRecord(sp.t1, stream) != hipSuccess) return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipEventRecord failed");
+    return rc;
+  }
+  int collect(float* stage_ms) {
+    for (int i = 0; i < WC_N_STAGES; ++i) stage_ms[i] = 0.f;
+    if (hipStreamSynchronize(stream) != hipSuccess) return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipStreamSynchronize failed");
+    for (Span& sp : spans) {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, sp.t0, sp.t1) != hipSuccess) return fail(WC_ERR_HIP, "wc_conv_forward_timed: hipEventElapsedTime failed");
+      stage_ms[sp.stage] += ms;
+    }
+    return WC_OK;
+  }
+};
+
+int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
+                 const void* U_cached, const void* bias, void* y, void* workspace,
+                 size_t workspace_bytes, void* stream, float* stage_ms);
+
 }  // namespace
 
 extern "C" {
@@ -150,6 +191,23 @@ int wc_conv_u_elems(const wc_conv_desc* d, size_t* elems) {
 int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
                     const void* U_cached, const void* bias, void* y, void* workspace,
                     size_t workspace_bytes, void* stream) {
+  return forward_impl(d, x, w, w_strides, U_cached, bias, y, workspace, workspace_bytes, stream, nullptr);
+}
+
+int wc_conv_forward_timed(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
+                          const void* U_cached, const void* bias, void* y, void* workspace,
+                          size_t workspace_bytes, void* stream, float stage_ms[WC_N_STAGES]) {
+  WC_CHECK_ARG(stage_ms != nullptr, "wc_conv_forward_timed: null stage_ms");
+  return forward_impl(d, x, w, w_strides, U_cached, bias, y, workspace, workspace_bytes, stream, stage_ms);
+}
+
+}  // extern "C"
+
+namespace {
+
+int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
+                 const void* U_cached, const void* bias, void* y, void* workspace,
+                 size_t workspace_bytes, void* stream, float* stage_ms) {
   Layout L;
   int rc = make_layout(d, &L);
   if (rc) return rc;
@@ -170,10 +228,10 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
                  d->ndim, dt[d->dtype], d->N, d->C, d->K, d->in[0], d->in[1], d->in[2], d->kernel[0], d->kernel[1], d->kernel[2],
                  d->stride, d->pad[0], d->pad[1], d->pad[2], L.plan.m[0], L.plan.m[1], L.plan.m[2], L.plan.n_pieces, L.plan.t_total,
                  d->stacked, d->whole_kernel ? " whole-kernel tile" : "",
-                 L.thin ? "one fused kernel" : (L.shared ? "input transform, shifted batched GEMM, output transform"
+                 L.direct ? "direct form: the product reads x" : L.thin ? "one fused kernel" : (L.shared ? "input transform, shifted batched GEMM, output transform"
                                                          : "input transform, batched GEMM, output transform"),
-                 L.thin ? d->N : L.chunk, L.tiles_per_image, need, L.u_bytes, L.thin ? (size_t)0 : L.v_bytes,
-                 L.thin ? (size_t)0 : L.m_bytes, L.xcl_bytes, L.ycl_bytes,
+                 L.thin || L.direct ? d->N : L.chunk, L.tiles_per_image, need, L.u_bytes, L.thin || L.direct ? (size_t)0 : L.v_bytes,
+                 L.thin || L.direct ? (size_t)0 : L.m_bytes, L.xcl_bytes, L.ycl_bytes,
                  d->x_layout ? (L.x_direct ? "channel-first, read by the input transform" : "channel-first, copied") : "channel-last",
                  d->y_layout ? "channel-first, copied" : "channel-last", U_cached ? "transformed by the caller" : "transformed here");
   }
@@ -184,9 +242,10 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
   unsigned char* tail = ws + (L.thin || L.direct ? L.u_bytes : L.u_bytes + L.v_bytes + L.m_bytes);
   void* Xcl = tail;                       // channel-last copies of channel-first tensors, one chunk each
   void* Ycl = tail + L.xcl_bytes;
+  StageTimer timer(stage_ms != nullptr, stream);
   const void* U = U_cached;
   if (!U) {
-    rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
+    rc = timer.run(WC_STAGE_FILTER, [&] { return wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream); });
     if (rc) return rc;
     U = Uws;
   }
@@ -203,36 +262,42 @@ int wc_conv_forward(const wc_conv_desc* d, const void* x, const void* w, const i
     const void* xin = static_cast<const unsigned char*>(x) + b0 * x_image;
     void* yout = static_cast<unsigned char*>(y) + b0 * y_image;
     if (L.xcl_bytes) {
-      rc = transpose_images(xin, Xcl, n, d->C, in_pos, (int)L.es, stream);
+      rc = timer.run(WC_STAGE_LAYOUT_IN, [&] { return transpose_images(xin, Xcl, n, d->C, in_pos, (int)L.es, stream); });
       if (rc) return rc;
       xin = Xcl;
     }
     void* ydst = L.ycl_bytes ? Ycl : yout;
     if (L.direct) {
-      rc = direct_conv(&dcl, xin, n, U, bias, ydst, stream);
+      rc = timer.run(WC_STAGE_PRODUCT, [&] { return direct_conv(&dcl, xin, n, U, bias, ydst, stream); });
       if (rc) return rc;
     } else if (L.thin) {
       // thin F(2x2, 3x3) layers: one kernel, no V and M
-      rc = thin_conv_forward(&dcl, &L.plan, xin, U, bias, ydst, stream);
+      rc = timer.run(WC_STAGE_PRODUCT, [&] { return thin_conv_forward(&dcl, &L.plan, xin, U, bias, ydst, stream); });
       if (rc) return rc;
     } else {
       const long long P = L.tiles_per_image * n;
       WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
-      rc = wc_input_transform(&dcl, &L.plan, xin, n, V, stream);
+      rc = timer.run(WC_STAGE_INPUT, [&] { return wc_input_transform(&dcl, &L.plan, xin, n, V, stream); });
       if (rc) return rc;
-      rc = L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
-                    : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+      rc = timer.run(WC_STAGE_PRODUCT, [&] {
+        return L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
+                        : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+      });
       if (rc) return rc;
-      rc = wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream);
+      rc = timer.run(WC_STAGE_OUTPUT, [&] { return wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream); });
       if (rc) return rc;
     }
     if (L.ycl_bytes) {
-      rc = transpose_images(Ycl, yout, n, out_pos, d->K, (int)L.es, stream);
+      rc = timer.run(WC_STAGE_LAYOUT_OUT, [&] { return transpose_images(Ycl, yout, n, out_pos, d->K, (int)L.es, stream); });
       if (rc) return rc;
     }
   }
-  return WC_OK;
+  return stage_ms ? timer.collect(stage_ms) : WC_OK;
 }
+
+}  // namespace
+
+extern "C" {
 
 int wc_conv_forward_static(const wc_conv_desc* d, const void* x, const void* w, const int64_t w_strides[5],
                            const void* U_cached, const void* bias, void* y, void* stream) {

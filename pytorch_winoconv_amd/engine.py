@@ -339,6 +339,25 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
     if USE_EXT:
         return _ext.conv_forward(x, w, bias, stride, padding, m, U, chunk_images, bool(whole_kernel), stacked,
                                  bool(unfused), bool(channels_first_out), direct)
+    return _conv_forward(x, w, bias, stride, padding, m, U, chunk_images, whole_kernel, stacked, unfused,
+                         channels_first_out, direct, None)
+
+
+STAGES = ("filter_transform", "layout_in", "input_transform", "product", "output_transform", "layout_out")
+
+
+def conv_forward_timed(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images=0, whole_kernel=False,
+                       stacked=None, unfused=False, channels_first_out=False, direct=None):
+    """conv_forward through wc_conv_forward_timed: returns (y, {stage: milliseconds on the device}) with the
+    stages of STAGES; waits for the device (the reference's timing prints: dwm.py:44-106)."""
+    times = (ctypes.c_float * len(STAGES))()
+    y = _conv_forward(x, w, bias, stride, padding, m, U, chunk_images, whole_kernel, stacked, unfused,
+                      channels_first_out, direct, times)
+    return y, dict(zip(STAGES, (float(t) for t in times)))
+
+
+def _conv_forward(x, w, bias, stride, padding, m, U, chunk_images, whole_kernel, stacked, unfused,
+                  channels_first_out, direct, times):
     check_operands(x, int(w.shape[0]), bias, U)
     _require_gpu(x, w, bias, U)
     if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
@@ -374,8 +393,12 @@ def conv_forward(x, w, bias=None, stride=1, padding=0, m=2, U=None, chunk_images
         bias = bias.contiguous()
     if U is not None and (not U.is_contiguous() or U.numel() != u_elems):
         check_u(desc, U)                                  # raises with the sizes in the message
-    check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_mem), _ptr(w), _w_strides(w), _ptr(U),
-                              _ptr(bias), _ptr(y), _ptr(ws), nbytes, _stream(x)))
+    if times is None:
+        check(lib.wc_conv_forward(ctypes.byref(desc), _ptr(x_mem), _ptr(w), _w_strides(w), _ptr(U),
+                                  _ptr(bias), _ptr(y), _ptr(ws), nbytes, _stream(x)))
+    else:
+        check(lib.wc_conv_forward_timed(ctypes.byref(desc), _ptr(x_mem), _ptr(w), _w_strides(w), _ptr(U),
+                                        _ptr(bias), _ptr(y), _ptr(ws), nbytes, _stream(x), times))
     return y if y_layout else channel_first_view(y)
 
 

@@ -260,3 +260,35 @@ def test_plan_dump_with_winoconv_log(dev):
         if expect:
             assert "tile m=1,3,3" in lines[0] and "pieces=9" in lines[0] and "stacked=2" in lines[0]
             assert "shifted batched GEMM" in lines[0] and "channel-first, copied" in lines[0]
+
+
+@pytest.mark.parametrize("case", [
+    # x shape, w shape, stride, pad, m, channel-first tensors, cached filter -> the stages that must have run
+    ((4, 48, 20, 22), (40, 48, 3, 3), 1, 1, 4, False, False, {"filter_transform", "input_transform", "product", "output_transform"}),
+    ((4, 48, 20, 22), (40, 48, 3, 3), 1, 1, 4, False, True, {"input_transform", "product", "output_transform"}),
+    ((2, 32, 18, 18), (16, 32, 5, 5), 1, 2, 2, True, False, set(pkg.engine.STAGES)),
+    ((4, 64, 20, 22), (64, 64, 3, 3), 1, 1, 2, False, False, {"filter_transform", "product"}),            # one fused kernel
+    ((4, 64, 20, 22), (64, 64, 3, 3), 2, 1, 2, False, False, {"filter_transform", "product"}),            # the direct form
+])
+def test_timed_forward_reports_the_stages_that_ran(dev, case):
+    """wc_conv_forward_timed: bit for bit the result of wc_conv_forward, a positive time for every stage the
+    plan runs and zero for the others, and together no more than the wall time of the call."""
+    import time
+    xs, ws, stride, pad, m, channel_first, cached, ran = case
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(*xs, generator=g).half().to(dev)
+    if not channel_first:
+        x = x.contiguous(memory_format=torch.channels_last)
+    w = torch.randn(*ws, generator=g).half().to(dev)
+    U = pkg.engine.transform_filter(w, xs, stride, pad, m) if cached else None
+    want = pkg.engine.conv_forward(x, w, None, stride, pad, m, U=U, channels_first_out=channel_first)
+    pkg.engine.conv_forward_timed(x, w, None, stride, pad, m, U=U, channels_first_out=channel_first)    # warm
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    y, times = pkg.engine.conv_forward_timed(x, w, None, stride, pad, m, U=U, channels_first_out=channel_first)
+    wall_ms = (time.perf_counter() - t0) * 1e3            # the call returns after the device has finished
+    assert torch.equal(y, want)
+    assert set(times) == set(pkg.engine.STAGES)
+    for name, ms in times.items():
+        assert (ms > 0) == (name in ran), (name, ms)
+    assert sum(times.values()) <= wall_ms
