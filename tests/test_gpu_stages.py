@@ -32,6 +32,8 @@ def _rel(a, b):
     ((1, 136, 9, 11, 13), (3, 136, 3, 3, 3), 2),     # 4 x 4 x 4 tiles
     ((1, 16, 7, 20, 22), (3, 16, 3, 3, 3), 4),       # 6 x 6 x 6 tiles: few tiles fit the staging buffer
     ((3, 256, 14, 14), (3, 256, 1, 1), 2),           # 2 x 2 tiles without overlap
+    ((1, 72, 20, 61), (3, 72, 3, 3), 4),             # 6 x 6 tiles, 15 per row (8 + 7), odd width, partial channel chunk
+    ((2, 128, 18, 35), (3, 128, 3, 3), 2),           # 4 x 4 tiles, 17 per row (8 + 8 + 1)
 ])
 def test_wino_split_bit_exact(dev, dtype, shape, wshape, m):
     torch.manual_seed(1)
@@ -46,7 +48,7 @@ def test_wino_split_bit_exact(dev, dtype, shape, wshape, m):
 @pytest.mark.parametrize("osize,K,B,m", [
     ((7, 9), 5, 2, 2), ((8, 8), 70, 1, 2), ((13, 10), 64, 2, 4), ((5, 7, 6), 6, 2, 2), ((4, 4, 5), 130, 1, 2),
     ((37, 41), 64, 2, 2), ((30, 19), 72, 1, 4), ((21, 23), 8, 2, 2), ((9, 11, 13), 136, 1, 2), ((7, 20, 22), 16, 1, 4),
-    ((56, 56), 256, 2, 4),
+    ((56, 56), 256, 2, 4), ((30, 61), 72, 1, 4), ((17, 35), 128, 2, 2),
 ])
 def test_wino_concat_bit_exact(dev, dtype, osize, K, B, m):
     torch.manual_seed(2)
