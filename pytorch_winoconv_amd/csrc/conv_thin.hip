@@ -83,23 +83,19 @@ struct ThinArgs {
   FastDiv div_nW, div_nH;
 };
 
-// Bias and store of one lane's share of an output tile: tile p, output channels ko .. ko + 4, the 2 x 2
-// output positions in out[oa][ob].  Stores go through a buffer descriptor: an output position outside
-// (oH, oW) gets an offset beyond the buffer and is dropped.
-template <typename T>
-__device__ __forceinline__ void store_tile(const ThinArgs& a, __amdgpu_buffer_rsrc_t ydesc, int p, int ko,
-                                           const floatx4 (&out)[2][2]) {
+// Store of one lane's share of an output tile: tile p, output channels ko .. ko + 4, the 2 x 2 output positions
+// in out[oa][ob], bias bv added.  Stores go through a buffer descriptor and are issued unconditionally: a
+// position outside (oH, oW), a tile beyond the last or a lane without work (`live` false) gets an offset beyond
+// the buffer and is dropped by the hardware.  No branch around the stores matters for speed: loads and stores
+// share one in-order counter, and only with straight-line code can the wait for the next block's window leave
+// this block's stores in flight.
+template <typename T, bool KW>
+__device__ __forceinline__ void store_tile(const ThinArgs& a, __amdgpu_buffer_rsrc_t ydesc, int p, int ko, bool live,
+                                           const float (&bv)[4], const floatx4 (&out)[2][2]) {
   const int q = fast_div(p, a.div_nW);
   const int tw = p - q * a.nW;
   const int b = fast_div(q, a.div_nH);
   const int th = q - b * a.nH;
-  const T* bias = static_cast<const T*>(a.bias);
-  float bv[4] = {0.f, 0.f, 0.f, 0.f};
-  if (bias) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (ko + r < a.K) bv[r] = static_cast<float>(bias[ko + r]);
-  }
   const unsigned o00 = (((unsigned)b * a.oH + 2 * th) * a.oW + 2 * tw) * a.K + ko;   // in elements
   const bool h1 = 2 * th + 1 < a.oH, w1 = 2 * tw + 1 < a.oW;
 #pragma unroll
@@ -107,12 +103,12 @@ __device__ __forceinline__ void store_tile(const ThinArgs& a, __amdgpu_buffer_rs
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
       const floatx4 s4 = out[oa][ob];
-      const bool inside = (oa == 0 || h1) && (ob == 0 || w1);
+      const bool inside = live && (oa == 0 || h1) && (ob == 0 || w1);
       const unsigned off = o00 + (oa * a.oW + ob) * a.K;
       Pack<T, 4> o;
 #pragma unroll
       for (int r = 0; r < 4; ++r) o.v[r] = static_cast<T>(s4[r] + bv[r]);
-      if (a.k_whole) {
+      if constexpr (KW) {
         const unsigned byte_off = inside ? off * (unsigned)sizeof(T) : kOutside;
         if constexpr (sizeof(T) == 4) {
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o), ydesc, byte_off, 0, 0);
@@ -134,6 +130,14 @@ __device__ __forceinline__ void store_tile(const ThinArgs& a, __amdgpu_buffer_rs
   }
 }
 
+// The bias of a lane's four output channels, loaded once per kernel.
+template <typename T>
+__device__ __forceinline__ void load_bias(const ThinArgs& a, int ko, float (&bv)[4]) {
+  const T* bias = static_cast<const T*>(a.bias);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) bv[r] = bias && ko + r < a.K ? static_cast<float>(bias[ko + r]) : 0.f;
+}
+
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
 // B^T of F(2,3) along one axis of a 4 x 4 block (STRIDE: distance between the four elements,
@@ -153,7 +157,9 @@ static_assert(Mats<KIND_23>::bt(0, 0) == 1 && Mats<KIND_23>::bt(0, 2) == -1 && M
               Mats<KIND_23>::bt(1, 2) == 1 && Mats<KIND_23>::bt(2, 1) == -1 && Mats<KIND_23>::bt(2, 2) == 1 &&
               Mats<KIND_23>::bt(3, 1) == 1 && Mats<KIND_23>::bt(3, 3) == -1, "B^T of F(2,3)");
 
-template <typename T, int CP>
+// KW: K is a multiple of 4, a lane's 4 output channels go out in one store (a compile-time choice: a branch
+// around the stores, even a uniform one, makes the compiler wait for all memory operations at the loop top)
+template <typename T, int CP, bool KW>
 __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
   // Up to 64 channels a wavefront holds U of all 16 elements (4 wavefronts).  With 128 that is twice
   // the register file, so SPLIT: 8 wavefronts, the upper four take the element rows 2 and 3 and hand
@@ -165,7 +171,16 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
   constexpr int VEC = kThinTiles * CP / NT;   // channels per thread in the transform
   constexpr int CVECS = CP / VEC;
   constexpr int KS = CP / (4 * EPF);      // fragment steps along the channels (four lane groups x EPF channels each)
-  constexpr int PITCH = CP * sizeof(T) + 16;   // bytes per (element, tile) row in LDS; the pad spreads 16 rows over all banks
+  // Bytes per (element, tile) row in LDS: no padding; the 16-byte chunks of a row are permuted by the row instead.
+  // A fragment read takes one chunk from each of 16 consecutive rows; the LDS of this part delivers 16-byte reads
+  // at 256 bytes per clock only if those 16 chunks fall into 16 different 16-byte columns of a 256-byte line
+  // (rows padded by 16 bytes, which are conflict-free for 128-byte wide LDS, measured half that rate).  With R rows
+  // per 256 bytes, chunk c of row r sits at position c ^ ((r / R) mod chunks per row).
+  constexpr int PITCH = CP * sizeof(T);
+  constexpr int CPRW = PITCH / 16;             // chunks per row: 4, 8 or 16
+  constexpr int RPL = 16 / CPRW;               // rows per 256-byte line
+  static_assert(CPRW == 4 || CPRW == 8 || CPRW == 16, "rows of 64, 128 or 256 bytes");
+  static_assert(VEC * sizeof(T) <= 16, "a thread's channels stay inside one chunk");
   constexpr int BUF = 16 * kThinTiles * PITCH;
   using MF = Mfma16<T>;
   using Frag = typename MF::Frag;
@@ -232,12 +247,25 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     });
   }
 
+  // U and the bias have arrived before the loop starts: a wait for them inside the loop would also wait, on
+  // every pass, for the window loads of the next block, which are younger (loads return in order).
+  float bv[4];
+  load_bias<T>(a, kbase + 4 * (lane >> 4), bv);
+#pragma unroll
+  for (int t = 0; t < NROW * 4; ++t)
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) asm volatile("" : "+v"(u[t][s2]));
+#pragma unroll
+  for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(bv[r]));
+
   for (int it = 0; blk < a.n_blocks; blk += nwg, ++it) {
     unsigned char* buf = lds + (it & 1) * BUF;
     // Input transform, two channels at a time.  fp16 adds pairs of channels
     // in fp16 like the reference's kernels (calculation_kernels.cu:786-806 computes in T); bf16,
     // which has no packed add, goes through fp32.
-    T* vdst = reinterpret_cast<T*>(buf + pl * PITCH) + c;
+    // all channels of this thread lie in one chunk
+    const int cb = c * (int)sizeof(T);
+    T* vdst = reinterpret_cast<T*>(buf + pl * PITCH + ((((cb >> 4) ^ ((pl / RPL) & (CPRW - 1))) << 4) | (cb & 15)));
     static_for<0, VEC / 2>([&](auto h_) {
       constexpr int h = decltype(h_)::value;
       if constexpr (std::is_same<T, half_t>::value) {
@@ -273,7 +301,8 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     floatx4 z0[NROW], zp[NROW], zn[NROW];
 #pragma unroll
     for (int i = 0; i < NROW; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-    const unsigned char* vrow = buf + (lane & 15) * PITCH + 16 * (lane >> 4) + row0i * 4 * kThinTiles * PITCH;
+    const unsigned char* vrow = buf + (lane & 15) * PITCH + row0i * 4 * kThinTiles * PITCH;
+    const int vswz = ((lane & 15) / RPL) & (CPRW - 1);
     static_for<0, KS>([&](auto s_) {
       constexpr int s = decltype(s_)::value;
       static_for<0, 4>([&](auto j_) {
@@ -281,7 +310,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
         Frag v[NROW];
         static_for<0, NROW>([&](auto i_) {
           constexpr int i = decltype(i_)::value;
-          v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + s * 64);
+          v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + ((((lane >> 4) + 4 * s) ^ vswz) << 4));
         });
         static_for<0, NROW>([&](auto i_) {
           constexpr int i = decltype(i_)::value;
@@ -331,7 +360,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     // lane = tile lane % 16, output channels ko .. ko + 4
     const int p = blk * kThinTiles + (lane & 15);
     const int ko = kbase + 4 * (lane >> 4);
-    if (p < a.P && ko < a.K && (!SPLIT || wave < 4)) store_tile<T>(a, ydesc, p, ko, out);
+    store_tile<T, KW>(a, ydesc, p, ko, p < a.P && ko < a.K && (!SPLIT || wave < 4), bv, out);
   }
 }
 
@@ -341,7 +370,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
 // v_mfma_f32_16x16x4_f32 in fp32 with a reduction of exactly 4 channels, U (16 elements x 16 output
 // channels x 4) is 16 registers per lane, and a block is 64 tiles: a thread transforms one channel of
 // one tile, a wavefront multiplies four column blocks of 16 tiles.
-template <typename T>
+template <typename T, bool KW>
 __global__ __launch_bounds__(256) void tiny_conv3x3_kernel(ThinArgs a) {
   constexpr int TILES = 64;
   constexpr int BUF = 16 * TILES * 4;     // floats per buffer, [element][tile][channel]
@@ -392,6 +421,13 @@ __global__ __launch_bounds__(256) void tiny_conv3x3_kernel(ThinArgs a) {
     for (int t = 0; t < 16; ++t) u[t] = static_cast<float>(U[(long long)t * a.K * a.Cp]);
   }
 
+  float bv[4];
+  load_bias<T>(a, kbase + 4 * (lane >> 4), bv);
+#pragma unroll
+  for (int t = 0; t < 16; ++t) asm volatile("" : "+v"(u[t]));
+#pragma unroll
+  for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(bv[r]));
+
   for (int it = 0; blk < a.n_blocks; blk += nwg, ++it) {
     float* buf = ldsf + (it & 1) * BUF;
     {
@@ -437,7 +473,7 @@ __global__ __launch_bounds__(256) void tiny_conv3x3_kernel(ThinArgs a) {
       }
       const int p = blk * TILES + cb * 16 + (lane & 15);
       const int ko = kbase + 4 * (lane >> 4);
-      if (p < a.P && ko < a.K) store_tile<T>(a, ydesc, p, ko, out);
+      store_tile<T, KW>(a, ydesc, p, ko, p < a.P && ko < a.K, bv, out);
     }
   }
 }
@@ -448,8 +484,12 @@ int launch_tiny(ThinArgs a, int k_groups, void* stream) {
   a.n_blocks = ceil_div(a.P, 64);
   int wgs = std::min(a.n_blocks, std::max(kXcds, 1024 / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
-  hipLaunchKernelGGL((tiny_conv3x3_kernel<T>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256), lds,
-                     as_stream(stream), a);
+  if (a.k_whole)
+    hipLaunchKernelGGL((tiny_conv3x3_kernel<T, true>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256), lds,
+                       as_stream(stream), a);
+  else
+    hipLaunchKernelGGL((tiny_conv3x3_kernel<T, false>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups), dim3(256), lds,
+                       as_stream(stream), a);
   WC_CHECK_LAUNCH("tiny_conv3x3_kernel");
   return WC_OK;
 }
@@ -457,13 +497,14 @@ int launch_tiny(ThinArgs a, int k_groups, void* stream) {
 template <typename T, int CP>
 int launch_thin(ThinArgs a, int k_groups, void* stream) {
   constexpr bool split = CP * sizeof(T) > 128;
-  constexpr int lds = 2 * 16 * kThinTiles * (CP * (int)sizeof(T) + 16) + (split ? 4 * 4 * 64 * 16 : 0);
+  constexpr int lds = 2 * 16 * kThinTiles * CP * (int)sizeof(T) + (split ? 4 * 4 * 64 * 16 : 0);
   // workgroups that stay resident (registers and LDS): two per CU, one of the eight-wavefront form;
   // shared among the groups of output channels, in whole multiples of the 8 XCDs
   int wgs = std::min(a.n_blocks, std::max(kXcds, (split ? 256 : 512) / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
-  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&thin_conv3x3_kernel<T, CP>), lds)) return rc;
-  hipLaunchKernelGGL((thin_conv3x3_kernel<T, CP>), dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups),
+  auto fn = a.k_whole ? &thin_conv3x3_kernel<T, CP, true> : &thin_conv3x3_kernel<T, CP, false>;
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
+  hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups),
                      dim3(split ? 512 : 256), lds, as_stream(stream), a);
   WC_CHECK_LAUNCH("thin_conv3x3_kernel");
   return WC_OK;
