@@ -165,6 +165,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
   // the register file, so SPLIT: 8 wavefronts, the upper four take the element rows 2 and 3 and hand
   // their share of the output tile to the lower four through LDS.
   constexpr bool SPLIT = CP * sizeof(T) > 128;       // 128 channels of a 16-bit type, 64 of fp32
+  constexpr bool PLAIN = sizeof(T) == 4;             // one accumulator per element, width transform in VALU (measured: no gain for 16-bit types)
   constexpr int EPF = 16 / sizeof(T);                // channels per 16-byte fragment
   constexpr int NT = SPLIT ? 512 : 256;
   constexpr int NROW = SPLIT ? 2 : 4;     // element rows per wavefront
@@ -295,46 +296,80 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     __syncthreads();
     if (blk + nwg < a.n_blocks) load_window(blk + nwg);
 
-    // Width half of the output transform in the accumulators, M[i][j] = U[i][j] V[i][j] over the channels:
-    // z0[i] = M[i][0] + M[i][1] + M[i][2], and M[i][1] - (M[i][2] + M[i][3]) as zp[i] - zn[i] (no operand
-    // needs its sign changed).  Consecutive MFMAs write different accumulators.
-    floatx4 z0[NROW], zp[NROW], zn[NROW];
-#pragma unroll
-    for (int i = 0; i < NROW; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // The products M[i][j] = U[i][j] V[i][j] over the channels, and the width half of the output transform,
+    // zw[i][0] = M[i][0] + M[i][1] + M[i][2], zw[i][1] = M[i][1] - M[i][2] - M[i][3].  16-bit types do the sums in
+    // the accumulators (z0 takes j = 0, 1, 2; zp takes j = 1 and zn j = 2, 3, so that no operand needs its sign
+    // changed): 24 MFMAs per channel step instead of 16, 12 accumulators instead of 16, no VALU work - their
+    // MFMAs are cheap and registers are what is short.  fp32, whose MFMAs are sixteen times slower and bound the
+    // kernel, keeps one accumulator per element and adds in VALU.  Consecutive MFMAs write different accumulators.
+    floatx4 zw[NROW][2];
     const unsigned char* vrow = buf + (lane & 15) * PITCH + row0i * 4 * kThinTiles * PITCH;
     const int vswz = ((lane & 15) / RPL) & (CPRW - 1);
-    static_for<0, KS>([&](auto s_) {
-      constexpr int s = decltype(s_)::value;
-      static_for<0, 4>([&](auto j_) {
-        constexpr int j = decltype(j_)::value;
-        Frag v[NROW];
-        static_for<0, NROW>([&](auto i_) {
-          constexpr int i = decltype(i_)::value;
-          v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + ((((lane >> 4) + 4 * s) ^ vswz) << 4));
-        });
-        static_for<0, NROW>([&](auto i_) {
-          constexpr int i = decltype(i_)::value;
-          if constexpr (j <= 2) z0[i] = MF::run(u[i * 4 + j][s], v[i], z0[i]);
-        });
-        static_for<0, NROW>([&](auto i_) {
-          constexpr int i = decltype(i_)::value;
-          if constexpr (j == 1) zp[i] = MF::run(u[i * 4 + j][s], v[i], zp[i]);
-          if constexpr (j >= 2) zn[i] = MF::run(u[i * 4 + j][s], v[i], zn[i]);
+    if constexpr (PLAIN) {
+      floatx4 mm[NROW][4];
+#pragma unroll
+      for (int i = 0; i < NROW; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mm[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+      static_for<0, KS>([&](auto s_) {
+        constexpr int s = decltype(s_)::value;
+        static_for<0, 4>([&](auto j_) {
+          constexpr int j = decltype(j_)::value;
+          Frag v[NROW];
+          static_for<0, NROW>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + ((((lane >> 4) + 4 * s) ^ vswz) << 4));
+          });
+          static_for<0, NROW>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            mm[i][j] = MF::run(u[i * 4 + j][s], v[i], mm[i][j]);
+          });
         });
       });
-    });
+#pragma unroll
+      for (int i = 0; i < NROW; ++i) {
+        zw[i][0] = mm[i][0] + mm[i][1] + mm[i][2];
+        zw[i][1] = mm[i][1] - mm[i][2] - mm[i][3];
+      }
+    } else {
+      floatx4 z0[NROW], zp[NROW], zn[NROW];
+#pragma unroll
+      for (int i = 0; i < NROW; ++i) z0[i] = zp[i] = zn[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+      static_for<0, KS>([&](auto s_) {
+        constexpr int s = decltype(s_)::value;
+        static_for<0, 4>([&](auto j_) {
+          constexpr int j = decltype(j_)::value;
+          Frag v[NROW];
+          static_for<0, NROW>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            v[i] = *reinterpret_cast<const Frag*>(vrow + (i * 4 + j) * kThinTiles * PITCH + ((((lane >> 4) + 4 * s) ^ vswz) << 4));
+          });
+          static_for<0, NROW>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            if constexpr (j <= 2) z0[i] = MF::run(u[i * 4 + j][s], v[i], z0[i]);
+          });
+          static_for<0, NROW>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            if constexpr (j == 1) zp[i] = MF::run(u[i * 4 + j][s], v[i], zp[i]);
+            if constexpr (j >= 2) zn[i] = MF::run(u[i * 4 + j][s], v[i], zn[i]);
+          });
+        });
+      });
+#pragma unroll
+      for (int i = 0; i < NROW; ++i) {
+        zw[i][0] = z0[i];
+        zw[i][1] = zp[i] - zn[i];
+      }
+    }
 
-    // Height half of the output transform: out[0][b] = z[0][b] + z[1][b] + z[2][b], out[1][b] = z[1][b] -
-    // z[2][b] - z[3][b] with z[i][0] = z0[i], z[i][1] = zp[i] - zn[i].
+    // Height half of the output transform: out[0][b] = zw[0][b] + zw[1][b] + zw[2][b], out[1][b] = zw[1][b] -
+    // zw[2][b] - zw[3][b].
     floatx4 out[2][2];
     if constexpr (!SPLIT) {
 #pragma unroll
       for (int ob = 0; ob < 2; ++ob) {
-        floatx4 z[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) z[i] = ob == 0 ? z0[i] : zp[i] - zn[i];
-        out[0][ob] = z[0] + z[1] + z[2];
-        out[1][ob] = z[1] - z[2] - z[3];
+        out[0][ob] = zw[0][ob] + zw[1][ob] + zw[2][ob];
+        out[1][ob] = zw[1][ob] - zw[2][ob] - zw[3][ob];
       }
     } else {
       // the upper wavefronts (rows 2, 3) pass their share through LDS to the lower ones (rows 0, 1)
@@ -342,7 +377,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
       const bool upper = wave >= 4;
 #pragma unroll
       for (int ob = 0; ob < 2; ++ob) {
-        const floatx4 za = ob == 0 ? z0[0] : zp[0] - zn[0], zb = ob == 0 ? z0[1] : zp[1] - zn[1];
+        const floatx4 za = zw[0][ob], zb = zw[1][ob];
         out[0][ob] = upper ? za : za + zb;
         out[1][ob] = upper ? -za - zb : zb;
       }

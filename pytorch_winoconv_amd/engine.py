@@ -294,8 +294,8 @@ def thin_preferred(dtype, nd, in_channels, out_channels, kernel, stride):
     """True where the fused F(2x2, 3x3) kernel also beats the three-kernel path with tile 4, so that a caller
     free to choose the tile should take 2: every 16-bit layer the kernel takes (1.25-1.7x), first layers, and in
     fp32 (where the products run on the eight times slower fp32 MFMA and F(4,3) needs 2.25x fewer of them) layers
-    with at most 32 input channels or at most 64 output channels (N=8, 64 -> 64 at 224x224: 194 against 227 us;
-    64 -> 128 at 112x112: 110 against 90 us, so tile 4 there)."""
+    with at most 32 input channels or at most 64 output channels (N=8, 64 -> 64 at 224x224: 160 against 231 us;
+    64 -> 128 at 112x112: 92 against 93 us, a tie, so tile 4 there)."""
     if not thin_layer(dtype, nd, in_channels, out_channels, kernel, stride):
         return False
     if dtype != torch.float32 or in_channels <= 4:
