@@ -121,10 +121,10 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 3x3 s2 direct form (the default)", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16"),
     ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 2, "f16-nodirect"),
     ("c4 fp16 N32 C128 112x112 3x3 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 3, 3), 2, 1, 4, "f16-nodirect"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 direct form", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-direct"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM shared input F(2,2) on the parity phases", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-stacked"),
-    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-stacked"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 direct form (the default)", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM shared input F(2,2) on the parity phases", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-nodirect"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(2,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 2, "f16-stacked-nodirect"),
+    ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-stacked-nodirect"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
@@ -152,8 +152,8 @@ def run_suite(steps=10, only=None):
         dtype = torch.float32 if dt == "f32" else torch.float16
         # None: the engine's default (16-bit: stride-1 kernels of 4..8 taps share one transformed input,
         # other DWM plans are stacked)
-        stacked = False if dt.endswith("-pieces") else True if dt.endswith("-stacked") else None
-        unfused = dt.endswith("-unfused")                          # thin layers: keep the three-kernel path
+        stacked = False if "-pieces" in dt else True if "-stacked" in dt else None
+        unfused = "-unfused" in dt                                 # thin layers: keep the three-kernel path
         direct = False if dt.endswith("-nodirect") else True if dt.endswith("-direct") else None
         g = torch.Generator().manual_seed(0)
         fan = 1
@@ -162,8 +162,15 @@ def run_suite(steps=10, only=None):
         x = torch.randn(*xs, generator=g).to(dtype).to(dev)
         x = x.contiguous(memory_format=torch.channels_last if len(xs) == 4 else torch.channels_last_3d)
         w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype).to(dev)
-        for _ in range(2):
-            y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
+        # warm-up by time, not by count: a configuration measured in the first few milliseconds after another one
+        # runs before the clocks have settled (fp32 layers measured 8-10 % slower that way)
+        y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
+        torch.cuda.synchronize()
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < 0.15:
+            for _ in range(5):
+                engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
+            torch.cuda.synchronize()
         # best of three rounds: a single round now and then includes a stall of tens of milliseconds
         # (the caching allocator returning memory between configurations of very different sizes)
         ms = float("inf")

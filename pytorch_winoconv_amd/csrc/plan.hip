@@ -341,16 +341,33 @@ static int auto_stacked(const wc_conv_desc* d) {
   return n > 1 && n <= 4 ? 1 : 0;
 }
 
-// Stride 2 in 16-bit: where the direct form measured faster than the parity-phase Winograd plans on MI355X
-// (fp16, filter conversion included on both sides).  It wins while the reduction kh kw C is short: 3x3 at
-// N=32, C=K=128, 112x112 runs 63 us against 128 (F(4,r)) and 164 (F(2,r)); C=K=256, 56x56 107 against 160;
-// 4x4 103 against 144; 5x5 at C=128 145 against 154.  Longer reductions favour the plans, whose saving in
-// multiplications grows with the kernel: 6x6 at C=128 200 against 182 us, 5x5 at C=256 257 against 194, 3x3 at
-// C=512 (14x14 images) 91 against 66.  With 64 output channels or fewer the direct form runs 64 x 64 tiles
-// only, which loses for kernels beyond 5x5 (7x7, C=K=64, 224x224: 387 against 371 us).
+// Stride 2 in 16-bit: where the direct form measured faster than the parity-phase Winograd plan the caller would
+// otherwise get (MI355X, fp16, warmed clocks, filter conversion included on both sides; us, direct | F(2,r) plan |
+// F(4,r) plan).
+//  * Short reductions (kh kw C <= 3200) always: 3x3 at N=32, C=K=128, 112x112 57 | 160 | 126; C=K=256, 56x56
+//    94 | 193 | 156; 256 -> 512 at 28x28 53 | 81 | 86; 5x5 at C=128 131 | 261 | 154; small layers too (N=8, 128 channels,
+//    56x56: 22 | 28 | 29).
+//  * With 64 output channels or fewer it runs 64 x 64 tiles only and loses beyond 5x5 kernels (7x7, C=K=64,
+//    224x224: 382 | 372; 128 -> 64 at 112x112: 209 | 201).
+//  * A long reduction needs enough output (pixels x channels >= 4 M, i.e. 256 tiles of 128 x 128) to keep the chip
+//    busy, else the latency of its k-steps decides: 3x3 at C=K=512 on 14x14 images 90 | 66, 7x7 at C=K=256 on 28x28
+//    240 | 139.  With that: against the plan that shares one transformed input (7 and 8 taps) 7x7 wins
+//    (C=K=128, 112x112: 246 | 267; 96 channels 184 | 206) and 8x8 loses (321 | 277); against stacked F(2,r) pieces it
+//    always wins (6x6 187 | 279, 5x5 at 256 channels 242 | 303, 9x9 399 | 845); against stacked F(4,r) pieces it wins
+//    at 4x4 (256 channels, 56x56: 87 | 96) and from 9x9 on (399 | 565) and loses or ties between (5x5 at 256 channels
+//    242 | 190, 6x6 at 128 187 | 179).
 static bool direct_preferred(const wc_conv_desc* d) {
   const int taps = d->kernel[1] * d->kernel[2];
-  return (long long)taps * d->C <= 3200 && (d->K > 64 || taps <= 25);
+  if (d->K <= 64 && taps > 25) return false;
+  if ((long long)taps * d->C <= 3200) return true;
+  wc_conv_desc e = *d;
+  e.direct = 0; e.stacked = 0; e.m = 2; e.whole_kernel = 0;
+  int out[3], grid[3];
+  if (wc_conv_out_dims(&e, out, grid) != WC_OK) return false;
+  if ((long long)d->N * out[1] * out[2] * d->K < (4ll << 20)) return false;
+  if (auto_stacked(d) == 2) return taps <= 49;
+  if (d->m == 2) return true;
+  return taps <= 16 || taps >= 81;
 }
 
 int wc_conv_auto(wc_conv_desc* d) {

@@ -453,12 +453,21 @@ def test_module_tables_equal_oracle_tables():
         assert np.allclose(pkg.matrix_conv.B[key], BT, atol=1e-16, rtol=0)
 
 
-@pytest.mark.parametrize("C,K,k,chosen", [
-    (128, 128, 3, 1), (256, 256, 3, 1), (128, 128, 4, 1), (128, 128, 5, 1), (64, 64, 3, 1), (32, 64, 5, 1), (64, 128, 7, 1),
-    (512, 512, 3, 0), (256, 256, 5, 0), (128, 128, 6, 0), (128, 128, 7, 0), (64, 64, 7, 0), (32, 8, 7, 0)])
-def test_the_library_chooses_the_direct_form_for_short_reductions(C, K, k, chosen):
-    """kh kw C <= 3200, and kernels of at most 25 taps when K <= 64: the side of the measured crossover each
-    stride-2 layer of the sweep behind the rule fell on."""
-    d = engine.make_desc((2, C, 28, 28), (K, C, k, k), torch.float16, 2, k // 2, 2, stacked=None)
+@pytest.mark.parametrize("N,C,K,H,k,m,chosen", [
+    # short reductions (kh kw C <= 3200): always
+    (32, 128, 128, 112, 3, 2, 1), (64, 256, 256, 56, 3, 4, 1), (32, 128, 128, 112, 4, 4, 1), (32, 128, 128, 112, 5, 4, 1),
+    (2, 64, 64, 28, 3, 2, 1), (2, 32, 64, 28, 5, 2, 1), (32, 64, 128, 112, 7, 2, 1),
+    # at most 64 output channels: kernels of at most 25 taps only
+    (32, 64, 64, 224, 7, 2, 0), (2, 32, 8, 28, 7, 2, 0), (32, 128, 64, 112, 7, 4, 0),
+    # long reductions need pixels x channels >= 4 M
+    (64, 512, 512, 14, 3, 4, 0), (128, 512, 512, 14, 3, 2, 0), (64, 256, 256, 28, 7, 2, 0), (2, 128, 128, 28, 7, 2, 0),
+    # ... then: against the shared-input plan 7x7 yes, 8x8 no
+    (32, 128, 128, 112, 7, 2, 1), (32, 128, 128, 112, 7, 4, 1), (32, 96, 96, 112, 7, 4, 1), (32, 128, 128, 112, 8, 4, 0),
+    # against stacked F(2,r) pieces always; against stacked F(4,r) pieces at 4x4 and from 9x9 on
+    (32, 128, 128, 112, 6, 2, 1), (32, 128, 128, 112, 6, 4, 0), (64, 256, 256, 56, 5, 2, 1), (64, 256, 256, 56, 5, 4, 0),
+    (32, 256, 256, 56, 4, 4, 1), (32, 128, 128, 112, 9, 4, 1), (32, 128, 128, 112, 9, 2, 1)])
+def test_the_library_chooses_the_direct_form_where_it_measured_faster(N, C, K, H, k, m, chosen):
+    """Each stride-2 layer of the sweep behind the rule, on the side of the crossover it measured on."""
+    d = engine.make_desc((N, C, H, H), (K, C, k, k), torch.float16, 2, k // 2, m, stacked=None)
     assert d.direct == chosen
-    assert engine.make_desc((2, C, 28, 28), (K, C, k, k), torch.bfloat16, 2, k // 2, 2, stacked=None).direct == chosen
+    assert engine.make_desc((N, C, H, H), (K, C, k, k), torch.bfloat16, 2, k // 2, m, stacked=None).direct == chosen

@@ -72,7 +72,9 @@ def test_full_size_config(dev, cfg):
     stacked = False if name.endswith("piece by piece") else None
 
     def forward(a):
-        return engine.conv_forward(a, wd, None, stride, pad, m, stacked=stacked)
+        # the Winograd / DWM plans are what this file covers at full size: the direct form, which the library would
+        # take for the stride-2 layers, has its own full-size test (test_gpu_direct.py)
+        return engine.conv_forward(a, wd, None, stride, pad, m, stacked=stacked, direct=False)
 
     y = forward(xd)
     conv = F.conv2d if len(xs) == 4 else F.conv3d
