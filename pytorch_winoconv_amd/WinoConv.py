@@ -86,6 +86,13 @@ class _WinoConvNd(nn.Module):
         self._cache = None
 
     def _winograd_ok(self, x):
+        # The reference hands every strided or dilated layer (and every kernel up to 3 x 3) to the stock
+        # convolution (conv.py:326-332, 467-473).  This engine keeps strided layers, with one exception: strided
+        # first layers with at most 8 input channels, whose parity-phase plans pad the channels to 32 once per
+        # phase (ResNet's 3 -> 64, 7 x 7, stride 2 at N = 32: 0.25 ms in fp16 and 1.0 ms in fp32 against 0.07 and
+        # 0.12 ms for torch's own convolution); they go the reference's way.
+        if self.stride[0] == 2 and self.in_channels <= 8:
+            return False
         return (self.groups == 1 and set(self.dilation) == {1} and len(set(self.stride)) == 1
                 and self.stride[0] in (1, 2) and max(self.kernel_size) <= 10)
 

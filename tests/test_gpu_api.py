@@ -182,6 +182,10 @@ def test_winoconv2d_module_routes_and_caches(dev, k, stride, pad):
     mod_d = pkg.WinoConv2d(16, 24, 3, 1, 2, dilation=2, dtype=torch.float16, device=dev)
     yd = mod_d(x)
     assert yd.shape == (2, 24, 20, 20)
+    # so does a strided first layer with at most 8 input channels (the reference sends every strided layer there)
+    mod_s = pkg.WinoConv2d(3, 16, 7, 2, 3, dtype=torch.float16, device=dev)
+    x3 = torch.randn(2, 3, 30, 30, device=dev).half()
+    assert torch.equal(mod_s(x3), F.conv2d(x3, mod_s.weight, mod_s.bias, 2, 3)) and mod_s._cache is None
 
 
 def test_winoconv3d_module(dev):
