@@ -118,11 +118,12 @@ typedef struct {
   int direct;      /* 1: the direct form, the degenerate end of the split: pieces of one tap on the trivial tile F(1,1),
                     *    for which there is nothing to transform, so the batched product reads the pixels of x as its V
                     *    operand, walks the taps along its reduction axis and writes y; no V or M in memory, U is the
-                    *    filter as (K, kH, kW, C).  2-D, fp16 / bf16, C a multiple of 32, K a multiple of 8; m, stacked
-                    *    and whole_kernel are ignored.  wc_conv_auto chooses it for stride 2, which the reference does
-                    *    not implement (src/winograd_conv.cpp:122-126) and where Winograd tiles on the parity phases
-                    *    save few or no multiplications.  wc_conv_forward, wc_filter_transform, wc_conv_workspace_bytes
-                    *    and wc_conv_u_elems honour it; the other stage functions do not apply. */
+                    *    filter as (K, kH, kW, C).  2-D, C a multiple of 32 (fp32: 16), K a multiple of 8; m, stacked
+                    *    and whole_kernel are ignored.  wc_conv_auto chooses it for kernels of one tap (every type: the
+                    *    tile F(m,1) saves nothing and its transforms are copies) and for 16-bit layers at stride 2, which
+                    *    the reference does not implement (src/winograd_conv.cpp:122-126) and where Winograd tiles on
+                    *    the parity phases save few or no multiplications.  wc_conv_forward, wc_filter_transform,
+                    *    wc_conv_workspace_bytes and wc_conv_u_elems honour it; the other stage functions do not apply. */
 } wc_conv_desc;
 
 /* ---- library ------------------------------------------------------------------------- */

@@ -78,7 +78,7 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   L->direct = d_in->direct == 1;
   if (L->direct) {
     if (!direct_conv_fits(d_in))
-      return fail(WC_ERR_UNSUPPORTED, "direct form: 2-D, fp16 / bf16, input channels a multiple of 32, output channels a multiple of 8");
+      return fail(WC_ERR_UNSUPPORTED, "direct form: 2-D, input channels a multiple of 32 (fp32: 16), output channels a multiple of 8");
     plain.direct = 0; plain.stacked = 0; plain.m = 2; plain.whole_kernel = 0; plain.unfused = 1;
   }
   const wc_conv_desc* d = &plain;

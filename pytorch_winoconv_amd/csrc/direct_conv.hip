@@ -1,10 +1,11 @@
-// Direct form of a 2-D convolution for 16-bit types (wc_conv_desc.direct): the degenerate end of the DWM split, pieces
+// Direct form of a 2-D convolution (wc_conv_desc.direct): the degenerate end of the DWM split, pieces
 // of ONE tap on the trivial tile F(1,1).  With one tap per piece there is nothing to transform - B^T, G and A^T
 // are 1 - so the batched product reads the pixels of x itself as its V operand, walks the taps along its reduction
 // axis (gemm_kernel<..., DIRECT> in gemm.hip) and writes y.  x is read once from HBM (the taps of neighbouring outputs
 // meet in the caches), y written once, nothing else moves.
 //
-// Where it is used: stride 2.  The reference leaves stride 2 unimplemented (src/winograd_conv.cpp:122-126); the plans
+// Where it is used: 1x1 kernels of every type (a Winograd tile of one tap saves nothing, and its transforms are copies:
+// three passes over memory instead of one), and 16-bit layers at stride 2.  The reference leaves stride 2 unimplemented (src/winograd_conv.cpp:122-126); the plans
 // built here for it run Winograd tiles on the parity phases of x, which saves no multiplications for small kernels
 // (F(2,2) on the phases of a 3x3 kernel needs the 9 products per output of the direct form) and moves V and M
 // through HBM.  Stride-1 layers keep their Winograd plans, which need 2.25x to 4x fewer products.
@@ -36,8 +37,8 @@ __global__ __launch_bounds__(256) void direct_filter_kernel(DirectFilterArgs a) 
 }
 
 bool direct_conv_fits(const wc_conv_desc* d) {
-  if (d->ndim != 2 || (d->dtype != WC_F16 && d->dtype != WC_BF16)) return false;
-  if (d->C % 32 != 0 || d->K % 8 != 0) return false;            // 16-byte accesses along C and along K
+  if (d->ndim != 2) return false;
+  if (d->C % (d->dtype == WC_F32 ? 16 : 32) != 0 || d->K % 8 != 0) return false;   // whole reduction blocks along C, 16-byte stores along K
   if (d->whole_kernel) return false;
   int out[3], grid[3];
   wc_conv_desc e = *d;
@@ -55,14 +56,15 @@ int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[
   a.K = d->K; a.C = d->C; a.kh = d->kernel[1]; a.kw = d->kernel[2];
   a.total = (long long)d->K * d->kernel[1] * d->kernel[2] * d->C;
   const unsigned blocks = (unsigned)ceil_div_ll(a.total, 256);
-  if (d->dtype == WC_F16) hipLaunchKernelGGL(direct_filter_kernel<half_t>, dim3(blocks), dim3(256), 0, as_stream(stream), a);
+  if (d->dtype == WC_F32) hipLaunchKernelGGL(direct_filter_kernel<float>, dim3(blocks), dim3(256), 0, as_stream(stream), a);
+  else if (d->dtype == WC_F16) hipLaunchKernelGGL(direct_filter_kernel<half_t>, dim3(blocks), dim3(256), 0, as_stream(stream), a);
   else hipLaunchKernelGGL(direct_filter_kernel<bf16_t>, dim3(blocks), dim3(256), 0, as_stream(stream), a);
   WC_CHECK_LAUNCH("direct_filter_kernel");
   return WC_OK;
 }
 
 int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y, void* stream) {
-  WC_CHECK_ARG(direct_conv_fits(d), "direct convolution: 2-D, fp16 / bf16, input channels a multiple of 32, output "
+  WC_CHECK_ARG(direct_conv_fits(d), "direct convolution: 2-D, input channels a multiple of 32 (fp32: 16), output "
                "channels a multiple of 8");
   int out[3], grid[3];
   wc_conv_desc e = *d;

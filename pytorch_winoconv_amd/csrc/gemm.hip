@@ -720,39 +720,47 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
 // Tiles of the direct form, chosen like those of the shifted operand.
 template <typename T>
 static GemmConfig choose_direct(int P, int K) {
+  constexpr int BK = sizeof(T) == 4 ? 16 : 32;
   auto blocks = [&](const GemmConfig& c) { return (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn); };
   switch (test_gemm_config()) {                       // wc_test_gemm_override: a tile shape forced by a test
-    case 0: return make_config<T, 2, 2, 32, 4, 2, true, true>();
-    case 1: return make_config<T, 2, 2, 32, 2, 2, true, true>();
-    case 2: return make_config<T, 4, 1, 32, 2, 2, true, true>();
-    case 3: return make_config<T, 1, 1, 32, 2, 2, true, true>();
-    case 4: return make_config<T, 4, 2, 32, 2, 2, true, true>();   // 256 x 128, four wavefronts
+    case 0: return make_config<T, 2, 2, BK, 4, 2, true, true>();
+    case 1: return make_config<T, 2, 2, BK, 2, 2, true, true>();
+    case 2: return make_config<T, 4, 1, BK, 2, 2, true, true>();
+    case 3: return make_config<T, 1, 1, BK, 2, 2, true, true>();
+    case 4: return make_config<T, 4, 2, BK, 2, 2, true, true>();   // 256 x 128, four wavefronts
     default: break;
   }
   // Measured on MI355X (fp16, stride 2): the largest tile that still gives every compute unit a workgroup
   // wins: 256 x 128 over 128 x 128 by 15-25 % at 392 workgroups (N=32, C=K=128, 112x112: 54.9 against
   // 63.7 us; C=K=256, 56x56: 93.5 against 115 us), and loses by 40 % at 196.  Four wavefronts of 128 x 64
   // beat eight of 64 x 64 for the large tile (54.9 against 73.0 us): half the LDS reads per MFMA.
+  // fp32 products are bound by the MFMA rate and fill the chip best with small tiles (as in choose()).
+  if constexpr (sizeof(T) == 4) {
+    GemmConfig mid = make_config<T, 2, 2, BK, 2, 2, true, true>();     // 128 x 128
+    if (K > 64 && blocks(mid) >= 2048) return mid;
+    return make_config<T, 1, 1, BK, 2, 2, true, true>();               // 64 x 64
+  }
   if (K > 64) {
-    GemmConfig big = make_config<T, 4, 2, 32, 2, 2, true, true>();   // 256 x 128, four wavefronts
+    GemmConfig big = make_config<T, 4, 2, BK, 2, 2, true, true>();   // 256 x 128, four wavefronts
     if (blocks(big) >= kCus) return big;
-    GemmConfig mid = make_config<T, 2, 2, 32, 2, 2, true, true>();   // 128 x 128
+    GemmConfig mid = make_config<T, 2, 2, BK, 2, 2, true, true>();   // 128 x 128
     if (blocks(mid) >= kCus) return mid;
   }
-  return make_config<T, 1, 1, 32, 2, 2, true, true>();               // 64 x 64
+  return make_config<T, 1, 1, BK, 2, 2, true, true>();               // 64 x 64
 }
 
 // y (N, oH, oW, K) = direct convolution of x (N, H, W, C) with U (K, kh kw C): the batched product with the
-// pixels of x as its V operand (no transform, no intermediate in memory); 16-bit types, C a multiple of 32,
-// K a multiple of 8.
+// pixels of x as its V operand (no transform, no intermediate in memory); C a multiple of the reduction block (32
+// elements of a 16-bit type, 16 of fp32), K a multiple of 8.
 int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,
                      int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream) {
   WC_CHECK_ARG(x && U && y, "gemm_direct_conv: null pointer");
-  WC_CHECK_ARG(C > 0 && C % 32 == 0 && K > 0 && K % 8 == 0, "gemm_direct_conv: C %d (multiple of 32), K %d (multiple of 8)", C, K);
-  if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "gemm_direct_conv: 16-bit types only");
+  WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_BF16 || dtype == WC_F32, "gemm_direct_conv: dtype %d", dtype);
+  const int cq = dtype == WC_F32 ? 16 : 32;
+  WC_CHECK_ARG(C > 0 && C % cq == 0 && K > 0 && K % 8 == 0, "gemm_direct_conv: C %d (multiple of %d), K %d (multiple of 8)", C, cq, K);
   const long long P = (long long)N * oH * oW;
   WC_CHECK_ARG(P > 0 && P < (1ll << 31) && (long long)kh * kw * C < (1ll << 24), "gemm_direct_conv: problem too large");
-  GemmConfig c = dtype == WC_F16 ? choose_direct<half_t>((int)P, K) : choose_direct<bf16_t>((int)P, K);
+  GemmConfig c = dispatch_dtype(dtype, [&](auto t) { return choose_direct<decltype(t)>((int)P, K); });
   GemmArgs g;
   g.V = x; g.U = U; g.M = y; g.bias = bias;
   g.P = (int)P; g.K = K; g.ldm = K;

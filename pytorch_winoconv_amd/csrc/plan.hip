@@ -341,9 +341,9 @@ static int auto_stacked(const wc_conv_desc* d) {
   return n > 1 && n <= 4 ? 1 : 0;
 }
 
-// Stride 2 in 16-bit: where the direct form measured faster than the parity-phase Winograd plan the caller would
-// otherwise get (MI355X, fp16, warmed clocks, filter conversion included on both sides; us, direct | F(2,r) plan |
-// F(4,r) plan).
+// Where the direct form measured faster than the Winograd plan the caller would otherwise get.  Stride 2 in 16-bit,
+// against the parity-phase plans (MI355X, fp16, warmed clocks, filter conversion included on both sides; us,
+// direct | F(2,r) plan | F(4,r) plan):
 //  * Short reductions (kh kw C <= 3200) always: 3x3 at N=32, C=K=128, 112x112 57 | 160 | 126; C=K=256, 56x56
 //    94 | 193 | 156; 256 -> 512 at 28x28 53 | 81 | 86; 5x5 at C=128 131 | 261 | 154; small layers too (N=8, 128 channels,
 //    56x56: 22 | 28 | 29).
@@ -356,8 +356,12 @@ static int auto_stacked(const wc_conv_desc* d) {
 //    always wins (6x6 187 | 279, 5x5 at 256 channels 242 | 303, 9x9 399 | 845); against stacked F(4,r) pieces it wins
 //    at 4x4 (256 channels, 56x56: 87 | 96) and from 9x9 on (399 | 565) and loses or ties between (5x5 at 256 channels
 //    242 | 190, 6x6 at 128 187 | 179).
+//  * A kernel of one tap at either stride, every type: the tile F(m,1) has nothing to save and its transforms are
+//    copies (fp16 N=64, 64 -> 256 channels, 56x56: three kernels 78 us).
 static bool direct_preferred(const wc_conv_desc* d) {
   const int taps = d->kernel[1] * d->kernel[2];
+  if (taps == 1) return true;
+  if (d->stride != 2 || d->dtype == WC_F32) return false;
   if (d->K <= 64 && taps > 25) return false;
   if ((long long)taps * d->C <= 3200) return true;
   wc_conv_desc e = *d;
@@ -378,7 +382,7 @@ int wc_conv_auto(wc_conv_desc* d) {
   const bool never_direct = d->direct == -1;
   if (never_direct) d->direct = 0;
   if (d->stacked == -1) {
-    if (d->stride == 2 && !d->direct && !never_direct && direct_conv_fits(d) && direct_preferred(d)) d->direct = 1;
+    if (!d->direct && !never_direct && direct_conv_fits(d) && direct_preferred(d)) d->direct = 1;
     d->stacked = d->direct ? 0 : auto_stacked(d);
   }
   if (d->stacked == 2 && d->m == 4) {

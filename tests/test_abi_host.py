@@ -471,3 +471,19 @@ def test_the_library_chooses_the_direct_form_where_it_measured_faster(N, C, K, H
     d = engine.make_desc((N, C, H, H), (K, C, k, k), torch.float16, 2, k // 2, m, stacked=None)
     assert d.direct == chosen
     assert engine.make_desc((N, C, H, H), (K, C, k, k), torch.bfloat16, 2, k // 2, m, stacked=None).direct == chosen
+    assert engine.make_desc((N, C, H, H), (K, C, k, k), torch.float32, 2, k // 2, m, stacked=None).direct == 0    # 16-bit only
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_one_tap_kernels_take_the_direct_form(dtype):
+    """1x1 kernels at either stride, every type, where the operands allow it (whole reduction blocks of channels,
+    16-byte rows of y); never when ruled out, never with an explicit plan form."""
+    for stride in (1, 2):
+        for m in (2, 4):
+            assert engine.make_desc((4, 64, 28, 28), (128, 64, 1, 1), dtype, stride, 0, m, stacked=None).direct == 1
+    assert engine.make_desc((4, 64, 28, 28), (128, 64, 1, 1), dtype, 1, 0, 2, stacked=None, direct=False).direct == 0
+    assert engine.make_desc((4, 64, 28, 28), (128, 64, 1, 1), dtype, 1, 0, 2, stacked=False).direct == 0
+    assert engine.make_desc((4, 20, 28, 28), (128, 20, 1, 1), dtype, 1, 0, 2, stacked=None).direct == 0          # 20 channels
+    assert engine.make_desc((4, 64, 28, 28), (100, 64, 1, 1), dtype, 1, 0, 2, stacked=None).direct == 0          # K no multiple of 8
+    assert engine.make_desc((4, 48, 28, 28), (128, 48, 1, 1), dtype, 1, 0, 2, stacked=None).direct == (1 if dtype == torch.float32 else 0)
+    assert engine.make_desc((4, 64, 28, 28), (128, 64, 1, 3), dtype, 1, (0, 1), 2, stacked=None).direct == 0     # three taps, stride 1

@@ -1,7 +1,7 @@
 """The direct form (wc_conv_desc.direct): pieces of one tap on the tile F(1,1), i.e. the batched product reading the
-pixels of x itself with the taps along its reduction axis.  The library chooses it for 16-bit stride-2 layers (which
-the reference does not implement: src/winograd_conv.cpp:122-126) where it measured faster than the parity-phase
-Winograd plan the caller would otherwise get; on request it runs any 2-D kernel and stride.
+pixels of x itself with the taps along its reduction axis.  The library chooses it for 1x1 kernels (every type) and for
+16-bit stride-2 layers (which the reference does not implement: src/winograd_conv.cpp:122-126) where it measured
+faster than the parity-phase Winograd plan the caller would otherwise get; on request it runs any 2-D kernel and stride.
 
 Pinned bit for bit on small integers (every product and sum exact), against fp64 torch convolution and the oracle on
 normal data, and against the Winograd / DWM plans of the same engine."""
@@ -23,14 +23,17 @@ CASES = [
     ((40, 32, 28, 28), (32, 32, 3, 3), 2, 1),     # enough output pixels for the largest tile
     # stride 1 on request
     ((2, 32, 9, 11), (8, 32, 3, 3), 1, 1), ((1, 64, 12, 12), (16, 64, 5, 5), 1, 2), ((1, 32, 8, 8), (8, 32, 1, 3), 1, (0, 1)),
+    # 1x1 kernels: the library's own choice at either stride
+    ((3, 64, 13, 11), (40, 64, 1, 1), 1, 0), ((2, 32, 10, 10), (8, 32, 1, 1), 1, 1), ((6, 96, 28, 28), (256, 96, 1, 1), 1, 0),
 ]
+DISC = {torch.float16: "fp16", torch.bfloat16: "bf16", torch.float32: "fp32"}
 
 
 def _rel(a, b):
     return float((a.double().cpu() - b.double().cpu()).abs().max() / b.double().abs().max().clamp_min(1e-30))
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case", CASES)
 def test_exact_on_small_integers(dev, dtype, case, host_layer):
     xs, ws, stride, pad = case
@@ -39,14 +42,14 @@ def test_exact_on_small_integers(dev, dtype, case, host_layer):
     w = torch.randint(-2, 3, ws, generator=g).double()
     b = torch.randint(-8, 9, (ws[0],), generator=g).double()
     ref = F.conv2d(x, w, b, stride=stride, padding=pad)
-    assert float(ref.abs().max()) < (2048 if dtype == torch.float16 else 256) * 8      # representable after the one rounding
+    assert float(ref.abs().max()) < {torch.float16: 2048, torch.bfloat16: 256, torch.float32: 1 << 21}[dtype] * 8      # representable after the one rounding
     y = engine.conv_forward(x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev), stride, pad, 2, direct=True)
     assert tuple(y.shape) == tuple(ref.shape)
     assert torch.equal(y.cpu(), ref.float().to(dtype))
-    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, stride, pad, "fp16" if dtype == torch.float16 else "bf16"))
+    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, stride, pad, DISC[dtype]))
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case", CASES)
 def test_against_fp64_the_oracle_and_the_winograd_plans(dev, dtype, case):
     xs, ws, stride, pad = case
@@ -58,14 +61,18 @@ def test_against_fp64_the_oracle_and_the_winograd_plans(dev, dtype, case):
     ref = F.conv2d(x.double(), w.double(), b.double(), stride=stride, padding=pad)
     xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
     y = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=True)
-    tol = 2e-3 if dtype == torch.float16 else 1.2e-2            # one rounding of an fp32 sum
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.2e-2, torch.float32: 2e-6}[dtype]            # one rounding of an fp32 sum
     assert _rel(y, ref) <= tol
-    assert _rel(y, ow.direct_conv(x, w, b, stride, pad, "fp16" if dtype == torch.float16 else "bf16")) <= tol
+    assert _rel(y, ow.direct_conv(x, w, b, stride, pad, DISC[dtype])) <= tol
     yw = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=False)          # the Winograd / DWM plan
-    assert _rel(yw, ref) <= 2e-2 and _rel(y, yw.cpu()) <= 2e-2
-    # the library's own choice is one of the two; at stride 1 it is never the direct form
+    assert _rel(yw, ref) <= (1e-3 if dtype == torch.float32 else 2e-2) and _rel(y, yw.cpu()) <= 2e-2
+    # the library's own choice is one of the two: always the direct form for one tap, never for more taps at stride 1
+    # or in fp32
     chosen = engine.make_desc(xs, ws, dtype, stride, pad, 2, stacked=None).direct
-    assert stride == 2 or chosen == 0
+    if ws[2] * ws[3] == 1:
+        assert chosen == 1
+    elif stride == 1 or dtype == torch.float32:
+        assert chosen == 0
     ya = engine.conv_forward(xd, wd, bd, stride, pad, 2)
     assert torch.equal(ya, y if chosen else yw)
     # cached filter, no bias, channel-first in and out, one image per pass
