@@ -361,7 +361,11 @@ static int auto_stacked(const wc_conv_desc* d) {
 static bool direct_preferred(const wc_conv_desc* d) {
   const int taps = d->kernel[1] * d->kernel[2];
   if (taps == 1) return true;
-  if (d->stride != 2 || d->dtype == WC_F32) return false;
+  if (d->stride != 2) return false;
+  // fp32 products are bound by the MFMA rate, where the multiplications F(4,r) tiles save count: the direct form wins
+  // for 3x3 kernels over at most 128 channels only (N=64, 128 channels, 56x56: 163 | 220 | 170; N=16, 64 channels,
+  // 112x112: 55 | 77 | 65; 32 -> 64 at 112x112: 49 | 86 | 75; 256 channels on 28x28: 187 | 173 | 176; 5x5 at 128: 798 | 708 | 426)
+  if (d->dtype == WC_F32) return taps <= 9 && d->C <= 128;
   if (d->K <= 64 && taps > 25) return false;
   if ((long long)taps * d->C <= 3200) return true;
   wc_conv_desc e = *d;

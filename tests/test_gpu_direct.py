@@ -71,7 +71,7 @@ def test_against_fp64_the_oracle_and_the_winograd_plans(dev, dtype, case):
     chosen = engine.make_desc(xs, ws, dtype, stride, pad, 2, stacked=None).direct
     if ws[2] * ws[3] == 1:
         assert chosen == 1
-    elif stride == 1 or dtype == torch.float32:
+    elif stride == 1:
         assert chosen == 0
     ya = engine.conv_forward(xd, wd, bd, stride, pad, 2)
     assert torch.equal(ya, y if chosen else yw)
@@ -94,7 +94,7 @@ def test_outside_its_range_the_direct_form_is_refused_or_not_chosen(dev):
     assert engine.make_desc(x.shape, w.shape, torch.float16, 2, 1, 2, stacked=None).direct == 0
     assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None).direct == 1
     assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 1, 1, 2, stacked=None).direct == 0      # stride 1
-    assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float32, 2, 1, 2, stacked=None).direct == 0      # fp32
+    assert engine.make_desc((2, 32, 12, 12), (8, 32, 5, 5), torch.float32, 2, 2, 2, stacked=None).direct == 0      # fp32 beyond 3x3
     assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None, direct=False).direct == 0
     assert engine.make_desc((2, 32, 12, 12), (12, 32, 3, 3), torch.float16, 2, 1, 2, stacked=None).direct == 0     # K no multiple of 8
     assert engine.make_desc((2, 32, 12, 12), (8, 32, 3, 3), torch.float16, 2, 1, 2, stacked=True).direct == 0      # an explicit plan form
