@@ -194,6 +194,10 @@ def test_winoconv3d_module(dev):
     x = torch.randn(1, 8, 6, 10, 10, device=dev)
     ref = F.conv3d(x.double().cpu(), mod.weight.detach().double().cpu(), mod.bias.detach().double().cpu(), padding=1)
     assert _nerr(mod(x), ref) < 1e-3
+    # a 3-D first layer with at most 4 input channels goes to torch (the reference sends every 3x3x3 layer there)
+    mod3 = pkg.WinoConv3d(3, 8, 3, 1, 1, device=dev)
+    x3 = torch.randn(1, 3, 6, 10, 10, device=dev)
+    assert torch.equal(mod3(x3), F.conv3d(x3, mod3.weight, mod3.bias, 1, 1)) and mod3._cache is None
 
 
 @pytest.mark.parametrize("ws,m,stacked", [
