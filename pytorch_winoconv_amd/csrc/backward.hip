@@ -231,9 +231,38 @@ struct BwdLayout {
   long long tiles_per_image;
   size_t es;
   size_t v_bytes, dm_bytes, du_bytes, acc_bytes;
+  bool one_tap;                     // 1x1 kernel, stride 1, no padding: dw = dy^T x, no transforms
 };
 
+// A kernel of one tap at stride 1 without padding: y = x w^T pixel by pixel, so dw (K x C) = sum over the pixels of
+// dy (x) x is the transposed product of the two tensors as they lie in memory, rows = pixels; F(m,1) has nothing to
+// transform and its dM and V would be copies (fp16 N=64, 64 -> 256 channels, 56x56: 92 us that way).
+bool one_tap_layout(const wc_conv_desc* d, BwdLayout* L) {
+  if (d->ndim != 2 || d->stride != 1 || d->whole_kernel) return false;
+  for (int a = 0; a < 3; ++a)
+    if (d->kernel[a] != 1 || d->pad[a] != 0) return false;
+  if (d->C % 8 != 0 || d->K % 8 != 0) return false;
+  const long long P = (long long)d->N * d->in[1] * d->in[2];
+  if (P >= (1ll << 31)) return false;
+  L->one_tap = true;
+  L->es = d->dtype == WC_F32 ? 4 : 2;
+  L->ldm = d->K; L->Cp = d->C; L->ncol = d->C; L->ldc = d->C; L->chunk = d->N;
+  L->tiles_per_image = (long long)d->in[1] * d->in[2];
+  const int bt = (d->K > 64 && d->C > 64) ? 128 : 64;
+  const long long tiles = (long long)((d->K + bt - 1) / bt) * ((d->C + bt - 1) / bt);
+  long long S = (1024 + tiles - 1) / tiles;                       // about four workgroups of the product per CU
+  S = std::max(1ll, std::min(S, std::min(64ll, P / 256)));
+  L->S = (int)S;
+  L->Pq = (int)(((P + S - 1) / S + 31) / 32 * 32);
+  L->v_bytes = L->dm_bytes = L->acc_bytes = 0;
+  L->du_bytes = round256((size_t)S * d->K * d->C * 4);
+  return true;
+}
+
 int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
+  WC_CHECK_ARG(d != nullptr, "null descriptor");
+  L->one_tap = false;
+  if (one_tap_layout(d, L)) return WC_OK;
   if (d && d->stacked == 2)
     return fail(WC_ERR_UNSUPPORTED, "the weight gradient is not built for plans with a shared transformed input (stacked = 2)");
   int rc = wc_plan_conv(d, &L->plan);
@@ -317,7 +346,18 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
   const size_t y_image = (size_t)L.out[0] * L.out[1] * L.out[2] * d->K * L.es;
   const int taps = d->kernel[0] * d->kernel[1] * d->kernel[2];
 
-  for (int b0 = 0; b0 < d->N; b0 += L.chunk) {
+  if (L.one_tap) {
+    const long long P = L.tiles_per_image * d->N;
+    rc = batched_gemm_tn(dy, x, dU, 1, P, d->K, d->C, d->K, d->C, d->C, L.S, L.Pq, d->dtype, stream);
+    if (rc) return rc;
+    if (L.S > 1) {
+      const long long n = (long long)d->K * d->C, total4 = n / 4;
+      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)ceil_div_ll(total4, 256)), dim3(256), 0, s, dU, L.S, n, total4);
+      WC_CHECK_LAUNCH("sum_parts_kernel");
+    }
+    acc = dU;
+  }
+  for (int b0 = 0; b0 < d->N && !L.one_tap; b0 += L.chunk) {
     const int n = std::min(L.chunk, d->N - b0);
     const long long P = L.tiles_per_image * n;
     rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);

@@ -25,6 +25,9 @@ CASES = [
     ((1, 4, 5, 7, 7), (4, 4, 2, 3, 1), 1, 0, 2),
     ((4, 64, 28, 28), (64, 64, 3, 3), 1, 1, 4),
     ((1, 3, 9, 9), (2, 3, 1, 1), 1, 0, 2),                # 1 x 1 kernel
+    ((3, 32, 17, 19), (40, 32, 1, 1), 1, 0, 2),           # 1 x 1, whole vectors of channels: dw = dy^T x, no transforms
+    ((9, 96, 28, 28), (136, 96, 1, 1), 1, 0, 4),          # the same with 128 x 128 product tiles and several parts
+    ((2, 32, 10, 10), (8, 32, 1, 1), 2, 0, 2),            # 1 x 1 at stride 2: the same
     ((6, 24, 40, 40), (40, 24, 3, 3), 1, 1, 2),           # tile sum split into 9 parts, the last one short
     ((8, 72, 40, 40), (136, 72, 3, 3), 1, 1, 4),          # 128 x 128 product tiles with partial edges, 3 parts
 ]
