@@ -274,6 +274,16 @@ int wc_conv_forward_static(const wc_conv_desc* desc, const void* x,
  * (dU = sum over tiles of dM x V, dw = G^T dU G) with every sum in fp32.  The input gradient needs
  * no entry point of its own: it is wc_conv_forward of dy with the flipped, transposed filter. */
 int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
+/* Input gradient of a 2-D layer at stride 2 (no counterpart in the reference either): dx (N, H, W, C) from dy
+ * (N, oH, oW, K) channel-last contiguous and the filter through its element strides, for the descriptor of the
+ * forward call.  The pixels of dx fall into four classes by their parity; each class is a stride-1 direct convolution
+ * of dy with the taps of its parity (flipped, channel axes exchanged), one launch of the direct form each, writing every
+ * second pixel: the multiplications of the forward pass, where convolving a zero-filled dy multiplies four times as
+ * much.  K a multiple of 32 (fp32: 16), C a multiple of 8, padding below the kernel extent; WC_ERR_UNSUPPORTED
+ * otherwise (a caller then runs wc_conv_forward on the zero-filled dy).  Sums in fp32, one rounding. */
+int wc_conv_backward_input_workspace_bytes(const wc_conv_desc* desc, size_t* bytes);
+int wc_conv_backward_input(const wc_conv_desc* desc, const void* dy, const void* w, const int64_t w_strides[5],
+                           void* dx, void* workspace, size_t workspace_bytes, void* stream);
 int wc_conv_backward_weight(const wc_conv_desc* desc, const void* x, const void* dy, void* dw,
                             const int64_t dw_strides[5], void* workspace, size_t workspace_bytes,
                             void* stream);

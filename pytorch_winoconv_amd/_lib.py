@@ -65,6 +65,8 @@ SIGNATURES = {
     "wc_conv_u_elems": (_i, [_desc_p, ctypes.POINTER(_sz)]),
     "wc_conv_forward": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _vp, _vp, _sz, _vp]),
     "wc_conv_forward_static": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _vp, _vp]),
+    "wc_conv_backward_input_workspace_bytes": (_i, [_desc_p, ctypes.POINTER(_sz)]),
+    "wc_conv_backward_input": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _sz, _vp]),
     "wc_conv_forward_timed": (_i, [_desc_p, _vp, _vp, _i64_5, _vp, _vp, _vp, _vp, _sz, _vp, ctypes.POINTER(ctypes.c_float)]),
     "wc_conv_backward_weight_workspace_bytes": (_i, [_desc_p, ctypes.POINTER(_sz)]),
     "wc_conv_backward_weight": (_i, [_desc_p, _vp, _vp, _vp, _i64_5, _vp, _sz, _vp]),

@@ -82,6 +82,10 @@ struct GemmArgs {
   // fall outside the image contribute zeros; `bias` (K values, may be null) is added before the result is rounded
   int H, W, oH, oW, conv_stride, pad_h, pad_w, kw, cblocks;
   const void* bias;
+  // direct form writing every o_step-th pixel of a larger image (the input gradient of a strided layer, one launch per
+  // parity class of its pixels): row (b, oy, ox) of the product goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of
+  // image b of an (o_H, o_W) tensor; o_step == 0: rows are written one after the other
+  int o_step, o_y0, o_x0, o_H, o_W;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -284,9 +288,19 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
       for (int r = 0; r < SROWS / RPPO; ++r) {
         const int srow = orow + r * RPPO;            // staged row: wavefront row, then (ii, l32)
         const int row = (srow / (EI * 32)) * WM * 32 + i0 * 32 + srow % (EI * 32);
-        if (p0 + row < g.P)
-          *reinterpret_cast<Chunk16*>(Mt + (long long)(p0 + row) * g.ldm + k0 + ocol) =
+        if (p0 + row < g.P) {
+          long long orow = p0 + row;
+          if constexpr (DIRECT) {
+            if (g.o_step) {
+              const int per = g.oH * g.oW;
+              const int b = (p0 + row) / per, rem = (p0 + row) - b * per;
+              const int oy = rem / g.oW, ox = rem - oy * g.oW;
+              orow = ((long long)b * g.o_H + oy * g.o_step + g.o_y0) * g.o_W + ox * g.o_step + g.o_x0;
+            }
+          }
+          *reinterpret_cast<Chunk16*>(Mt + orow * g.ldm + k0 + ocol) =
               *reinterpret_cast<const Chunk16*>(cs + srow * CS + ocol);
+        }
       }
     }
   }
@@ -703,6 +717,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   g.plane_runs = sh.n_runs;
   g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
   g.n_run = sh.n_run; g.total_runs = sh.n_planes * sh.n_runs;
   g.run_rows = sh.run_rows; g.plane_extra = sh.plane_rows - sh.n_runs * sh.run_rows;
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
@@ -753,7 +768,8 @@ static GemmConfig choose_direct(int P, int K) {
 // pixels of x as its V operand (no transform, no intermediate in memory); C a multiple of the reduction block (32
 // elements of a 16-bit type, 16 of fp32), K a multiple of 8.
 int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,
-                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream) {
+                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream,
+                     int o_step, int o_y0, int o_x0, int o_H, int o_W) {
   WC_CHECK_ARG(x && U && y, "gemm_direct_conv: null pointer");
   WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_BF16 || dtype == WC_F32, "gemm_direct_conv: dtype %d", dtype);
   const int cq = dtype == WC_F32 ? 16 : 32;
@@ -772,6 +788,7 @@ int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, in
   g.n_run = kw; g.total_runs = kh; g.run_rows = W; g.plane_extra = 0;
   g.H = H; g.W = W; g.oH = oH; g.oW = oW; g.conv_stride = stride; g.pad_h = pad_h; g.pad_w = pad_w;
   g.kw = kw; g.cblocks = C / c.bk;
+  g.o_step = o_step; g.o_y0 = o_y0; g.o_x0 = o_x0; g.o_H = o_H; g.o_W = o_W;
   g.sV = 0; g.sU = 0; g.sM = 0;
   g.tiles_p = ceil_div((int)P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 1;
   const long long blocks = (long long)g.tiles_p * g.tiles_k;
@@ -802,6 +819,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
   g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

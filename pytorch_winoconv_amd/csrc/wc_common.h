@@ -131,8 +131,11 @@ int transpose_images(const void* src, void* dst, long long n, long long R, long 
 bool direct_conv_fits(const wc_conv_desc* d);
 int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
 int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y, void* stream);
+// o_step > 0: row (b, oy, ox) of the result goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of image b of an
+// (o_H, o_W) tensor instead of to row b oH oW + oy oW + ox
 int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,
-                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream);
+                     int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream,
+                     int o_step = 0, int o_y0 = 0, int o_x0 = 0, int o_H = 0, int o_W = 0);
 
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;

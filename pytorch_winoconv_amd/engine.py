@@ -472,6 +472,25 @@ def conv_backward_input(dy, w, x_spatial, stride=1, padding=0, m=2):
     if any(k - 1 - p < 0 for k, p in zip(ks, pads)):
         raise NotImplementedError("input gradient needs padding <= kernel - 1 on every axis")
     want = tuple(int(v) for v in x_spatial)
+    if stride == 2 and nd == 2 and dy.shape[0] > 0:
+        # the library's own input gradient of strided layers: one direct-form launch per parity class of the pixels of
+        # dx (wc_conv_backward_input); where it does not apply, the zero-filled dy below
+        lib = _lib.load()
+        x_shape = (dy.shape[0], w.shape[1]) + want
+        desc = make_desc(x_shape, w.shape, dy.dtype, 2, padding, 2, 0, False, False, direct=False)
+        out, _ = out_dims(desc)
+        if tuple(dy.shape[2:]) != tuple(out[1:]):
+            raise ValueError("dy of shape %r does not belong to an input of extent %r" % (tuple(dy.shape), want))
+        nbytes = ctypes.c_size_t()
+        if lib.wc_conv_backward_input_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0:
+            if w.dtype != dy.dtype:
+                raise TypeError("dy and the filter must share one dtype")
+            dy_cl = channel_last(dy)
+            dx = torch.empty((x_shape[0],) + want + (x_shape[1],), dtype=dy.dtype, device=dy.device)
+            ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dy.device)
+            check(lib.wc_conv_backward_input(ctypes.byref(desc), _ptr(dy_cl), _ptr(w), _w_strides(w), _ptr(dx), _ptr(ws),
+                                             nbytes.value, _stream(dy)))
+            return channel_first_view(dx)
     if stride == 2:
         # zeros between the elements of dy, and at the end as many as it takes for the result to have
         # the input's extent (one more when the strided forward pass left an odd remainder)

@@ -28,6 +28,14 @@ CASES = [
     ((3, 32, 17, 19), (40, 32, 1, 1), 1, 0, 2),           # 1 x 1, whole vectors of channels: dw = dy^T x, no transforms
     ((9, 96, 28, 28), (136, 96, 1, 1), 1, 0, 4),          # the same with 128 x 128 product tiles and several parts
     ((2, 32, 10, 10), (8, 32, 1, 1), 2, 0, 2),            # 1 x 1 at stride 2: the same
+    # stride 2 with the channel counts the library's own input gradient takes (one direct-form launch per parity class)
+    ((2, 8, 15, 14), (32, 8, 3, 3), 2, 1, 2),
+    ((3, 16, 21, 20), (64, 16, 7, 7), 2, 3, 2),
+    ((2, 24, 12, 13), (32, 24, 1, 1), 2, 0, 2),           # one tap: three of the four classes are zero
+    ((2, 8, 13, 16), (32, 8, 4, 2), 2, (1, 0), 2),
+    ((2, 8, 10, 11), (32, 8, 2, 2), 2, 1, 2),             # padding that moves a class beyond the first row of dy
+    ((2, 8, 9, 9), (32, 8, 3, 3), 2, 2, 2),
+    ((4, 64, 56, 56), (64, 64, 3, 3), 2, 1, 4),
     ((6, 24, 40, 40), (40, 24, 3, 3), 1, 1, 2),           # tile sum split into 9 parts, the last one short
     ((8, 72, 40, 40), (136, 72, 3, 3), 1, 1, 4),          # 128 x 128 product tiles with partial edges, 3 parts
 ]
