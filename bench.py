@@ -33,10 +33,10 @@ sys.path.insert(0, ROOT)
 N, C, K, H, W, R, PAD, M_TILE = 64, 256, 256, 56, 56, 3, 1, 4
 MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
 HBM_PEAK_GB_S = 8000.0              # MI355X published HBM3E bandwidth
-# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116740 KiB, x2.00 by the copy
+# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116806 KiB, x2.00 by the copy
 # probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
 # profiles/mfma_utilisation_shipped_gemms.md.
-GEMM_HBM_TRAFFIC_BYTES = int((116740 * 2.0 + 225792 * 1.0) * 1024)
+GEMM_HBM_TRAFFIC_BYTES = int((116806 * 2.0 + 225792 * 1.0) * 1024)
 
 
 def synthetic(n):
@@ -138,7 +138,13 @@ VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256
          (512, 512, 14)]
 
 
-def run_suite(steps=10, only=None):
+# the default form of every configuration of BASELINE.json: what a plain `python bench.py` adds to its JSON line
+DEFAULTS = ("c1 ", "c2 vgg16 fp32 N8 F(4,3)", "c2 vgg16 fp32 N8 F(2,3)", "c3 fp16 N64 C64 56x56 F(2,3)", "c3 fp16 N64 C128 28x28 F(2,3)",
+            "c3 fp16 N64 C256", "c3 fp16 N64 C512", "5x5 s1 DWM shared input F(3,3)", "7x7 s1 DWM shared input F(3,3)",
+            "3x3 s2 direct form", "7x7 s2 direct form", "c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3")
+
+
+def run_suite(steps=10, only=None, defaults=False):
     """ms per layer (whole forward through the one-call entry point, filter transform included;
     `ms_filter_cached`: with the filter transformed beforehand) and direct-convolution-equivalent
     TFLOP/s for every other benchmark configuration (`only`: just the configurations whose name
@@ -210,6 +216,8 @@ def run_suite(steps=10, only=None):
 
     for name, xs, ws, stride, pad, m, dt in SUITE:
         if only and only not in name:
+            continue
+        if defaults and not any(key in name for key in DEFAULTS):
             continue
         if xs == "vgg":
             ms = fl = msc = mst = 0.0
@@ -385,7 +393,9 @@ def main():
     ap.add_argument("--gemm-config", type=int, default=-1, metavar="I",
                     help="force tile shape I of the batched GEMM through the library's test hook (-1: its own choice)")
     ap.add_argument("--suite", action="store_true",
-                    help="also time every other benchmark configuration (adds a 'suite' list)")
+                    help="time every form of every other benchmark configuration (the 'suite' list); without it the "
+                         "list holds the default form of each configuration of BASELINE.json (c1..c5), about 20 s")
+    ap.add_argument("--no-suite", action="store_true", help="no 'suite' list at all: the metric layer only")
     ap.add_argument("--event-every", type=int, default=4, metavar="N",
                     help="record the per-stage HIP events on every N-th timed step (an event record between two "
                          "kernels keeps the second from starting under the tail of the first: about 13 us per "
@@ -549,8 +559,10 @@ def main():
         "effective_tflops_filter_cached": direct_flops / (ms_cached * 1e-3) / 1e12,
         "one_call_matches_stages": same,
     }
-    if args.suite:
+    if args.suite or args.suite_only:
         result["suite"] = run_suite(only=args.suite_only)
+    elif not args.no_suite:
+        result["suite"] = run_suite(defaults=True)
     if args.backward:
         result["backward_us"] = run_backward()
     if args.split_concat:
