@@ -21,6 +21,8 @@ CALLS = [
     ((5, 64, 12, 12), (64, 64, 3, 3), 1, 1, 2, H16, False),       # thin layer: one fused kernel, only U in the buffer
     ((2, 16, 6, 10, 9), (8, 16, 3, 3, 3), 1, 1, 2, H16, False),   # 3-D
     ((2, 32, 21, 20), (16, 32, 7, 7), 2, 3, 2, H16, True),        # stride 2, stacked pieces
+    ((4, 64, 21, 20), (32, 64, 3, 3), 2, 1, 2, H16, None),        # stride 2, the library's choice: the direct form, only U in the buffer
+    ((3, 32, 10, 11), (16, 32, 1, 1), 1, 0, 2, F32, None),        # one tap, fp32: the direct form
 ]
 
 
