@@ -198,6 +198,22 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ dU, 
   *reinterpret_cast<float4*>(base) = sum;
 }
 
+// acc[t][i] = sum over s of dU[t][s][i]: the same sum, written densely (the layout grad_filter_store_kernel reads)
+__global__ __launch_bounds__(256) void sum_parts_out_kernel(const float* __restrict__ dU, float* __restrict__ acc, int S,
+                                                            long long n, long long total4) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total4) return;
+  const long long n4 = n / 4;
+  const long long t = idx / n4, i = (idx % n4) * 4;
+  const float* base = dU + t * S * n + i;
+  float4 sum = *reinterpret_cast<const float4*>(base);
+  for (int sp = 1; sp < S; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(base + sp * n);
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  }
+  *reinterpret_cast<float4*>(acc + t * n + i) = sum;
+}
+
 // dw[k][c][tap] through element strides <- acc (taps, K, C)
 template <typename T>
 __global__ __launch_bounds__(256) void grad_filter_store_kernel(const float* __restrict__ acc, T* __restrict__ dw,
@@ -222,6 +238,23 @@ namespace {
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 
+// Parts the reduction over the tiles is split into.  The product's workgroups run in rounds of as many as the chip
+// holds at once (two per CU for 128 x 128 tiles, four for 64 x 64: what their LDS stages allow), and a round that is nearly empty costs as much
+// as a full one: the most parts that still fit r rounds, for the r with the least work per round-limited workgroup
+// (metric shape, 144 tiles: 7 parts = 1008 workgroups in two rounds, where 8 parts made 1152 = three rounds).
+int pick_parts(long long tiles, long long rows, bool big_tiles) {
+  const long long slots = big_tiles ? 512 : 1024;
+  long long best = 1;
+  double best_cost = 1e30;
+  for (int r = 1; r <= 4; ++r) {
+    long long S = slots * r / tiles;
+    S = std::max(1ll, std::min(S, std::min(64ll, rows / 256)));
+    const double cost = (double)((tiles * S + slots - 1) / slots) / (double)S;
+    if (cost < best_cost * (1.0 - 1e-9)) { best = S; best_cost = cost; }
+  }
+  return (int)best;
+}
+
 struct BwdLayout {
   wc_plan plan;
   int out[3], grid[3];
@@ -232,7 +265,36 @@ struct BwdLayout {
   size_t es;
   size_t v_bytes, dm_bytes, du_bytes, acc_bytes;
   bool one_tap;                     // 1x1 kernel, stride 1, no padding: dw = dy^T x, no transforms
+  bool gathered;                    // 2-D stride 2: dw[tap] = dy^T (the pixels of x that tap reads), no transforms
 };
+
+// A 2-D layer at stride 2: the transform-domain gradient runs Winograd tiles on the parity phases of x (V and dM
+// through memory, few multiplications saved); taken directly, tap (ky, kx) is one transposed product of dy with the
+// pixels of x that tap reads, gathered row by row inside the product (fp16 N=32, 128 channels, 112x112, 3x3: 159 us
+// in the transform domain).
+bool gathered_layout(const wc_conv_desc* d, BwdLayout* L) {
+  if (d->ndim != 2 || d->stride != 2 || d->whole_kernel) return false;
+  if (d->C % 8 != 0 || d->K % 8 != 0) return false;
+  wc_conv_desc e = *d;
+  e.direct = 0; e.stacked = 0; e.m = 2;
+  if (wc_conv_out_dims(&e, L->out, L->grid) != WC_OK) return false;
+  const long long P = (long long)d->N * L->out[1] * L->out[2];
+  if (P >= (1ll << 31) || (long long)d->N * d->in[1] * d->in[2] >= (1ll << 31)) return false;
+  const int taps = d->kernel[1] * d->kernel[2];
+  L->gathered = true;
+  L->es = d->dtype == WC_F32 ? 4 : 2;
+  L->ldm = d->K; L->Cp = d->C; L->ncol = d->C; L->ldc = d->C; L->chunk = d->N;
+  L->tiles_per_image = (long long)L->out[1] * L->out[2];
+  const int bt = (d->K > 64 && d->C > 64) ? 128 : 64;
+  const long long tiles = (long long)taps * ((d->K + bt - 1) / bt) * ((d->C + bt - 1) / bt);
+  const long long S = pick_parts(tiles, P, bt == 128);
+  L->S = (int)S;
+  L->Pq = (int)(((P + S - 1) / S + 31) / 32 * 32);
+  L->v_bytes = L->dm_bytes = 0;
+  L->du_bytes = round256((size_t)taps * S * d->K * d->C * 4);
+  L->acc_bytes = round256((size_t)taps * d->K * d->C * 4);
+  return true;
+}
 
 // A kernel of one tap at stride 1 without padding: y = x w^T pixel by pixel, so dw (K x C) = sum over the pixels of
 // dy (x) x is the transposed product of the two tensors as they lie in memory, rows = pixels; F(m,1) has nothing to
@@ -250,8 +312,7 @@ bool one_tap_layout(const wc_conv_desc* d, BwdLayout* L) {
   L->tiles_per_image = (long long)d->in[1] * d->in[2];
   const int bt = (d->K > 64 && d->C > 64) ? 128 : 64;
   const long long tiles = (long long)((d->K + bt - 1) / bt) * ((d->C + bt - 1) / bt);
-  long long S = (1024 + tiles - 1) / tiles;                       // about four workgroups of the product per CU
-  S = std::max(1ll, std::min(S, std::min(64ll, P / 256)));
+  const long long S = pick_parts(tiles, P, bt == 128);
   L->S = (int)S;
   L->Pq = (int)(((P + S - 1) / S + 31) / 32 * 32);
   L->v_bytes = L->dm_bytes = L->acc_bytes = 0;
@@ -261,8 +322,9 @@ bool one_tap_layout(const wc_conv_desc* d, BwdLayout* L) {
 
 int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   WC_CHECK_ARG(d != nullptr, "null descriptor");
-  L->one_tap = false;
+  L->one_tap = L->gathered = false;
   if (one_tap_layout(d, L)) return WC_OK;
+  if (gathered_layout(d, L)) return WC_OK;
   if (d && d->stacked == 2)
     return fail(WC_ERR_UNSUPPORTED, "the weight gradient is not built for plans with a shared transformed input (stacked = 2)");
   int rc = wc_plan_conv(d, &L->plan);
@@ -296,11 +358,10 @@ int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   L->chunk = chunk;
   const long long Pc = L->tiles_per_image * chunk;
   if (Pc >= (1ll << 31)) return fail(WC_ERR_UNSUPPORTED, "chunk of %d images has too many tiles", chunk);
-  // split of the tile axis: about four workgroups of the product per CU, every part >= 256 tiles
+  // split of the tile axis: whole rounds of resident workgroups, every part >= 256 tiles
   const int bt = (d->K > 64 && L->ncol > 64) ? 128 : 64;
   const long long tiles = T * ((d->K + bt - 1) / bt) * ((L->ncol + bt - 1) / bt);
-  long long S = (1024 + tiles - 1) / tiles;
-  S = std::max(1ll, std::min(S, std::min(64ll, Pc / 256)));
+  const long long S = pick_parts(tiles, Pc, bt == 128);
   L->S = (int)S;
   L->Pq = (int)(((Pc + S - 1) / S + 31) / 32 * 32);
   L->v_bytes = round256((size_t)T * Pc * L->Cp * L->es);
@@ -357,7 +418,15 @@ int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy
     }
     acc = dU;
   }
-  for (int b0 = 0; b0 < d->N && !L.one_tap; b0 += L.chunk) {
+  if (L.gathered) {
+    rc = gemm_tn_conv(dy, x, dU, d->N, d->in[1], d->in[2], d->C, d->K, d->kernel[1], d->kernel[2], d->stride, d->pad[1],
+                      d->pad[2], L.out[1], L.out[2], L.S, L.Pq, d->dtype, stream);
+    if (rc) return rc;
+    const long long n = (long long)d->K * d->C, total4 = (long long)taps * n / 4;
+    hipLaunchKernelGGL(sum_parts_out_kernel, dim3((unsigned)ceil_div_ll(total4, 256)), dim3(256), 0, s, dU, acc, L.S, n, total4);
+    WC_CHECK_LAUNCH("sum_parts_out_kernel");
+  }
+  for (int b0 = 0; b0 < d->N && !L.one_tap && !L.gathered; b0 += L.chunk) {
     const int n = std::min(L.chunk, d->N - b0);
     const long long P = L.tiles_per_image * n;
     rc = wc_input_transform(d, &L.plan, static_cast<const unsigned char*>(x) + b0 * x_image, n, V, stream);

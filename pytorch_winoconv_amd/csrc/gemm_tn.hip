@@ -19,6 +19,7 @@
 // W x W blocks of 32 x 32.  V feeds the MFMA "A" side, so a lane ends up with 4 consecutive
 // columns of D and stores them as one 16-byte write.
 #include "wc_common.h"
+#include "wc_transform.h"
 
 namespace wc {
 
@@ -41,6 +42,11 @@ struct GemmTnArgs {
   int S, Pq;
   int tiles_a, tiles_b;
   int n_blocks, per_xcd;
+  // GATHER (the weight gradient of a convolution taken directly, one batch per tap): A is dy (P = N oH oW rows, the
+  // same for every batch), B is x itself, and row p = (b, oy, ox) of batch t = (ky, kx) is the pixel
+  // (stride oy + ky - pad_h, stride ox + kx - pad_w) of image b, zeros outside the image
+  int H, W, oH, oW, conv_stride, pad_h, pad_w, kw;
+  FastDiv div_per, div_oW;
 };
 
 __device__ __forceinline__ floatx16 mfma16(short8v a, short8v b, floatx16 c, half_t) {
@@ -50,7 +56,7 @@ __device__ __forceinline__ floatx16 mfma16(short8v a, short8v b, floatx16 c, bf1
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <typename T, int W, int BK>
+template <typename T, int W, int BK, bool GATHER = false>
 __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(GemmTnArgs g) {
   constexpr int BT = 64 * W;                       // tile extent on both output axes
   constexpr int EPC = 16 / sizeof(T);              // elements per 16-byte chunk
@@ -76,8 +82,9 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(GemmTnArgs g) {
   const long long p_end = min(g.P, p_begin + g.Pq);
   const int nk = p_end > p_begin ? (int)((p_end - p_begin + BK - 1) / BK) : 0;
 
-  const T* Ap = static_cast<const T*>(g.A) + (long long)t * g.P * g.lda;
-  const T* Bp = static_cast<const T*>(g.B) + (long long)t * g.P * g.ldb;
+  const T* Ap = static_cast<const T*>(g.A) + (GATHER ? 0 : (long long)t * g.P * g.lda);
+  const T* Bp = static_cast<const T*>(g.B) + (GATHER ? 0 : (long long)t * g.P * g.ldb);
+  const int tap_y = GATHER ? t / g.kw : 0, tap_x = GATHER ? t - tap_y * g.kw : 0;
 
   const int tid = threadIdx.x;
   const int lrow = tid / CPR, lcol = (tid % CPR) * EPC;
@@ -90,7 +97,17 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(GemmTnArgs g) {
       const long long p = p_begin + (long long)kt * BK + lrow + i * RPP;
       const Chunk16 zero = {0u, 0u, 0u, 0u};
       ra[i] = (p < p_end && a_in) ? *reinterpret_cast<const Chunk16*>(Ap + p * g.lda + a0 + lcol) : zero;
-      rb[i] = (p < p_end && b_in) ? *reinterpret_cast<const Chunk16*>(Bp + p * g.ldb + b0 + lcol) : zero;
+      if constexpr (GATHER) {
+        const int pi = (int)min(p, g.P - 1);
+        const int b = fast_div(pi, g.div_per), rem = pi - b * (g.oH * g.oW);
+        const int oy = fast_div(rem, g.div_oW), ox = rem - oy * g.oW;
+        const int iy = oy * g.conv_stride + tap_y - g.pad_h, ix = ox * g.conv_stride + tap_x - g.pad_w;
+        const bool inside = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+        rb[i] = (p < p_end && b_in && inside)
+                    ? *reinterpret_cast<const Chunk16*>(Bp + (((long long)b * g.H + iy) * g.W + ix) * g.ldb + b0 + lcol) : zero;
+      } else {
+        rb[i] = (p < p_end && b_in) ? *reinterpret_cast<const Chunk16*>(Bp + p * g.ldb + b0 + lcol) : zero;
+      }
     }
   };
   auto lstore = [&](int buf) {
@@ -199,7 +216,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(GemmTnArgs g) {
   }
 }
 
-template <typename T, int W>
+template <typename T, int W, bool GATHER = false>
 int launch_tn(GemmTnArgs g, int T_, void* stream) {
   constexpr int BT = 64 * W;
   constexpr int BK = sizeof(T) == 2 ? 64 : 16;     // reduction rows per stage (64: measured 5 % faster than 32)
@@ -210,8 +227,8 @@ int launch_tn(GemmTnArgs g, int T_, void* stream) {
   WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_tn: problem too large");
   g.n_blocks = (int)blocks;
   g.per_xcd = ceil_div((int)blocks, kXcds);
-  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tn_kernel<T, W, BK>), lds)) return rc;
-  hipLaunchKernelGGL((gemm_tn_kernel<T, W, BK>), dim3((unsigned)(g.per_xcd * kXcds)), dim3(256), lds, as_stream(stream), g);
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tn_kernel<T, W, BK, GATHER>), lds)) return rc;
+  hipLaunchKernelGGL((gemm_tn_kernel<T, W, BK, GATHER>), dim3((unsigned)(g.per_xcd * kXcds)), dim3(256), lds, as_stream(stream), g);
   WC_CHECK_LAUNCH("gemm_tn_kernel");
   return WC_OK;
 }
@@ -229,10 +246,34 @@ int batched_gemm_tn(const void* A, const void* B, float* D, int T_, long long P,
   g.A = A; g.B = B; g.D = D; g.P = P;
   g.lda = lda; g.ldb = ldb; g.na = na; g.nb = nb; g.ldd = ldd;
   g.S = S; g.Pq = Pq;
+  g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = 0;
+  g.div_per = g.div_oW = make_fast_div(1);
   const bool big = na > 64 && nb > 64;
   return dispatch_dtype(dtype, [&](auto t) {
     using TT = decltype(t);
     return big ? launch_tn<TT, 2>(g, T_, stream) : launch_tn<TT, 1>(g, T_, stream);
+  });
+}
+
+// dW[(ky, kx)][s] (K x C, fp32) = sum over the output pixels p = (b, oy, ox) of part s of dy[p][0..K) (x)
+// x[b][stride oy + ky - pad_h][stride ox + kx - pad_w][0..C): the weight gradient taken directly, one batch per tap,
+// x gathered row by row (zeros outside the image).  dy (N oH oW, K) and x (N, H, W, C) as they lie in memory.
+int gemm_tn_conv(const void* dy, const void* x, float* D, int N, int H, int W, int C, int K, int kh, int kw, int stride,
+                 int pad_h, int pad_w, int oH, int oW, int S, int Pq, int dtype, void* stream) {
+  WC_CHECK_ARG(dy && x && D, "gemm_tn_conv: null pointer");
+  WC_CHECK_ARG(C % 8 == 0 && K % 8 == 0 && S > 0 && Pq > 0, "gemm_tn_conv: C %d, K %d (multiples of 8)", C, K);
+  const long long P = (long long)N * oH * oW;
+  WC_CHECK_ARG(P > 0 && P < (1ll << 31) && (long long)S * Pq >= P, "gemm_tn_conv: %d parts of %d rows and %lld rows", S, Pq, P);
+  GemmTnArgs g;
+  g.A = dy; g.B = x; g.D = D; g.P = P;
+  g.lda = K; g.ldb = C; g.na = K; g.nb = C; g.ldd = C;
+  g.S = S; g.Pq = Pq;
+  g.H = H; g.W = W; g.oH = oH; g.oW = oW; g.conv_stride = stride; g.pad_h = pad_h; g.pad_w = pad_w; g.kw = kw;
+  g.div_per = make_fast_div(oH * oW); g.div_oW = make_fast_div(oW);
+  const bool big = K > 64 && C > 64;
+  return dispatch_dtype(dtype, [&](auto t) {
+    using TT = decltype(t);
+    return big ? launch_tn<TT, 2, true>(g, kh * kw, stream) : launch_tn<TT, 1, true>(g, kh * kw, stream);
   });
 }
 

@@ -157,6 +157,10 @@ int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const floa
 // A[t][p][.] (x) B[t][p][.], operands (T, P, ld) of storage type `dtype` (gemm_tn.hip).
 int batched_gemm_tn(const void* A, const void* B, float* D, int T, long long P, int lda, int ldb, int na, int nb,
                     int ldd, int S, int Pq, int dtype, void* stream);
+// The weight gradient of a 2-D convolution taken directly: dW[(ky, kx)][s] (K x C) = sum over the output pixels of
+// part s of dy (x) the pixel of x that tap reads (gemm_tn.hip)
+int gemm_tn_conv(const void* dy, const void* x, float* D, int N, int H, int W, int C, int K, int kh, int kw, int stride,
+                 int pad_h, int pad_w, int oH, int oW, int S, int Pq, int dtype, void* stream);
 
 // One-kernel F(2x2, 3x3) forward pass for thin 16-bit layers (conv_thin.hip): whether the problem
 // with this single-piece plan is in its range, and the launch.  U (16, K, Cp) from wc_filter_transform.
