@@ -136,6 +136,8 @@ const char* wc_last_error(void);
  * library's list of shapes; -1 = choose by problem size) on wc_batched_gemm, and for plans that
  * share one transformed input the kernel with one operand tile per piece (rows_mode 0), the
  * choice by size (1, the default) or one tile per run of pieces wherever the plan has runs (2).
+ * config 8 / 9: the one-kernel F(2x2,3x3) path with workgroups of 64 / 32 output channels whatever
+ * the number of tiles (9 only where the channel count allows it).
  * Process-wide; production code never calls it. */
 int wc_test_gemm_override(int config, int rows_mode);
 

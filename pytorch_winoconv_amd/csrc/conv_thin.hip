@@ -158,16 +158,20 @@ static_assert(Mats<KIND_23>::bt(0, 0) == 1 && Mats<KIND_23>::bt(0, 2) == -1 && M
               Mats<KIND_23>::bt(3, 1) == 1 && Mats<KIND_23>::bt(3, 3) == -1, "B^T of F(2,3)");
 
 // KW: K is a multiple of 4, a lane's 4 output channels go out in one store (a compile-time choice: a branch
-// around the stores, even a uniform one, makes the compiler wait for all memory operations at the loop top)
-template <typename T, int CP, bool KW>
-__global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2))) void thin_conv3x3_kernel(ThinArgs a) {
+// around the stores, even a uniform one, makes the compiler wait for all memory operations at the loop top).
+// KSUB: groups of 16 output channels per workgroup, 4 or 2.  With 2 a workgroup has half the wavefronts, half of
+// U to fetch and half the products, and the launch has twice the workgroups: for layers whose blocks of tiles
+// would leave more than half of the CUs idle (a workgroup with one block spends most of its time fetching U and,
+// in fp32, multiplying).
+template <typename T, int CP, bool KW, int KSUB>
+__global__ __launch_bounds__((CP * sizeof(T) > 128 ? 128 : 64) * KSUB) __attribute__((amdgpu_waves_per_eu(KSUB / 2, KSUB / 2))) void thin_conv3x3_kernel(ThinArgs a) {
   // Up to 64 channels a wavefront holds U of all 16 elements (4 wavefronts).  With 128 that is twice
   // the register file, so SPLIT: 8 wavefronts, the upper four take the element rows 2 and 3 and hand
   // their share of the output tile to the lower four through LDS.
   constexpr bool SPLIT = CP * sizeof(T) > 128;       // 128 channels of a 16-bit type, 64 of fp32
   constexpr bool PLAIN = sizeof(T) == 4;             // one accumulator per element, width transform in VALU (measured: no gain for 16-bit types)
   constexpr int EPF = 16 / sizeof(T);                // channels per 16-byte fragment
-  constexpr int NT = SPLIT ? 512 : 256;
+  constexpr int NT = (SPLIT ? 128 : 64) * KSUB;
   constexpr int NROW = SPLIT ? 2 : 4;     // element rows per wavefront
   constexpr int VEC = kThinTiles * CP / NT;   // channels per thread in the transform
   constexpr int CVECS = CP / VEC;
@@ -188,8 +192,8 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int kbase = blockIdx.y * kThinK + (wave & 3) * 16;
-  const int row0i = SPLIT ? 2 * (wave >> 2) : 0;       // first element row of this wavefront
+  const int kbase = (blockIdx.y * KSUB + wave % KSUB) * 16;
+  const int row0i = SPLIT ? 2 * (wave / KSUB) : 0;       // first element row of this wavefront
 
   // transform role: tile pl of the block, channels c .. c + VEC.  x is read through a buffer descriptor:
   // one 32-bit offset per load, and a window element outside the image is an offset beyond the
@@ -234,17 +238,59 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
   // this wavefront's part of U: row operand, lane = output channel kbase + lane % 16, 8 channels
   // from 8 * (lane / 16).  Rows beyond K repeat row K - 1: a row of U only reaches the same row of the
   // product, and those rows are never stored.
+  // Memory is read in whole rows (consecutive lanes take consecutive 16 bytes) and the fragments go to the lanes
+  // that need them through this wavefront's own slice of LDS, which nothing else uses yet: a load whose
+  // neighbouring lanes address different rows, as the operand layout would have it, measured 3.8 times slower per
+  // byte with every line in L2, and for a workgroup with one block of tiles that load is most of the kernel.
   Frag u[NROW * 4][KS];
   {
-    const int ko = kbase + (lane & 15);
-    const T* U = static_cast<const T*>(a.U) + (long long)min(ko, a.K - 1) * CP + EPF * (lane >> 4) +
-                 (long long)row0i * 4 * a.K * CP;
-    static_for<0, NROW * 4>([&](auto t_) {
+    constexpr int NW = NT / 64;
+    constexpr int SLICE = 2 * BUF / NW;                // bytes of LDS per wavefront
+    constexpr int EPR = SLICE / (16 * PITCH);          // elements per round: 16 rows of U each
+    constexpr int NEL = NROW * 4;
+    static_assert(EPR >= 1 && NEL % EPR == 0 && KS == PITCH / 64, "staging of U");
+    unsigned char* slice = lds + wave * SLICE;
+    const unsigned char* Ub = static_cast<const unsigned char*>(a.U);
+    uint4v tmp[NEL][KS];
+    int srow[KS], scol[KS];
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const int off = (i * 64 + lane) * 16;            // byte of the 16-row block
+      srow[i] = off / PITCH;
+      scol[i] = off % PITCH;
+    }
+    static_for<0, NEL>([&](auto t_) {
       constexpr int t = decltype(t_)::value;
-      static_for<0, KS>([&](auto s_) {
-        constexpr int s = decltype(s_)::value;
-        u[t][s] = *reinterpret_cast<const Frag*>(U + (long long)t * a.K * CP + s * 4 * EPF);
+#pragma unroll
+      for (int i = 0; i < KS; ++i) {
+        const long long row = (long long)(row0i * 4 + t) * a.K + min(kbase + srow[i], a.K - 1);
+        tmp[t][i] = *reinterpret_cast<const uint4v*>(Ub + row * PITCH + scol[i]);
+      }
+    });
+    const int fswz = ((lane & 15) / RPL) & (CPRW - 1);
+    static_for<0, NEL / EPR>([&](auto r_) {
+      constexpr int rd = decltype(r_)::value;
+      static_for<0, EPR>([&](auto e_) {
+        constexpr int e = decltype(e_)::value;
+#pragma unroll
+        for (int i = 0; i < KS; ++i)
+          *reinterpret_cast<uint4v*>(slice + (e * 16 + srow[i]) * PITCH +
+                                     (((scol[i] >> 4) ^ ((srow[i] / RPL) & (CPRW - 1))) << 4)) = tmp[rd * EPR + e][i];
       });
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      static_for<0, EPR>([&](auto e_) {
+        constexpr int e = decltype(e_)::value;
+        static_for<0, KS>([&](auto s_) {
+          constexpr int s2 = decltype(s_)::value;
+          u[rd * EPR + e][s2] = *reinterpret_cast<const Frag*>(slice + (e * 16 + (lane & 15)) * PITCH +
+                                                              ((((lane >> 4) + 4 * s2) ^ fswz) << 4));
+        });
+      });
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     });
   }
 
@@ -258,6 +304,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     for (int s2 = 0; s2 < KS; ++s2) asm volatile("" : "+v"(u[t][s2]));
 #pragma unroll
   for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(bv[r]));
+  __syncthreads();   // the first block's V goes where other wavefronts staged their U
 
   for (int it = 0; blk < a.n_blocks; blk += nwg, ++it) {
     unsigned char* buf = lds + (it & 1) * BUF;
@@ -373,8 +420,8 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
       }
     } else {
       // the upper wavefronts (rows 2, 3) pass their share through LDS to the lower ones (rows 0, 1)
-      floatx4* xch = reinterpret_cast<floatx4*>(lds + 2 * BUF) + ((wave & 3) * 4) * 64 + lane;
-      const bool upper = wave >= 4;
+      floatx4* xch = reinterpret_cast<floatx4*>(lds + 2 * BUF) + ((wave % KSUB) * 4) * 64 + lane;
+      const bool upper = wave >= KSUB;
 #pragma unroll
       for (int ob = 0; ob < 2; ++ob) {
         const floatx4 za = zw[0][ob], zb = zw[1][ob];
@@ -395,7 +442,7 @@ __global__ __launch_bounds__(CP * sizeof(T) > 128 ? 512 : 256) __attribute__((am
     // lane = tile lane % 16, output channels ko .. ko + 4
     const int p = blk * kThinTiles + (lane & 15);
     const int ko = kbase + 4 * (lane >> 4);
-    store_tile<T, KW>(a, ydesc, p, ko, p < a.P && ko < a.K && (!SPLIT || wave < 4), bv, out);
+    store_tile<T, KW>(a, ydesc, p, ko, p < a.P && ko < a.K && (!SPLIT || wave < KSUB), bv, out);
   }
 }
 
@@ -529,20 +576,32 @@ int launch_tiny(ThinArgs a, int k_groups, void* stream) {
   return WC_OK;
 }
 
-template <typename T, int CP>
-int launch_thin(ThinArgs a, int k_groups, void* stream) {
+template <typename T, int CP, int KSUB>
+int launch_thin_groups(ThinArgs a, void* stream) {
   constexpr bool split = CP * sizeof(T) > 128;
-  constexpr int lds = 2 * 16 * kThinTiles * CP * (int)sizeof(T) + (split ? 4 * 4 * 64 * 16 : 0);
+  constexpr int lds = 2 * 16 * kThinTiles * CP * (int)sizeof(T) + (split ? KSUB * 4 * 64 * 16 : 0);
+  const int k_groups = ceil_div(a.K, 16 * KSUB);
   // workgroups that stay resident (registers and LDS): two per CU, one of the eight-wavefront form;
   // shared among the groups of output channels, in whole multiples of the 8 XCDs
   int wgs = std::min(a.n_blocks, std::max(kXcds, (split ? 256 : 512) / k_groups / kXcds * kXcds));
   a.per_xcd = ceil_div(wgs, kXcds);
-  auto fn = a.k_whole ? &thin_conv3x3_kernel<T, CP, true> : &thin_conv3x3_kernel<T, CP, false>;
+  auto fn = a.k_whole ? &thin_conv3x3_kernel<T, CP, true, KSUB> : &thin_conv3x3_kernel<T, CP, false, KSUB>;
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
   hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds), (unsigned)k_groups),
-                     dim3(split ? 512 : 256), lds, as_stream(stream), a);
+                     dim3((split ? 128 : 64) * KSUB), lds, as_stream(stream), a);
   WC_CHECK_LAUNCH("thin_conv3x3_kernel");
   return WC_OK;
+}
+
+template <typename T, int CP>
+int launch_thin(ThinArgs a, void* stream) {
+  // half-size workgroups while the full-size ones would fill at most half of the CUs (their threads transform
+  // twice the channels each, and a thread's channels must be all inside C or all outside)
+  constexpr int vec2 = kThinTiles * CP / ((CP * sizeof(T) > 128 ? 128 : 64) * 2);
+  const int forced = test_gemm_config();            // wc_test_gemm_override: 8 = full size, 9 = half size
+  const bool half = forced == 9 || (forced != 8 && (long long)a.n_blocks * ceil_div(a.K, kThinK) * 2 <= kCus);
+  if (half && a.C % vec2 == 0) return launch_thin_groups<T, CP, 2>(a, stream);
+  return launch_thin_groups<T, CP, 4>(a, stream);
 }
 
 }  // namespace
@@ -600,10 +659,10 @@ int thin_conv_forward(const wc_conv_desc* d, const wc_plan* plan, const void* x,
   return dispatch_dtype(d->dtype, [&](auto t) -> int {
     using T = decltype(t);
     if constexpr (sizeof(T) == 2) {
-      if (Cp == 128) return launch_thin<T, 128>(a, k_groups, stream);
-      return Cp == 64 ? launch_thin<T, 64>(a, k_groups, stream) : launch_thin<T, 32>(a, k_groups, stream);
+      if (Cp == 128) return launch_thin<T, 128>(a, stream);
+      return Cp == 64 ? launch_thin<T, 64>(a, stream) : launch_thin<T, 32>(a, stream);
     } else {
-      return Cp == 64 ? launch_thin<T, 64>(a, k_groups, stream) : launch_thin<T, 32>(a, k_groups, stream);
+      return Cp == 64 ? launch_thin<T, 64>(a, stream) : launch_thin<T, 32>(a, stream);
     }
   });
 }

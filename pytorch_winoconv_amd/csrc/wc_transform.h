@@ -84,10 +84,14 @@ __device__ __forceinline__ Pack<T, VEC> buffer_load_pack(__amdgpu_buffer_rsrc_t 
   } else if constexpr (sizeof(T) * VEC == 4) {
     const unsigned raw = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
     return __builtin_bit_cast(Pack<T, VEC>, raw);
-  } else {
-    static_assert(sizeof(T) * VEC == 8, "buffer_load_pack: 2, 4 or 8 bytes per lane");
+  } else if constexpr (sizeof(T) * VEC == 8) {
     typedef unsigned u2 __attribute__((ext_vector_type(2)));
     const u2 raw = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+    return __builtin_bit_cast(Pack<T, VEC>, raw);
+  } else {
+    static_assert(sizeof(T) * VEC == 16, "buffer_load_pack: 2, 4, 8 or 16 bytes per lane");
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const u4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
     return __builtin_bit_cast(Pack<T, VEC>, raw);
   }
 }

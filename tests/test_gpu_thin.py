@@ -265,3 +265,31 @@ def test_fp32_layers_of_at_most_64_channels(dev, shape):
     assert stages["product"] > 0 and stages["input_transform"] == 0 and stages["output_transform"] == 0
     U = engine.transform_filter(wd, x.shape, 1, pad, 2)
     assert torch.equal(engine.conv_forward(xd, wd, bd, 1, pad, 2, U=U), y)
+
+
+@pytest.mark.parametrize("config", [8, 9])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_both_workgroup_sizes_are_exact_on_small_integers(dev, dtype, shape, config, gemm_override):
+    """The kernel has workgroups of 64 output channels and, for layers with few blocks of tiles, of 32 (half the
+    wavefronts, each transforming twice the channels).  The library chooses by the number of tiles; here each form is
+    forced on every shape (the small form falls back where a thread's channels would straddle C)."""
+    N, C, K, H, W, pad = shape
+    if not engine.thin_layer(dtype, 2, C, K, (3, 3), 1):
+        pytest.skip("outside the range of the one-kernel path for this type")
+    gemm_override(config=config)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(-3, 4, (N, C, H, W), generator=g).double()
+    w = 4.0 * torch.randint(-2, 3, (K, C, 3, 3), generator=g).double()
+    b = torch.randint(-8, 9, (K,), generator=g).double()
+    ref = F.conv2d(x, w, b, padding=pad).float().to(dtype)
+    xd, wd, bd = x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev)
+    yt, stages = engine.conv_forward_timed(xd, wd, bd, 1, pad, 2)
+    assert stages["product"] > 0 and stages["input_transform"] == 0 and stages["output_transform"] == 0
+    assert torch.equal(yt.cpu(), ref)
+    # normal data: both forms add in the same order, so they agree bit for bit
+    x2 = torch.randn(N, C, H, W, generator=g).to(dtype).to(dev)
+    w2 = (torch.randn(K, C, 3, 3, generator=g) * (2.0 / (9 * C)) ** 0.5).to(dtype).to(dev)
+    y_forced = engine.conv_forward(x2, w2, bd, 1, pad, 2)
+    gemm_override(config=8 if config == 9 else 9)
+    assert torch.equal(engine.conv_forward(x2, w2, bd, 1, pad, 2), y_forced)
