@@ -37,63 +37,109 @@ struct FilterFastArgs {
   int t_offset;
 };
 
-// One (k, c) of one piece with compile-time kinds: loads the taps once, transforms in registers
+// VEC channels of one k of one piece with compile-time kinds: loads the taps once, transforms in registers
 // and writes the alpha^d elements (lanes along c: coalesced rows of U).
 // `taps`: how many of the tile's taps per axis the piece really has; the others count as zero (a
 // stacked plan transforms every piece with the tile of the longest one).
-template <typename T, int K0, int K1, int K2>
+// DENSE: w is a contiguous (K, C, taps) array, the piece is the whole kernel and C a multiple of VEC, so the
+// VEC * taps values of a thread are one contiguous run, read 8 (or 4) bytes at a time.
+template <typename T, int K0, int K1, int K2, int VEC = 1, bool DENSE = false>
 __device__ __forceinline__ void transform_taps(const T* __restrict__ w, const long long (&s)[5], int k, int c,
-                                               bool ok, const int (&tap0)[3], int step, T* __restrict__ U,
+                                               int C, const int (&tap0)[3], int step, T* __restrict__ U,
                                                long long plane, const int (&taps)[3]) {
   constexpr int R0 = Mats<K0>::r, R1 = Mats<K1>::r, R2 = Mats<K2>::r;
   constexpr int A0 = Mats<K0>::alpha, A1 = Mats<K1>::alpha, A2 = Mats<K2>::alpha;
-  float g[R0 * R1 * R2][1];
-  const T* wp = w + k * s[0] + (ok ? c : 0) * s[1];
-  static_for<0, R0>([&](auto j0_) {
-    static_for<0, R1>([&](auto j1_) {
-      static_for<0, R2>([&](auto j2_) {
-        constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
-        const bool real = j0 < taps[0] && j1 < taps[1] && j2 < taps[2];
-        const float v = static_cast<float>(wp[(tap0[0] + (real ? j0 : 0) * step) * s[2] +
-                                             (tap0[1] + (real ? j1 : 0) * step) * s[3] +
-                                             (tap0[2] + (real ? j2 : 0) * step) * s[4]]);
-        g[(j0 * R1 + j1) * R2 + j2][0] = (ok && real) ? v : 0.f;
+  constexpr int R = R0 * R1 * R2;
+  float g[R][VEC];
+  if constexpr (DENSE && VEC > 1) {
+    constexpr int BYTES = VEC * R * (int)sizeof(T);
+    constexpr int CH = BYTES % 8 == 0 ? 8 : 4;             // bytes per load
+    static_assert(BYTES % CH == 0, "a thread's taps are whole 4-byte words");
+    constexpr int EPL = CH / (int)sizeof(T);               // elements per load
+    T flat[VEC * R];                                        // [channel][tap]
+    if (c < C) {
+      const T* wp = w + ((long long)k * C + c) * R;
+#pragma unroll
+      for (int i = 0; i < BYTES / CH; ++i) {
+        const Pack<T, EPL> q = *reinterpret_cast<const Pack<T, EPL>*>(wp + i * EPL);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) flat[i * EPL + e] = q.v[e];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) g[j][v] = c < C ? static_cast<float>(flat[v * R + j]) : 0.f;
+  } else {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const bool ok = c + v < C;
+      const T* wp = w + k * s[0] + (ok ? c + v : 0) * s[1];
+      static_for<0, R0>([&](auto j0_) {
+        static_for<0, R1>([&](auto j1_) {
+          static_for<0, R2>([&](auto j2_) {
+            constexpr int j0 = decltype(j0_)::value, j1 = decltype(j1_)::value, j2 = decltype(j2_)::value;
+            const bool real = j0 < taps[0] && j1 < taps[1] && j2 < taps[2];
+            const float val = static_cast<float>(wp[(tap0[0] + (real ? j0 : 0) * step) * s[2] +
+                                                   (tap0[1] + (real ? j1 : 0) * step) * s[3] +
+                                                   (tap0[2] + (real ? j2 : 0) * step) * s[4]]);
+            g[(j0 * R1 + j1) * R2 + j2][v] = (ok && real) ? val : 0.f;
+          });
+        });
       });
-    });
-  });
-  float u2[R0 * R1 * A2][1];
-  apply_axis<MatG<K2>, 2, R0, R1, R2, 1>(g, u2);
-  float u1[R0 * A1 * A2][1];
-  apply_axis<MatG<K1>, 1, R0, R1, A2, 1>(u2, u1);
-  float u0[A0 * A1 * A2][1];
-  apply_axis<MatG<K0>, 0, R0, A1, A2, 1>(u1, u0);
+    }
+  }
+  float u2[R0 * R1 * A2][VEC];
+  apply_axis<MatG<K2>, 2, R0, R1, R2, VEC>(g, u2);
+  float u1[R0 * A1 * A2][VEC];
+  apply_axis<MatG<K1>, 1, R0, R1, A2, VEC>(u2, u1);
+  float u0[A0 * A1 * A2][VEC];
+  apply_axis<MatG<K0>, 0, R0, A1, A2, VEC>(u1, u0);
   static_for<0, A0 * A1 * A2>([&](auto e_) {
     constexpr int e = decltype(e_)::value;
-    U[e * plane] = static_cast<T>(u0[e][0]);
+    store_pack<T, VEC>(U + e * plane, u0[e]);
   });
 }
 
-// Single piece with compile-time kinds: one thread per (k, c).
+// Channels per thread of the single-piece kernel: 8-byte stores for 2-D tiles, 2 channels for the 64 elements of
+// F(2,3)^3, one for the 144 of F(2,3) x F(4,3)^2 (registers).
 template <typename T, int K0, int K1, int K2>
+constexpr int fast_vec() {
+  constexpr int elems = Mats<K0>::alpha * Mats<K1>::alpha * Mats<K2>::alpha;
+  return elems <= 36 ? 8 / (int)sizeof(T) : elems <= 64 ? 2 : 1;
+}
+
+// Single piece with compile-time kinds: one thread per (k, VEC channels).
+template <typename T, int K0, int K1, int K2, bool DENSE>
 __global__ __launch_bounds__(256) void filter_transform_fast_kernel(const FilterFastArgs a) {
+  constexpr int VEC = fast_vec<T, K0, K1, K2>();
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= a.K * a.Cp) return;
-  const int c = idx % a.Cp, k = idx / a.Cp;
-  T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + idx;
+  const int cvecs = a.Cp / VEC;
+  if (idx >= a.K * cvecs) return;
+  const int c = (idx % cvecs) * VEC, k = idx / cvecs;
+  T* U = static_cast<T*>(a.U) + (long long)a.t_offset * a.K * a.Cp + (long long)k * a.Cp + c;
   const int all[3] = {Mats<K0>::r, Mats<K1>::r, Mats<K2>::r};
-  transform_taps<T, K0, K1, K2>(static_cast<const T*>(a.w), a.s, k, c, c < a.C, a.tap0, a.step, U,
-                                (long long)a.K * a.Cp, all);
+  transform_taps<T, K0, K1, K2, VEC, DENSE>(static_cast<const T*>(a.w), a.s, k, c, a.C, a.tap0, a.step, U,
+                                            (long long)a.K * a.Cp, all);
 }
 
 using FilterFastKernel = void (*)(FilterFastArgs);
 
-template <typename T>
+template <typename T, bool DENSE>
 static FilterFastKernel pick_fast(int k0, int k1, int k2) {
-  if (k0 == KIND_11 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_11, KIND_43, KIND_43>;
-  if (k0 == KIND_11 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_11, KIND_23, KIND_23>;
-  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_23, KIND_23, KIND_23>;
-  if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_23, KIND_43, KIND_43>;
+  if (k0 == KIND_11 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_11, KIND_43, KIND_43, DENSE>;
+  if (k0 == KIND_11 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_11, KIND_23, KIND_23, DENSE>;
+  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23) return &filter_transform_fast_kernel<T, KIND_23, KIND_23, KIND_23, DENSE>;
+  if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43) return &filter_transform_fast_kernel<T, KIND_23, KIND_43, KIND_43, DENSE>;
   return nullptr;
+}
+
+// channels per thread of the kernel pick_fast returns (0: none)
+static int fast_vec_of(int dtype, int k0, int k1, int k2) {
+  const int es = dtype == WC_F32 ? 4 : 2;
+  if (k0 == KIND_11) return 8 / es;
+  if (k0 == KIND_23 && k1 == KIND_23) return 2;
+  return 1;
 }
 
 struct FilterArgs {
@@ -129,10 +175,9 @@ __global__ __launch_bounds__(256) void filter_transform_pieces_kernel(const Filt
   T* U = static_cast<T*>(a.U) + (long long)pc.t_offset * plane + (long long)k * row +
          (a.stacked ? (int)blockIdx.y * a.Cp : 0) + c;
   const T* w = static_cast<const T*>(a.w);
-  const bool ok = c < a.C;
   const int r0 = a.stacked ? a.rp[0] : pc.r[0], r1 = a.stacked ? a.rp[1] : pc.r[1], r2 = a.stacked ? a.rp[2] : pc.r[2];
   constexpr int KA = MO == 4 ? KIND_41 : KIND_21, KB = MO == 4 ? KIND_42 : KIND_22, KC = MO == 4 ? KIND_43 : KIND_23;
-#define WC_BODY(K0, K1, K2) transform_taps<T, K0, K1, K2>(w, a.s, k, c, ok, pc.tap0, a.step, U, plane, pc.r)
+#define WC_BODY(K0, K1, K2) transform_taps<T, K0, K1, K2>(w, a.s, k, c, a.C, pc.tap0, a.step, U, plane, pc.r)
 #define WC_ROW(K0, K1) \
   switch (r2) { case 1: WC_BODY(K0, K1, KA); break; case 2: WC_BODY(K0, K1, KB); break; default: WC_BODY(K0, K1, KC); }
 #define WC_PLANE(K0) \
@@ -203,7 +248,16 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
   if (plan->n_pieces == 1) {
     const wc_piece& pc = plan->piece[0];
     const int k0 = kind_of(plan->m[0], pc.r[0]), k1 = kind_of(plan->m[1], pc.r[1]), k2 = kind_of(plan->m[2], pc.r[2]);
-    FilterFastKernel fn = dispatch_dtype(d->dtype, [&](auto t) { return pick_fast<decltype(t)>(k0, k1, k2); });
+    const int vec = fast_vec_of(d->dtype, k0, k1, k2);
+    // a contiguous (K, C, taps) filter whose channels split evenly among the threads is read in 8-byte pieces
+    const long long taps = (long long)pc.r[0] * pc.r[1] * pc.r[2];
+    const bool dense = w_strides[4] == 1 && w_strides[3] == pc.r[2] && (pc.r[0] == 1 || w_strides[2] == (long long)pc.r[1] * pc.r[2]) &&
+                       w_strides[1] == taps && w_strides[0] == taps * d->C && plan->tap_step == 1 &&
+                       pc.tap0[0] == 0 && pc.tap0[1] == 0 && pc.tap0[2] == 0 && vec > 1 && d->C % vec == 0 &&
+                       (reinterpret_cast<uintptr_t>(w) & 7) == 0;
+    FilterFastKernel fn = dispatch_dtype(d->dtype, [&](auto t) {
+      return dense ? pick_fast<decltype(t), true>(k0, k1, k2) : pick_fast<decltype(t), false>(k0, k1, k2);
+    });
     if (fn) {
       FilterFastArgs f;
       f.w = w; f.U = U;
@@ -212,7 +266,7 @@ extern "C" int wc_filter_transform(const wc_conv_desc* d, const wc_plan* plan, c
       for (int i = 0; i < 3; ++i) f.tap0[i] = pc.tap0[i];
       f.step = plan->tap_step;
       f.t_offset = pc.t_offset;
-      const long long n = (long long)d->K * f.Cp;
+      const long long n = (long long)d->K * (f.Cp / vec);
       WC_CHECK_ARG(n < (1ll << 31), "wc_filter_transform: problem too large");
       hipLaunchKernelGGL(fn, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, as_stream(stream), f);
       WC_CHECK_LAUNCH("filter_transform_fast_kernel");
