@@ -459,16 +459,25 @@ def main():
     ws = engine._w_strides(w)
     px, pw, pU, pV, pM, py = (engine._ptr(t) for t in (x_cl, w, U, V, Mb, y))
 
+    pws, nws = engine._ptr(wsbuf), nb.value
+
     def step(ev=None):
-        if ev: ev[0].record()
+        """One pass of the layer into y.  Without events: one call of wc_conv_forward, the entry point a caller of
+        the reference's DWM binds, on the caller-provided workspace.  With events: the same four stages through
+        their own entry points (what wc_conv_forward runs inside, except that it transforms the filter in the
+        launch of the input transform), with a record between them."""
+        if not ev:
+            _lib.check(lib.wc_conv_forward(d_, px, pw, ws, None, None, py, pws, nws, st))
+            return
+        if ev[0]: ev[0].record()
         _lib.check(lib.wc_filter_transform(d_, p_, pw, ws, pU, st))
-        if ev: ev[1].record()
+        if ev[1]: ev[1].record()
         _lib.check(lib.wc_input_transform(d_, p_, px, N, pV, st))
-        if ev: ev[2].record()
+        ev[2].record()
         _lib.check(lib.wc_batched_gemm(pV, pU, pM, T, P, Cp, K, ldm, desc.dtype, st))
-        if ev: ev[3].record()
+        ev[3].record()
         _lib.check(lib.wc_output_transform(d_, p_, pM, None, N, py, st))
-        if ev: ev[4].record()
+        if ev[4]: ev[4].record()
 
     if args.copy_probe:
         src = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=dev)
@@ -477,22 +486,27 @@ def main():
             dst.copy_(src)
     # Untimed steps for a fixed wall time first: a GPU that has been idle needs a few tenths of a second of
     # work to reach its steady clocks, far more than a handful of 0.25 ms warm-up steps provide.
+    # The untimed steps mix the two forms of a step like the timed ones (a kernel's first launch loads its code).
+    spare = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
     t_pre = time.perf_counter()
     while time.perf_counter() - t_pre < args.prewarm:
-        for _ in range(10):
-            step()
+        for i in range(10):
+            step(spare if i % args.event_every == 0 else None)
         torch.cuda.synchronize()
     prewarm_s = time.perf_counter() - t_pre
-    for _ in range(args.warmup):
-        step()
+    for i in range(args.warmup):
+        step(spare if i % args.event_every == 0 else None)
     torch.cuda.synchronize()
-    # Stage durations come from HIP events inside the timed region, on every fourth step by default
-    # (--event-every): they agree with the profiler's kernel durations (120.6 against 120.4 us for
-    # the GEMM on one box).  A step with event records takes about 13 us longer than one without
-    # (0.252 against 0.239 ms measured with events on every step / on none), because each record
-    # sits between two kernels; the steps without records run the same four C-ABI calls.
+    # The batched GEMM, the kernel of the roofline figure, is bracketed by two HIP events inside the timed region,
+    # on every fourth step by default (--event-every); its average agrees with the profiler's kernel duration
+    # (120.6 against 120.4 us on one box).  Those steps run the four stage entry points; the steps without
+    # records are single calls of wc_conv_forward.  The other stages are timed the same way, with a record between
+    # every two of them, in a few untimed steps right afterwards (a step with five records takes about 13 us
+    # longer than one with none, because each record sits between two kernels).
     sampled = [i % args.event_every == 0 for i in range(args.steps)]
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] if s else None for s in sampled]
+    def gemm_events():
+        return [None, None, torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), None]
+    events = [gemm_events() if s else None for s in sampled]
     t0 = time.perf_counter()
     for ev in events:
         step(ev)
@@ -502,13 +516,21 @@ def main():
 
     names = ("filter_transform", "input_transform", "batched_gemm", "output_transform")
     timed = [ev for ev in events if ev]
-    stage_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in timed) / len(timed) * 1e3
+    gemm_us = sum(ev[2].elapsed_time(ev[3]) for ev in timed) / len(timed) * 1e3
+    after = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(8)]
+    for ev in after:
+        step(ev)
+    torch.cuda.synchronize()
+    stage_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in after) / len(after) * 1e3
                 for i, n in enumerate(names)}
+    stage_us["batched_gemm"] = gemm_us          # the one measured inside the timed region
 
     # the product's one-call entry point on the same inputs, for comparison
     def one_call():
         return engine.conv_forward(x, w, None, 1, PAD, M_TILE)
     y1 = one_call()
+    y.zero_()
+    step([torch.cuda.Event(enable_timing=True) for _ in range(5)])      # y from the four stage entry points
     torch.cuda.synchronize()
     same = bool(torch.equal(y1.permute(0, 2, 3, 1), y))
     def best_of_three(fn):
@@ -565,6 +587,7 @@ def main():
         "ms_per_layer_filter_cached": ms_cached,
         "effective_tflops_filter_cached": direct_flops / (ms_cached * 1e-3) / 1e12,
         "one_call_matches_stages": same,
+        "timed_steps": {"wc_conv_forward": sampled.count(False), "four_stage_calls_with_events": sampled.count(True)},
     }
     if args.suite or args.suite_only:
         result["suite"] = run_suite(only=args.suite_only)

@@ -244,11 +244,14 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
   void* Ycl = tail + L.xcl_bytes;
   StageTimer timer(stage_ms != nullptr, stream);
   const void* U = U_cached;
-  if (!U) {
+  // the three-kernel path transforms the filter in the launch of the first chunk's input transform (unless the
+  // stages are being timed one by one)
+  bool filter_with_input = !U && !stage_ms && !L.thin && !L.direct;
+  if (!U && !filter_with_input) {
     rc = timer.run(WC_STAGE_FILTER, [&] { return wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream); });
     if (rc) return rc;
-    U = Uws;
   }
+  if (!U) U = Uws;
   wc_conv_desc dcl = *d;                  // the stages behind a scratch copy see channel-last tensors
   dcl.x_layout = L.x_direct ? 1 : 0;
   dcl.y_layout = 0;
@@ -277,8 +280,12 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
     } else {
       const long long P = L.tiles_per_image * n;
       WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
-      rc = timer.run(WC_STAGE_INPUT, [&] { return wc_input_transform(&dcl, &L.plan, xin, n, V, stream); });
+      rc = timer.run(WC_STAGE_INPUT, [&] {
+        return filter_with_input ? input_filter_transform(&dcl, &L.plan, xin, n, V, w, w_strides, Uws, stream)
+                                 : wc_input_transform(&dcl, &L.plan, xin, n, V, stream);
+      });
       if (rc) return rc;
+      filter_with_input = false;
       rc = timer.run(WC_STAGE_PRODUCT, [&] {
         return L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
                         : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);

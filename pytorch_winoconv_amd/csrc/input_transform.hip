@@ -1,11 +1,16 @@
 // Host entry of the input transform: picks the kernel of each piece and launches it.
+#include "filter_transform_impl.h"
 #include "input_transform_impl.h"
 #include <algorithm>
 
 using namespace wc;
 
-extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x,
-                                  int n_images, void* V, void* stream) {
+namespace {
+
+// filt: the filter transform of the same call, to be run in the same launch where a kernel for that exists;
+// *filt_done tells whether it was
+int input_transform_impl(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V, void* stream,
+                         const FilterFastArgs* filt, bool* filt_done) {
   WC_CHECK_ARG(d && plan && x && V, "wc_input_transform: null pointer");
   WC_CHECK_ARG(n_images > 0, "wc_input_transform: n_images %d", n_images);
   int out[3], grid[3];
@@ -163,8 +168,43 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
     a.base0 = pc.tap0[0] - d->pad[0]; a.base1 = pc.tap0[1] - d->pad[1]; a.base2 = pc.tap0[2] - d->pad[2];
     a.t_offset = pc.t_offset;
     a.V = static_cast<char*>(V) + (stacked ? (long long)s * Cp * (d->dtype == WC_F32 ? 4 : 2) : 0);
+    if (filt && plan->n_pieces == 1 && k[0] == KIND_11) {
+      if (InFilterKernel both = pick_in_filter_2d(d->dtype, k[1], k[2], vec)) {
+        const int fv = in_filter_vec(d->dtype == WC_F32 ? 4 : 2, k[1]);
+        const long long fb = ceil_div_ll((long long)filt->K * (filt->Cp / fv), 256);
+        if (fb + launch_grid.x < (1ll << 31)) {
+          hipLaunchKernelGGL(both, dim3((unsigned)(fb + launch_grid.x)), dim3(256), 0, as_stream(stream), a, *filt, (int)fb);
+          WC_CHECK_LAUNCH("input_filter_kernel");
+          *filt_done = true;
+          continue;
+        }
+      }
+    }
     hipLaunchKernelGGL(fn, launch_grid, dim3(256), 0, as_stream(stream), a);
     WC_CHECK_LAUNCH("input_transform_kernel");
   }
   return WC_OK;
 }
+
+}  // namespace
+
+extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x,
+                                  int n_images, void* V, void* stream) {
+  return input_transform_impl(d, plan, x, n_images, V, stream, nullptr, nullptr);
+}
+
+namespace wc {
+
+int input_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V,
+                           const void* w, const int64_t w_strides[5], void* U, void* stream) {
+  WC_CHECK_ARG(w && w_strides && U, "input_filter_transform: null pointer");
+  FilterFastArgs f;
+  int vec = 1;
+  bool dense = false, done = false;
+  const bool try_both = d->x_layout == 0 && filter_fast_setup(d, plan, w, w_strides, U, &f, &vec, &dense) && dense;
+  int rc = input_transform_impl(d, plan, x, n_images, V, stream, try_both ? &f : nullptr, &done);
+  if (rc || done) return rc;
+  return wc_filter_transform(d, plan, w, w_strides, U, stream);
+}
+
+}  // namespace wc

@@ -145,6 +145,11 @@ InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec);    // ... whole-k
 InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
 InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
 InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);
+struct FilterFastArgs;
+// channels per thread of the filter part of that launch
+constexpr int in_filter_vec(int elem_bytes, int k1) { return elem_bytes == 4 && k1 == KIND_43 ? 1 : 8 / elem_bytes; }
+using InFilterKernel = void (*)(InArgs, FilterFastArgs, int);
+InFilterKernel pick_in_filter_2d(int dtype, int k1, int k2, int vec);   // 3x3 kernels, tile 2 or 4, with the filter transform in the same launch; nullptr otherwise
 InKernel pick_in_3d_planes(int dtype, int vec);                   // tile 2 x 4 x 4 of a 3x3x3 kernel, plane by plane, vec 2 or 1
 
 }  // namespace wc

@@ -150,6 +150,10 @@ __device__ __forceinline__ int xcd_remap(int hw_id, int per_xcd) {
 
 // acc (taps, K, C) (+)= G^T dU G per piece of the plan; dU (T, S, K, ldc) with the parts already
 // summed into part 0; `first` overwrites acc instead of adding (backward_filter.hip).
+// wc_input_transform and wc_filter_transform of one call: one launch where a kernel holds both (single-piece 2-D
+// plans of 3x3 kernels with a dense filter), two launches otherwise
+int input_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V,
+                           const void* w, const int64_t w_strides[5], void* U, void* stream);
 int grad_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const float* dU, float* acc, int ldc, int S,
                           bool first, void* stream);
 

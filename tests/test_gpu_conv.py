@@ -213,3 +213,46 @@ def test_empty_batch_and_single_pixel_outputs(dev):
         ref = _conv64(x, wt, b, stride, pad)
         yy = engine.conv_forward(x.to(dev), wt.to(dev), b.to(dev), stride, pad, m)
         assert tuple(yy.shape) == tuple(ref.shape) and _nerr(yy, ref) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("m", [2, 4])
+@pytest.mark.parametrize("shape", [
+    # N, C, K, H, W
+    (3, 64, 72, 13, 11),       # dense filter, channels split evenly: one launch for both transforms
+    (2, 256, 40, 9, 9),
+    (2, 36, 24, 10, 12),       # channels padded to 64
+    (2, 30, 16, 8, 8),         # fp16: 30 channels are no multiple of the filter threads' 4: two launches
+    (5, 8, 8, 30, 30),
+])
+def test_filter_transformed_beside_the_input_equals_the_separate_launches(dev, dtype, m, shape):
+    """With a fresh filter the three-kernel path of a 3x3 layer transforms the filter in the first workgroups of the
+    input transform's launch.  Same arithmetic, so: bit-equal to a call with the filter transformed beforehand, to
+    the stage-by-stage (timed) call and to a call with a second chunk of images; a filter in the reference's (kH, kW, C, K)
+    memory is read through strides by another kernel in a launch of its own; integer inputs come out exact."""
+    N, C, K, H, W = shape
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(N, C, H, W, generator=g).to(dtype).to(dev)
+    w = (torch.randn(K, C, 3, 3, generator=g) * (2.0 / (9 * C)) ** 0.5).to(dtype).to(dev)
+    b = torch.randn(K, generator=g).to(dtype).to(dev)
+    kw = dict(unfused=True)              # thin layers would take the one-kernel path
+    y = engine.conv_forward(x, w, b, 1, 1, m, **kw)
+    U = engine.transform_filter(w, x.shape, 1, 1, m)
+    assert torch.equal(engine.conv_forward(x, w, b, 1, 1, m, U=U, **kw), y)
+    yt, stages = engine.conv_forward_timed(x, w, b, 1, 1, m, **kw)
+    assert torch.equal(yt, y) and stages["filter_transform"] > 0 and stages["input_transform"] > 0
+    w_ref = w.permute(2, 3, 1, 0).contiguous().permute(3, 2, 0, 1)       # same values, (kH, kW, C, K) memory
+    assert not w_ref.is_contiguous() and torch.equal(w_ref, w)
+    y_ref = engine.conv_forward(x, w_ref, b, 1, 1, m, **kw)      # another filter kernel: equal to the last bit or two
+    assert float((y_ref.double() - y.double()).abs().max() / y.double().abs().max()) <= {torch.float32: 1e-6, torch.float16: 4e-3, torch.bfloat16: 3e-2}[dtype]
+    if N > 1:
+        assert torch.equal(engine.conv_forward(x, w, b, 1, 1, m, chunk_images=N - 1, **kw), y)
+    ref = F.conv2d(x.double().cpu(), w.double().cpu(), b.double().cpu(), padding=1)
+    tol = {torch.float32: 1e-3, torch.float16: 2e-2, torch.bfloat16: 2e-2 if m == 2 else 2e-1}[dtype]      # bf16 with tile 4: as everywhere
+    assert float((y.double().cpu() - ref).abs().max() / ref.abs().max()) <= tol
+    xi = torch.randint(-3, 4, (N, C, H, W), generator=g).double()
+    wi = (4.0 if m == 2 else 24.0) * torch.randint(-2, 3, (K, C, 3, 3), generator=g).double()      # G g G^T stays integral
+    if float(F.conv2d(xi, wi, padding=1).abs().max()) < (2048 if dtype == torch.float16 else 256 if dtype == torch.bfloat16 else 1 << 24):
+        yi = engine.conv_forward(xi.to(dtype).to(dev), wi.to(dtype).to(dev), None, 1, 1, m, **kw)
+        if m == 2:
+            assert torch.equal(yi.cpu().double(), F.conv2d(xi, wi, padding=1))
