@@ -93,7 +93,7 @@ def cpu_baseline(sample_images=32, repeats=3):
 
 
 SUITE = [
-    # name, x shape, w shape, stride, pad, m, dtype  (BASELINE.json configs[0..4] at full size).
+    # name, x shape, w shape, stride, pad, m, dtype  (the five benchmark configurations c1..c5 at full size).
     # c3, 64 and 128 channels: the default is the fused F(2,3) kernel; the three-kernel F(4,3) line stands beside it.
     # c4: the 16-bit default adds the DWM pieces in the batched GEMM; at stride 1 the pieces share one
     # transformed input (tile 3 / F(3,3) with the reference's three-tap pieces where the caller asks for tile 4,
@@ -138,7 +138,7 @@ VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256
          (512, 512, 14)]
 
 
-# the default form of every configuration of BASELINE.json: what a plain `python bench.py` adds to its JSON line
+# the default form of every benchmark configuration (c1..c5): what a plain `python bench.py` adds to its JSON line
 DEFAULTS = ("c1 ", "c2 vgg16 fp32 N8 F(4,3)", "c2 vgg16 fp32 N8 F(2,3)", "c3 fp16 N64 C64 56x56 F(2,3)", "c3 fp16 N64 C128 28x28 F(2,3)",
             "c3 fp16 N64 C256", "c3 fp16 N64 C512", "5x5 s1 DWM shared input F(3,3)", "7x7 s1 DWM shared input F(3,3)",
             "3x3 s2 direct form", "7x7 s2 direct form", "c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3")
@@ -401,7 +401,7 @@ def main():
                     help="force tile shape I of the batched GEMM through the library's test hook (-1: its own choice)")
     ap.add_argument("--suite", action="store_true",
                     help="time every form of every other benchmark configuration (the 'suite' list); without it the "
-                         "list holds the default form of each configuration of BASELINE.json (c1..c5), about 20 s")
+                         "list holds the default form of each benchmark configuration (c1..c5), about 20 s")
     ap.add_argument("--no-suite", action="store_true", help="no 'suite' list at all: the metric layer only")
     ap.add_argument("--event-every", type=int, default=4, metavar="N",
                     help="record the per-stage HIP events on every N-th timed step (an event record between two "

@@ -277,7 +277,7 @@ def test_stride_2_is_exact_on_small_integers(dev, case):
 
 
 def test_c4_stride_2_layer_at_full_size(dev):
-    """BASELINE configuration c4, 7x7 stride 2 (fp16, N=32, 128 channels, 112x112): the default plan is
+    """Benchmark configuration c4, 7x7 stride 2 (fp16, N=32, 128 channels, 112x112): the default plan is
     the shared-input one; checked against torch's own GPU convolution accumulated in fp32."""
     g = torch.Generator().manual_seed(0)
     x = torch.randn(32, 128, 112, 112, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
