@@ -1,5 +1,5 @@
-// One-kernel F(2x2, 3x3) convolution for thin layers: fp16 / bf16 with at most 128 input channels, and any
-// storage type with at most 4 (tiny_conv3x3_kernel, further down).
+// One-kernel F(2x2, 3x3) convolution for thin layers: fp16 / bf16 with at most 128 input channels, fp32 with at
+// most 64, and any storage type with at most 4 (tiny_conv3x3_kernel, further down).
 //
 // Same arithmetic as the three-kernel path (input transform of src/split_kernel.cu:60-120, the
 // batched product of src/base_conv_launchers.cu:353-367, output transform of
@@ -20,6 +20,8 @@
 // double-buffered, so there is one barrier per block.  With 128 channels U would take the whole
 // register file: eight wavefronts then share a block, four per pair of element rows, and the
 // upper four hand their share of each output tile to the lower four through LDS (a second barrier).
+// Launches with few blocks of tiles use workgroups of half the size (32 output channels), and U reaches the
+// registers through LDS: see thin_conv3x3_kernel.
 #include "wc_transform.h"
 #include <algorithm>
 
