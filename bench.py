@@ -154,7 +154,7 @@ def run_suite(steps=10, only=None, defaults=False):
     dev = torch.device("cuda:0")
     out = []
 
-    def one(xs, ws, stride, pad, m, dt):
+    def one(xs, ws, stride, pad, m, dt, steps=steps):
         dtype = torch.float32 if dt == "f32" else torch.float16
         # None: the engine's default (16-bit: stride-1 kernels of 4..8 taps share one transformed input,
         # other DWM plans are stacked)
@@ -173,10 +173,16 @@ def run_suite(steps=10, only=None, defaults=False):
         y = engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
         torch.cuda.synchronize()
         t_warm = time.perf_counter()
+        warm_calls = 0
         while time.perf_counter() - t_warm < 0.15:
             for _ in range(5):
                 engine.conv_forward(x, w, None, stride, pad, m, stacked=stacked, unfused=unfused, direct=direct)
             torch.cuda.synchronize()
+            warm_calls += 5
+        # calls per timed round: at least `steps`, and enough of them for about 3 ms, so that the one wait for the
+        # device at the end of a round is not a visible part of a layer that takes 10 us (it was, at 10 calls)
+        per_call = (time.perf_counter() - t_warm) / warm_calls
+        steps = max(steps, min(1000, int(3e-3 / per_call) + 1))
         # best of three rounds: a single round now and then includes a stall of tens of milliseconds
         # (the caching allocator returning memory between configurations of very different sizes)
         ms = float("inf")
