@@ -9,7 +9,7 @@
  * device: work is enqueued on the caller's stream and scratch memory comes from the
  * caller (`workspace`).  Nothing a call computes depends on earlier calls; the library
  * only remembers which of its kernels it has already granted more than 64 KB of LDS on
- * which device (and what the test hook wc_test_gemm_override last set).
+ * which device (the test hook wc_test_gemm_override is inert unless the process opts in).
  *
  * Data layouts (row-major, innermost last).  "Channel-last" means NHWC / NDHWC.
  *   x   (N, D, H, W, C)        D = 1 for 2-D problems (or channel-first, see wc_conv_desc.x_layout)
@@ -120,9 +120,11 @@ typedef struct {
                     *    operand, walks the taps along its reduction axis and writes y; no V or M in memory, U is the
                     *    filter as (K, kH, kW, C).  2-D, C a multiple of 32 (fp32: 16), K a multiple of 8; m, stacked
                     *    and whole_kernel are ignored.  wc_conv_auto chooses it for kernels of one tap (every type: the
-                    *    tile F(m,1) saves nothing and its transforms are copies) and for 16-bit layers at stride 2, which
-                    *    the reference does not implement (src/winograd_conv.cpp:122-126) and where Winograd tiles on
-                    *    the parity phases save few or no multiplications.  wc_conv_forward, wc_filter_transform,
+                    *    tile F(m,1) saves nothing and its transforms are copies), for 16-bit layers at stride 2 (short
+                    *    reductions always, longer ones where the output fills the chip) and for fp32 3x3 layers at
+                    *    stride 2 over at most 128 channels: strides the reference does not implement
+                    *    (src/winograd_conv.cpp:122-126) and where Winograd tiles on the parity phases save few or no
+                    *    multiplications.  wc_conv_forward, wc_filter_transform,
                     *    wc_conv_workspace_bytes and wc_conv_u_elems honour it; the other stage functions do not apply. */
 } wc_conv_desc;
 
@@ -138,7 +140,9 @@ const char* wc_last_error(void);
  * choice by size (1, the default) or one tile per run of pieces wherever the plan has runs (2).
  * config 8 / 9: the one-kernel F(2x2,3x3) path with workgroups of 64 / 32 output channels whatever
  * the number of tiles (9 only where the channel count allows it).
- * Process-wide; production code never calls it. */
+ * Works only in a process started with WINOCONV_TEST_HOOKS=1 in its environment (WC_ERR_UNSUPPORTED
+ * otherwise, and nothing changes); what it sets holds for the calling host thread only, so a caller
+ * cannot change what the launches of another thread do.  Production code never calls it. */
 int wc_test_gemm_override(int config, int rows_mode);
 
 /* ---- planning (host only) --------------------------------------------------------------- */

@@ -129,7 +129,10 @@ class _WinoConvNd(nn.Module):
             return conv(x, self.weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
         w = self.weight.to(x.dtype)
         m = self._tile_for(x.dtype)
-        key = (self.weight._version, self.weight.data_ptr(), tuple(x.shape[2:]), x.dtype, m)
+        # the form of the plan (Winograd pieces, or the direct form the library takes for large strided problems)
+        # depends on the batch size too, and the transformed filter of one form does not fit the other
+        form = engine.plan_form(x.shape, w.shape, x.dtype, self.stride[0], self.padding, m)
+        key = (self.weight._version, self.weight.data_ptr(), tuple(x.shape[2:]), x.dtype, m, form)
         if self._cache is None or self._cache[0] != key:
             U = engine.transform_filter(w.detach(), x.shape, self.stride[0], self.padding, m)
             self._cache = (key, U)

@@ -141,8 +141,8 @@ def winograd_conv(Input, Weight, Output, bias=None, stride=1, padding=0, m=2, al
     if isinstance(padding, int):
         padding = (0 if flat else padding, padding, padding)
     w_kc = Weight.permute(4, 3, 0, 1, 2)                 # (K, C, kD, kH, kW) view, no copy
-    stacked = engine._stack(stacked, Input.dtype, 2 if flat else 3, whole,
-                            (K, C, kH, kW) if flat else (K, C, kD, kH, kW), stride, m)
+    # `stacked` left open (None) goes to the library as it is, which then also may take the direct form: the same
+    # call of wc_conv_auto that the compiled host layer makes, so both bindings run the same plan
     unfused = engine.misaligned(Input, Output, U)        # the one-kernel path of thin layers wants 16-byte alignment
     if flat:
         desc = make_desc((B, C, H, W), (K, C, kH, kW), Input.dtype, stride, padding[1:], m, chunk_images, whole,

@@ -322,6 +322,8 @@ bool one_tap_layout(const wc_conv_desc* d, BwdLayout* L) {
 
 int make_bwd_layout(const wc_conv_desc* d, BwdLayout* L) {
   WC_CHECK_ARG(d != nullptr, "null descriptor");
+  WC_CHECK_ARG(d->dtype == WC_F32 || d->dtype == WC_F16 || d->dtype == WC_BF16, "dtype %d", d->dtype);
+  WC_CHECK_ARG((d->ndim == 2 || d->ndim == 3) && d->N > 0 && d->C > 0 && d->K > 0, "ndim %d, N %d, C %d, K %d", d->ndim, d->N, d->C, d->K);
   L->one_tap = L->gathered = false;
   if (one_tap_layout(d, L)) return WC_OK;
   if (gathered_layout(d, L)) return WC_OK;
@@ -377,7 +379,7 @@ extern "C" {
 
 int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* d, size_t* bytes) {
   WC_CHECK_ARG(bytes != nullptr, "wc_conv_backward_weight_workspace_bytes: null output");
-  BwdLayout L;
+  BwdLayout L{};
   int rc = make_bwd_layout(d, &L);
   if (rc) return rc;
   *bytes = L.v_bytes + L.dm_bytes + L.du_bytes + L.acc_bytes;
@@ -386,7 +388,7 @@ int wc_conv_backward_weight_workspace_bytes(const wc_conv_desc* d, size_t* bytes
 
 int wc_conv_backward_weight(const wc_conv_desc* d, const void* x, const void* dy, void* dw,
                             const int64_t dw_strides[5], void* workspace, size_t workspace_bytes, void* stream) {
-  BwdLayout L;
+  BwdLayout L{};
   int rc = make_bwd_layout(d, &L);
   if (rc) return rc;
   WC_CHECK_ARG(x && dy && dw && dw_strides, "wc_conv_backward_weight: null pointer");

@@ -329,9 +329,14 @@ int wc_conv_forward_static(const wc_conv_desc* d, const void* x, const void* w, 
     long long fit = per_image ? 1 + (long long)((cap - L.need()) / per_image) : 1;
     if (fit > d->N) fit = d->N;
     if (d->chunk_images > 0 && d->chunk_images < fit) fit = d->chunk_images;
-    dd.chunk_images = (int)fit;
-    rc = make_layout(&dd, &L);
-    if (rc) return rc;
+    // the estimate ignores that V, M and the layout copies are each rounded up to 256 bytes: step down until it fits
+    for (;;) {
+      dd.chunk_images = (int)fit;
+      rc = make_layout(&dd, &L);
+      if (rc) return rc;
+      if (L.need() <= cap || fit <= 1) break;
+      --fit;
+    }
     if (L.need() > cap) return fail(WC_ERR_WORKSPACE, "wc_conv_forward_static: chunk of %d images needs %zu bytes", dd.chunk_images, L.need());
   }
   void* ws = nullptr;

@@ -17,6 +17,7 @@
 #include <sstream>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../../include/winoconv.h"
@@ -64,25 +65,51 @@ void* stream_of(const at::Tensor& t) {
 }
 
 // Workspace of a call.  Small ones (the filter of a one-kernel layer: a few hundred KB, where the 1.6 us of an
-// allocation is a visible part of a 10 us call) are kept, one per thread, device and stream: calls on one stream
-// run in order, so the next call may write where the last one read.  Never freed (a tensor destroyed at thread or
-// process exit would reach the allocator after the runtime has gone).  A stream under capture gets a fresh
-// allocation from the graph's own pool instead.
+// allocation is a visible part of a 10 us call) are kept per thread, device and stream: calls on one stream
+// run in order, so the next call may write where the last one read.  A thread keeps at most kKeptSlots of them
+// (4 MB): a further (device, stream) pair takes the slot used longest ago, whose tensor goes back to the caching
+// allocator, which hands a block to later allocations of the stream it was allocated on only, in stream order.
+// A thread that ends returns its workspaces; the thread that imported the module keeps them until the process ends
+// (its thread-local objects are destroyed during exit(), when the interpreter has already been finalised).
+// A stream under capture gets a fresh allocation from the graph's own pool instead.
+const std::thread::id g_import_thread = std::this_thread::get_id();
+
+struct KeptWorkspaces {
+  struct Kept { int device; void* stream; at::Tensor ws; uint64_t used; };
+  std::vector<Kept> slots;
+  uint64_t clock = 0;
+  ~KeptWorkspaces() {
+    if (std::this_thread::get_id() == g_import_thread) new std::vector<Kept>(std::move(slots));   // never freed
+  }
+};
+
 at::Tensor workspace_for(const at::Tensor& like, size_t bytes, void* stream) {
   constexpr size_t kKept = 1u << 20;
+  constexpr size_t kKeptSlots = 4;
   auto fresh = [&](size_t n) { return at::empty({(int64_t)n}, like.options().dtype(at::kByte)); };
   if (bytes > kKept) return fresh(bytes);
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
-      capturing != hipStreamCaptureStatusNone)
-    return fresh(bytes);
-  struct Kept { int device; void* stream; at::Tensor ws; };
-  thread_local std::vector<Kept>* kept = new std::vector<Kept>();
+  if (stream != nullptr) {                      // the default stream cannot be captured
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
+        capturing != hipStreamCaptureStatusNone)
+      return fresh(bytes);
+  }
+  thread_local KeptWorkspaces kept;
   const int device = like.device().index();
-  for (const Kept& k : *kept)
-    if (k.device == device && k.stream == stream) return k.ws;
-  kept->push_back(Kept{device, stream, fresh(kKept)});
-  return kept->back().ws;
+  for (auto& k : kept.slots)
+    if (k.device == device && k.stream == stream) {
+      k.used = ++kept.clock;
+      return k.ws;
+    }
+  if (kept.slots.size() < kKeptSlots) {
+    kept.slots.push_back(KeptWorkspaces::Kept{device, stream, fresh(kKept), ++kept.clock});
+    return kept.slots.back().ws;
+  }
+  auto* oldest = &kept.slots[0];
+  for (auto& k : kept.slots)
+    if (k.used < oldest->used) oldest = &k;
+  *oldest = KeptWorkspaces::Kept{device, stream, fresh(kKept), ++kept.clock};
+  return oldest->ws;
 }
 
 std::string shape_str(at::IntArrayRef s) {

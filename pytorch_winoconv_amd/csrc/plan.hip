@@ -9,6 +9,8 @@
 // separating the taps of each axis by parity first:
 //   y[o] = sum_k x[2o + k - pad] w[k] = sum_q sum_j x[2(o + j) + q - pad] w[2j + q].
 #include "wc_common.h"
+
+#include <cstdlib>
 #include "wc_tables.h"
 #include <atomic>
 #include <cstring>
@@ -55,9 +57,16 @@ int ensure_dynamic_lds(const void* fn, size_t bytes) {
   return WC_OK;
 }
 
-std::atomic<int> g_gemm_config{-1}, g_gemm_rows{1};
-int test_gemm_config() { return g_gemm_config.load(std::memory_order_relaxed); }
-int test_gemm_rows() { return g_gemm_rows.load(std::memory_order_relaxed); }
+// State of the test hook wc_test_gemm_override: per host thread, and writable only in a process whose environment
+// holds WINOCONV_TEST_HOOKS=1 when the hook is first called (the test suite sets it); elsewhere the hook refuses and
+// these stay at their defaults, so no caller can change what another caller's launches do.
+thread_local int t_gemm_config = -1, t_gemm_rows = 1;
+int test_gemm_config() { return t_gemm_config; }
+int test_gemm_rows() { return t_gemm_rows; }
+static bool test_hooks_enabled() {
+  static const bool on = [] { const char* e = std::getenv("WINOCONV_TEST_HOOKS"); return e && e[0] == '1'; }();
+  return on;
+}
 
 struct AxisPiece { int tap0, r; };
 
@@ -101,8 +110,10 @@ extern "C" {
 int wc_test_gemm_override(int config, int rows_mode) {
   WC_CHECK_ARG(config >= -1 && config < 16 && rows_mode >= 0 && rows_mode <= 2,
                "wc_test_gemm_override: config %d, rows_mode %d", config, rows_mode);
-  g_gemm_config.store(config, std::memory_order_relaxed);
-  g_gemm_rows.store(rows_mode, std::memory_order_relaxed);
+  if (!test_hooks_enabled())
+    return fail(WC_ERR_UNSUPPORTED, "wc_test_gemm_override: test hooks are off (set WINOCONV_TEST_HOOKS=1 before the first call)");
+  t_gemm_config = config;
+  t_gemm_rows = rows_mode;
   return WC_OK;
 }
 

@@ -124,6 +124,15 @@ def effective_tile(x_shape, w_shape, dtype, stride=1, padding=0, m=2, whole_kern
     return d.m, d.stacked
 
 
+def plan_form(x_shape, w_shape, dtype, stride=1, padding=0, m=2):
+    """(direct, stacked, tile) of the plan conv_forward runs for this problem with everything left to the library:
+    what a cached transformed filter depends on beside the filter itself (the library's choice between the
+    Winograd pieces and the direct form looks at the batch size)."""
+    pad = padding if isinstance(padding, int) else tuple(padding)
+    d = _forward_setup(tuple(x_shape), tuple(w_shape), dtype, stride, pad, m, 0, False, None)[0]
+    return int(d.direct), int(d.stacked), int(d.m)
+
+
 def plan_conv(desc):
     plan = Plan()
     check(_lib.load().wc_plan_conv(ctypes.byref(desc), ctypes.byref(plan)))

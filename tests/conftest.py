@@ -3,6 +3,9 @@ import sys
 
 import pytest
 
+# the library's test hook (wc_test_gemm_override) works only in a process that opts in before its first call
+os.environ.setdefault("WINOCONV_TEST_HOOKS", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -488,3 +488,20 @@ def test_one_tap_kernels_take_the_direct_form(dtype):
     assert engine.make_desc((4, 64, 28, 28), (100, 64, 1, 1), dtype, 1, 0, 2, stacked=None).direct == 0          # K no multiple of 8
     assert engine.make_desc((4, 48, 28, 28), (128, 48, 1, 1), dtype, 1, 0, 2, stacked=None).direct == (1 if dtype == torch.float32 else 0)
     assert engine.make_desc((4, 64, 28, 28), (128, 64, 1, 3), dtype, 1, (0, 1), 2, stacked=None).direct == 0     # three taps, stride 1
+
+
+def test_the_test_hook_is_inert_in_a_process_that_did_not_opt_in():
+    """wc_test_gemm_override changes what launches do, so it works only where WINOCONV_TEST_HOOKS=1 was in the
+    environment before its first call (this suite sets it in conftest.py); elsewhere it refuses."""
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from pytorch_winoconv_amd import _lib\n"
+            "lib = _lib.load()\n"
+            "rc = lib.wc_test_gemm_override(0, 1)\n"
+            "print(rc, lib.wc_last_error().decode())\n" % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    env = {k: v for k, v in os.environ.items() if k != "WINOCONV_TEST_HOOKS"}
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout
+    assert out.split()[0] == str(_lib.WC_ERR_UNSUPPORTED) and "WINOCONV_TEST_HOOKS" in out
+    lib = _lib.load()
+    assert lib.wc_test_gemm_override(-1, 1) == 0            # this process opted in

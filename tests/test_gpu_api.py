@@ -5,6 +5,7 @@ import torch
 import torch.nn.functional as F
 
 import pytorch_winoconv_amd as pkg
+from pytorch_winoconv_amd import engine
 from oracle import winograd as ow
 
 pytestmark = pytest.mark.gpu
@@ -186,6 +187,21 @@ def test_winoconv2d_module_routes_and_caches(dev, k, stride, pad):
     mod_s = pkg.WinoConv2d(3, 16, 7, 2, 3, dtype=torch.float16, device=dev)
     x3 = torch.randn(2, 3, 30, 30, device=dev).half()
     assert torch.equal(mod_s(x3), F.conv2d(x3, mod_s.weight, mod_s.bias, 2, 3)) and mod_s._cache is None
+
+
+def test_winoconv2d_module_follows_the_plan_form_when_the_batch_size_changes(dev):
+    """The library takes the direct form for this strided layer at N = 32 and a Winograd plan at N = 8; the
+    transformed filters of the two forms differ in size, so the module's cached one must follow the form."""
+    torch.manual_seed(0)
+    mod = pkg.WinoConv2d(128, 128, 7, 2, 3, bias=False, dtype=torch.float16, device=dev)
+    forms = set()
+    for n in (32, 8, 32):
+        x = torch.randn(n, 128, 112, 112, device=dev).half()
+        forms.add(engine.plan_form(x.shape, mod.weight.shape, x.dtype, 2, (3, 3), mod._tile_for(x.dtype)))
+        y = mod(x)
+        ref = F.conv2d(x[:2].double().cpu(), mod.weight.detach().double().cpu(), stride=2, padding=3)
+        assert _nerr(y[:2], ref) < 2e-2
+    assert len(forms) == 2
 
 
 def test_winoconv3d_module(dev):
