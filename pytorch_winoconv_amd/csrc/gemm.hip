@@ -340,7 +340,7 @@ static GemmConfig make_config() {
 constexpr int kRunExtra = 8;       // pieces per run are at most kRunExtra + 1
 
 template <typename T, int WM, int WN, int NWP, int NWK>
-__global__ __launch_bounds__(64 * NWP * NWK, (NWP * NWK == 4 ? 2 : 1)) void gemm_rows_kernel(GemmArgs g) {
+__global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2 : 1)) void gemm_rows_kernel(GemmArgs g) {
   using MF = Mfma<T>;
   constexpr int BK = 32;
   constexpr int NT = 64 * NWP * NWK;
@@ -575,9 +575,10 @@ static GemmConfig make_rows_config() {
 // Tile shapes: 0..4 four wavefronts, largest first; 5 (16-bit types) 128 x 256 with eight wavefronts.
 template <typename T> struct Configs;
 template <> struct Configs<half_t> {
-  static constexpr int n = 6;
+  static constexpr int n = 7;
   static GemmConfig get(int i) {
     switch (i) {
+      case 6: return make_config<half_t, 4, 4, 32>();   // 256 x 256, four wavefronts of 128 x 128
       case 0: return make_config<half_t, 4, 2, 32>();   // 256 x 128
       case 1: return make_config<half_t, 2, 2, 32>();   // 128 x 128
       case 2: return make_config<half_t, 4, 1, 32>();   // 256 x 64
@@ -776,6 +777,19 @@ int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, in
   WC_CHECK_ARG(C > 0 && C % cq == 0 && K > 0 && K % 8 == 0, "gemm_direct_conv: C %d (multiple of %d), K %d (multiple of 8)", C, cq, K);
   const long long P = (long long)N * oH * oW;
   WC_CHECK_ARG(P > 0 && P < (1ll << 31) && (long long)kh * kw * C < (1ll << 24), "gemm_direct_conv: problem too large");
+  // Kernel rows of four and more taps over enough output to give a quarter of the CUs a 256 x 128 tile: one operand
+  // tile per kernel row (direct_rows.hip).  Measured against the tile per tap, fp16, stride 2, ms: N=32, 128 channels,
+  // 112x112: 4x4 0.091 | 0.102, 5x5 0.116 | 0.151, 7x7 0.181 | 0.264, 8x8 0.222 | 0.340; N=8: 7x7 0.081 | 0.122;
+  // 256 channels on 56x56: 7x7 0.166 | 0.249; 256 -> 512 on 28x28, N=64: 5x5 0.100 | 0.137; stride 1, 128 channels
+  // on 56x56: 5x5 0.103 | 0.135.  wc_test_gemm_override(., 2) takes it wherever it fits, (., 0) never.
+  if (direct_rows_fits(N, C, K, kw, stride, oH, oW, dtype)) {
+    const int mode = test_gemm_rows();
+    const long long tiles = ceil_div_ll(P, 256) * ceil_div(K, 128);
+    const bool k_fills = K % 128 == 0 || K % 128 >= 96;      // the last 128-channel tile is at least three quarters full
+    if (mode == 2 || (mode != 0 && tiles >= 64 && k_fills))
+      return direct_rows_conv(x, U, bias, y, N, H, W, C, K, kh, kw, stride, pad_h, pad_w, oH, oW, dtype, stream, o_step, o_y0,
+                              o_x0, o_H, o_W);
+  }
   GemmConfig c = dispatch_dtype(dtype, [&](auto t) { return choose_direct<decltype(t)>((int)P, K); });
   GemmArgs g;
   g.V = x; g.U = U; g.M = y; g.bias = bias;

@@ -362,11 +362,13 @@ static int auto_stacked(const wc_conv_desc* d) {
 //    224x224: 382 | 372; 128 -> 64 at 112x112: 209 | 201).
 //  * A long reduction needs enough output (pixels x channels >= 4 M, i.e. 256 tiles of 128 x 128) to keep the chip
 //    busy, else the latency of its k-steps decides: 3x3 at C=K=512 on 14x14 images 90 | 66, 7x7 at C=K=256 on 28x28
-//    240 | 139.  With that: against the plan that shares one transformed input (7 and 8 taps) 7x7 wins
-//    (C=K=128, 112x112: 246 | 267; 96 channels 184 | 206) and 8x8 loses (321 | 277); against stacked F(2,r) pieces it
-//    always wins (6x6 187 | 279, 5x5 at 256 channels 242 | 303, 9x9 399 | 845); against stacked F(4,r) pieces it wins
-//    at 4x4 (256 channels, 56x56: 87 | 96) and from 9x9 on (399 | 565) and loses or ties between (5x5 at 256 channels
-//    242 | 190, 6x6 at 128 187 | 179).
+//    240 | 139.  With that, and with one operand tile per kernel row for rows of 4 to 8 taps (direct_rows.hip): against
+//    the plan that shares one transformed input (7 and 8 taps) it wins (C=K=128, 112x112: 7x7 181 | 270, 8x8 234 | 284;
+//    96 channels 7x7 146 | 214, 8x8 182 | 224; 256 -> 512 on 28x28 7x7 173 | 228, 8x8 230 | 277); against stacked
+//    F(2,r) pieces it wins (128 channels, 112x112: 6x6 168 | 281, 9x9 421 | 845; 256 -> 512 on 28x28 5x5 111 | 115);
+//    against stacked F(4,r) pieces it wins at 4x4 (128 channels: 91 | 143; 256 -> 512: 77 | 83), from 9x9 on
+//    (414 | 554) and between while the reduction stays short of 4800 (6x6 at 128 channels 152 | 182, at 96 118 | 141),
+//    and loses beyond (256 -> 512 on 28x28: 5x5 101 | 98, 6x6 143 | 99).
 //  * A kernel of one tap at either stride, every type: the tile F(m,1) has nothing to save and its transforms are
 //    copies (fp16 N=64, 64 -> 256 channels, 56x56: three kernels 78 us).
 static bool direct_preferred(const wc_conv_desc* d) {
@@ -377,16 +379,16 @@ static bool direct_preferred(const wc_conv_desc* d) {
   // for 3x3 kernels over at most 128 channels only (N=64, 128 channels, 56x56: 163 | 220 | 170; N=16, 64 channels,
   // 112x112: 55 | 77 | 65; 32 -> 64 at 112x112: 49 | 86 | 75; 256 channels on 28x28: 187 | 173 | 176; 5x5 at 128: 798 | 708 | 426)
   if (d->dtype == WC_F32) return taps <= 9 && d->C <= 128;
-  if (d->K <= 64 && taps > 25) return false;
+  if (d->K <= 64 && taps > 25 && taps < 81) return false;      // (9x9, 64 channels, 112x112: 180 | 482 | 286)
   if ((long long)taps * d->C <= 3200) return true;
   wc_conv_desc e = *d;
   e.direct = 0; e.stacked = 0; e.m = 2; e.whole_kernel = 0;
   int out[3], grid[3];
   if (wc_conv_out_dims(&e, out, grid) != WC_OK) return false;
   if ((long long)d->N * out[1] * out[2] * d->K < (4ll << 20)) return false;
-  if (auto_stacked(d) == 2) return taps <= 49;
+  if (auto_stacked(d) == 2) return taps <= 64;
   if (d->m == 2) return true;
-  return taps <= 16 || taps >= 81;
+  return taps <= 16 || taps >= 81 || (long long)taps * d->C <= 4800;
 }
 
 int wc_conv_auto(wc_conv_desc* d) {

@@ -137,6 +137,15 @@ int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, in
                      int kh, int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream,
                      int o_step = 0, int o_y0 = 0, int o_x0 = 0, int o_H = 0, int o_W = 0);
 
+// The direct form with one operand tile per kernel row (direct_rows.hip; 16-bit types, kernel rows of 4 to 8 taps, stride
+// 1 or 2): whether a problem is in its range (the input rows that 256 consecutive output pixels read, with their
+// padding, must fit a stage of kDirectRowsPixels pixels), and the launch, with the arguments of gemm_direct_conv.
+constexpr int kDirectRowsPixels = 768;
+bool direct_rows_fits(int N, int C, int K, int kw, int stride, int oH, int oW, int dtype);
+int direct_rows_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K, int kh,
+                     int kw, int stride, int pad_h, int pad_w, int oH, int oW, int dtype, void* stream, int o_step,
+                     int o_y0, int o_x0, int o_H, int o_W);
+
 // Number of XCDs (L2 domains) a launch is spread over round-robin by workgroup id.
 constexpr int kXcds = 8;
 constexpr int kCus = 256;                  // compute units of an MI355X

@@ -461,11 +461,13 @@ def test_module_tables_equal_oracle_tables():
     (32, 64, 64, 224, 7, 2, 0), (2, 32, 8, 28, 7, 2, 0), (32, 128, 64, 112, 7, 4, 0),
     # long reductions need pixels x channels >= 4 M
     (64, 512, 512, 14, 3, 4, 0), (128, 512, 512, 14, 3, 2, 0), (64, 256, 256, 28, 7, 2, 0), (2, 128, 128, 28, 7, 2, 0),
-    # ... then: against the shared-input plan 7x7 yes, 8x8 no
-    (32, 128, 128, 112, 7, 2, 1), (32, 128, 128, 112, 7, 4, 1), (32, 96, 96, 112, 7, 4, 1), (32, 128, 128, 112, 8, 4, 0),
-    # against stacked F(2,r) pieces always; against stacked F(4,r) pieces at 4x4 and from 9x9 on
-    (32, 128, 128, 112, 6, 2, 1), (32, 128, 128, 112, 6, 4, 0), (64, 256, 256, 56, 5, 2, 1), (64, 256, 256, 56, 5, 4, 0),
-    (32, 256, 256, 56, 4, 4, 1), (32, 128, 128, 112, 9, 4, 1), (32, 128, 128, 112, 9, 2, 1)])
+    # ... then: against the shared-input plan (7x7 and 8x8) yes
+    (32, 128, 128, 112, 7, 2, 1), (32, 128, 128, 112, 7, 4, 1), (32, 96, 96, 112, 7, 4, 1), (32, 128, 128, 112, 8, 4, 1),
+    # against stacked F(2,r) pieces always; against stacked F(4,r) pieces at 4x4, from 9x9 on, and between for
+    # reductions of at most 4800
+    (32, 128, 128, 112, 6, 2, 1), (32, 128, 128, 112, 6, 4, 1), (64, 256, 256, 56, 5, 2, 1), (64, 256, 256, 56, 5, 4, 0),
+    (64, 256, 512, 28, 6, 4, 0), (32, 256, 256, 56, 4, 4, 1), (32, 128, 128, 112, 9, 4, 1), (32, 128, 128, 112, 9, 2, 1),
+    (32, 64, 64, 112, 9, 2, 1)])
 def test_the_library_chooses_the_direct_form_where_it_measured_faster(N, C, K, H, k, m, chosen):
     """Each stride-2 layer of the sweep behind the rule, on the side of the crossover it measured on."""
     d = engine.make_desc((N, C, H, H), (K, C, k, k), torch.float16, 2, k // 2, m, stacked=None)

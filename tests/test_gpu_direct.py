@@ -117,3 +117,68 @@ def test_c4_stride_2_layers_at_full_size(dev):
             y = engine.conv_forward(xd, w.to(dev), None, 2, pad, 2, direct=direct)
             assert _rel(y[31:], ref) <= tol
             assert torch.equal(engine.conv_forward(xp, w.to(dev), None, 2, pad, 2, direct=direct), y[perm])
+
+
+ROWS_CASES = [
+    # x shape, w shape, stride, pad: kernel rows of 4 to 8 taps, which the kernel with one operand tile per kernel row takes
+    ((2, 32, 15, 14), (8, 32, 7, 7), 2, 3), ((1, 96, 17, 19), (40, 96, 5, 5), 2, 2), ((2, 32, 10, 11), (8, 32, 4, 6), 2, (1, 2)),
+    ((3, 64, 30, 30), (136, 64, 7, 7), 2, 3),          # two channel tiles, the second 8 wide; 675 pixels: three pixel tiles
+    ((1, 32, 40, 61), (16, 32, 3, 8), 2, (1, 3)),      # rows of 8 taps, odd width
+    ((2, 64, 12, 12), (16, 64, 5, 5), 1, 2), ((1, 32, 9, 23), (8, 32, 2, 4), 1, (0, 2)), ((1, 32, 14, 14), (8, 32, 7, 7), 2, 3),
+    ((2, 32, 20, 20), (24, 32, 6, 6), 2, 0), ((1, 32, 6, 120), (8, 32, 1, 5), 1, (0, 2)),     # 120 output pixels per row: few, long slots
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", ROWS_CASES)
+def test_one_operand_tile_per_kernel_row_is_exact_on_small_integers(dev, dtype, case, gemm_override):
+    """direct_rows_kernel, forced through the test hook on shapes far below the size at which the library takes it by
+    itself: bit-equal to direct convolution on small integers (bias included), to the oracle, and to the kernel with
+    one operand tile per tap."""
+    xs, ws, stride, pad = case
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = torch.randint(-2, 3, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    ref = F.conv2d(x, w, b, stride=stride, padding=pad)
+    assert float(ref.abs().max()) < {torch.float16: 2048, torch.bfloat16: 256}[dtype] * 8
+    xd, wd, bd = x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev)
+    gemm_override(-1, 2)
+    y = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=True)
+    gemm_override(-1, 0)
+    y_tap = engine.conv_forward(xd, wd, bd, stride, pad, 2, direct=True)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert torch.equal(y.cpu(), ref.float().to(dtype))
+    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, stride, pad, DISC[dtype]))
+    assert torch.equal(y, y_tap)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", ROWS_CASES)
+def test_one_operand_tile_per_kernel_row_against_fp64_and_the_oracle(dev, dtype, case, gemm_override):
+    xs, ws, stride, pad = case
+    g = torch.Generator().manual_seed(6)
+    fan = ws[1] * ws[2] * ws[3]
+    x = torch.randn(*xs, generator=g).to(dtype)
+    w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), None, stride=stride, padding=pad)
+    gemm_override(-1, 2)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, stride, pad, 2, direct=True)
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.2e-2}[dtype]
+    assert _rel(y, ref) <= tol
+    assert _rel(y, ow.direct_conv(x, w, None, stride, pad, DISC[dtype])) <= tol
+
+
+def test_strided_input_gradient_through_the_kernel_row_tiles(dev, gemm_override):
+    """The input gradient of a 7x7 stride-2 layer is four stride-1 direct convolutions of dy, two of them with kernel
+    rows of four taps, each writing every second pixel of dx: with the kernel-row tiles forced, on small integers,
+    bit-equal to the gradient autograd gives in fp64."""
+    g = torch.Generator().manual_seed(7)
+    x = torch.zeros(2, 40, 18, 20, dtype=torch.double, requires_grad=True)
+    w = torch.randint(-2, 3, (32, 40, 7, 7), generator=g).double()
+    dy = torch.randint(-2, 3, (2, 32, 9, 10), generator=g).double()
+    F.conv2d(x, w, None, stride=2, padding=3).backward(dy)
+    gemm_override(-1, 2)
+    dx = engine.conv_backward_input(dy.half().to(dev), w.half().to(dev), (18, 20), 2, 3, 2)
+    assert float(x.grad.abs().max()) < 2048
+    assert torch.equal(dx.cpu().double(), x.grad)
