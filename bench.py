@@ -127,6 +127,7 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 7x7 s2 DWM F(4,r) stacked", (32, 128, 112, 112), (128, 128, 7, 7), 2, 3, 4, "f16-stacked-nodirect"),
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
+    ("first layer fp16 N32 3->64 224x224 7x7 s2 (the direct form's first-layer kernel)", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 4, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)xF(4,3)^2", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, "f16"),
     ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 shared input F(2,2)^3", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16"),
@@ -141,7 +142,7 @@ VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256
 # the default form of every benchmark configuration (c1..c5): what a plain `python bench.py` adds to its JSON line
 DEFAULTS = ("c1 ", "c2 vgg16 fp32 N8 F(4,3)", "c2 vgg16 fp32 N8 F(2,3)", "c3 fp16 N64 C64 56x56 F(2,3)", "c3 fp16 N64 C128 28x28 F(2,3)",
             "c3 fp16 N64 C64 56x56 F(4,3)", "c3 fp16 N64 C128 28x28 F(4,3)", "c3 fp16 N64 C256", "c3 fp16 N64 C512", "5x5 s1 DWM shared input F(3,3)", "7x7 s1 DWM shared input F(3,3)",
-            "3x3 s2 direct form", "7x7 s2 direct form", "c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3")
+            "3x3 s2 direct form", "7x7 s2 direct form", "first layer fp16", "c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3")
 
 
 def run_suite(steps=10, only=None, defaults=False):

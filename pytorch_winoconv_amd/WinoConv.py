@@ -91,8 +91,14 @@ class _WinoConvNd(nn.Module):
         # first layers with at most 8 input channels, whose parity-phase plans pad the channels to 32 once per
         # phase (ResNet's 3 -> 64, 7 x 7, stride 2 at N = 32: 0.25 ms in fp16 and 1.0 ms in fp32 against 0.07 and
         # 0.12 ms for torch's own convolution); they go the reference's way.
+        # ... except where the engine has a kernel for them: at most 4 channels in a 16-bit type, kernels of 3, 5 or 7
+        # rows and at most 8 columns (the direct form's first-layer kernel: ResNet's layer in fp16).
         if self.stride[0] == 2 and self.in_channels <= 8:
-            return False
+            first = (self.nd == 2 and self.in_channels <= 4 and x.dtype in (torch.float16, torch.bfloat16)
+                     and self.kernel_size[0] in (3, 5, 7) and self.kernel_size[1] <= 8 and self.out_channels % 8 == 0
+                     and len(set(self.stride)) == 1 and self.groups == 1 and set(self.dilation) == {1})
+            if not first:
+                return False
         # ... and so do 3-D first layers with at most 4 input channels, for which there is no fused kernel like the
         # 2-D one: F(2,3)^3 on 3 channels padded to 32 makes V eighty times the input (N=2, 3 -> 64, 16x112x112:
         # 0.27 ms in fp16 and 0.52 ms in fp32 against 0.12 and 0.11 ms)

@@ -78,7 +78,8 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   L->direct = d_in->direct == 1;
   if (L->direct) {
     if (!direct_conv_fits(d_in))
-      return fail(WC_ERR_UNSUPPORTED, "direct form: 2-D, input channels a multiple of 32 (fp32: 16), output channels a multiple of 8");
+      return fail(WC_ERR_UNSUPPORTED, "direct form: 2-D, input channels a multiple of 32 (fp32: 16; or at most 4 at stride 2 in a 16-bit type), "
+                  "output channels a multiple of 8");
     plain.direct = 0; plain.stacked = 0; plain.m = 2; plain.whole_kernel = 0; plain.unfused = 1;
   }
   const wc_conv_desc* d = &plain;
@@ -110,14 +111,15 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   const long long Pc = L->tiles_per_image * chunk;
   if (T * Pc * (long long)(L->Cp > L->ldm ? L->Cp : L->ldm) >= (1ll << 40))
     return fail(WC_ERR_UNSUPPORTED, "chunk of %d images is too large", chunk);
-  L->u_bytes = L->direct ? round256((size_t)d->K * d->kernel[1] * d->kernel[2] * d->C * L->es)
+  L->u_bytes = L->direct ? round256(direct_u_elems(d) * L->es)
                          : round256((size_t)T * d->K * L->Cp * L->es);
   L->v_bytes = round256((size_t)T * (Pc + (L->shared ? L->shift.tail : 0)) * L->vrow * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
   L->thin = !L->direct && !d->unfused && thin_conv_fits(d, &L->plan);
   // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
   // through a channel-last copy of one chunk (the one-kernel path: of the whole batch)
-  L->x_direct = d->x_layout == 1 && !L->thin && !L->direct && input_transform_nchw_fits(d, &L->plan);
+  L->x_direct = d->x_layout == 1 && ((!L->thin && !L->direct && input_transform_nchw_fits(d, &L->plan)) ||
+                                     (L->direct && direct_first_fits(d_in)));      // ... and so does the first-layer kernel
   const size_t images = L->thin || L->direct ? d->N : chunk;
   const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L->es;
   const size_t y_image = (size_t)L->out[0] * L->out[1] * L->out[2] * d->K * L->es;
@@ -184,7 +186,7 @@ int wc_conv_u_elems(const wc_conv_desc* d, size_t* elems) {
   Layout L;
   int rc = make_layout(d, &L);
   if (rc) return rc;
-  *elems = L.direct ? (size_t)d->K * d->kernel[1] * d->kernel[2] * d->C : (size_t)L.plan.t_total * d->K * L.Cp;
+  *elems = L.direct ? direct_u_elems(d) : (size_t)L.plan.t_total * d->K * L.Cp;
   return WC_OK;
 }
 

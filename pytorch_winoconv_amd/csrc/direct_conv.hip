@@ -40,6 +40,7 @@ __global__ __launch_bounds__(256) void direct_filter_kernel(DirectFilterArgs a) 
 
 bool direct_conv_fits(const wc_conv_desc* d) {
   if (d->ndim != 2) return false;
+  if (direct_first_fits(d)) return true;          // strided first layers: their own kernel and filter layout (direct_first.hip)
   if (d->C % (d->dtype == WC_F32 ? 16 : 32) != 0 || d->K % 8 != 0) return false;   // whole reduction blocks along C, 16-byte stores along K
   if (d->whole_kernel) return false;
   int out[3], grid[3];
@@ -50,8 +51,13 @@ bool direct_conv_fits(const wc_conv_desc* d) {
   return P < (1ll << 31) && (long long)d->N * d->in[1] * d->in[2] < (1ll << 31);
 }
 
+size_t direct_u_elems(const wc_conv_desc* d) {
+  return direct_first_fits(d) ? direct_first_u_elems(d) : (size_t)d->K * d->kernel[1] * d->kernel[2] * d->C;
+}
+
 int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream) {
   WC_CHECK_ARG(w && w_strides && U, "direct filter copy: null pointer");
+  if (direct_first_fits(d)) return direct_first_filter(d, w, w_strides, U, stream);
   DirectFilterArgs a;
   a.w = w; a.U = U;
   for (int i = 0; i < 5; ++i) a.s[i] = w_strides[i];
@@ -73,6 +79,7 @@ int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* 
   e.direct = 0; e.stacked = 0; e.m = 2;
   int rc = wc_conv_out_dims(&e, out, grid);
   if (rc) return rc;
+  if (direct_first_fits(d)) return direct_first_conv(d, x, n_images, U, bias, y, out[1], out[2], stream);
   return gemm_direct_conv(x, U, bias, y, n_images, d->in[1], d->in[2], d->C, d->K, d->kernel[1], d->kernel[2], d->stride,
                           d->pad[1], d->pad[2], out[1], out[2], d->dtype, stream);
 }

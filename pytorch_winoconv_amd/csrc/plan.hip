@@ -379,6 +379,9 @@ static bool direct_preferred(const wc_conv_desc* d) {
   // for 3x3 kernels over at most 128 channels only (N=64, 128 channels, 56x56: 163 | 220 | 170; N=16, 64 channels,
   // 112x112: 55 | 77 | 65; 32 -> 64 at 112x112: 49 | 86 | 75; 256 channels on 28x28: 187 | 173 | 176; 5x5 at 128: 798 | 708 | 426)
   if (d->dtype == WC_F32) return taps <= 9 && d->C <= 128;
+  // strided first layers have a kernel of their own (direct_first.hip; N=32, 3 -> 64, 7x7 on 224x224: the parity-phase
+  // plans pad the 3 channels to 32 per phase)
+  if (direct_first_fits(d)) return true;
   if (d->K <= 64 && taps > 25 && taps < 81) return false;      // (9x9, 64 channels, 112x112: 180 | 482 | 286)
   if ((long long)taps * d->C <= 3200) return true;
   wc_conv_desc e = *d;

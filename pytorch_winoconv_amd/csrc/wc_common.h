@@ -131,6 +131,14 @@ int transpose_images(const void* src, void* dst, long long n, long long R, long 
 bool direct_conv_fits(const wc_conv_desc* d);
 int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
 int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y, void* stream);
+size_t direct_u_elems(const wc_conv_desc* d);     // elements of the direct form's U
+// Strided first layers (direct_first.hip): at most 4 input channels, stride 2, kernels of 3, 5 or 7 rows and at most 8
+// columns, 16-bit types.  U is (K, kh, 8 taps, 4 channels), zero where the filter has no tap or channel.
+bool direct_first_fits(const wc_conv_desc* d);
+size_t direct_first_u_elems(const wc_conv_desc* d);
+int direct_first_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
+int direct_first_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y,
+                      int oH, int oW, void* stream);
 // o_step > 0: row (b, oy, ox) of the result goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of image b of an
 // (o_H, o_W) tensor instead of to row b oH oW + oy oW + ox
 int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,

@@ -329,7 +329,14 @@ def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, s
     _require_gpu(w)
     desc = make_desc(x_shape, w.shape, w.dtype, stride, padding, m, 0, whole_kernel, stacked, direct=direct)
     if desc.direct:
-        U = torch.empty(desc.K, desc.kernel[1], desc.kernel[2], desc.C, dtype=w.dtype, device=w.device)
+        # the filter with its taps outermost and channels innermost, (K, kH, kW, C); strided first layers (at most 4
+        # channels) pad every kernel row to 8 taps of 4 channels, (K, kH, 8, 4)
+        n = ctypes.c_size_t()
+        check(_lib.load().wc_conv_u_elems(ctypes.byref(desc), ctypes.byref(n)))
+        shape = (desc.K, desc.kernel[1], desc.kernel[2], desc.C)
+        if n.value != shape[0] * shape[1] * shape[2] * shape[3]:
+            shape = (desc.K, desc.kernel[1], 8, 4)
+        U = torch.empty(shape, dtype=w.dtype, device=w.device)
         plan = Plan()
         check(_lib.load().wc_filter_transform(ctypes.byref(desc), ctypes.byref(plan), _ptr(w), _w_strides(w), _ptr(U), _stream(w)))
         return U

@@ -183,10 +183,14 @@ def test_winoconv2d_module_routes_and_caches(dev, k, stride, pad):
     mod_d = pkg.WinoConv2d(16, 24, 3, 1, 2, dilation=2, dtype=torch.float16, device=dev)
     yd = mod_d(x)
     assert yd.shape == (2, 24, 20, 20)
-    # so does a strided first layer with at most 8 input channels (the reference sends every strided layer there)
-    mod_s = pkg.WinoConv2d(3, 16, 7, 2, 3, dtype=torch.float16, device=dev)
-    x3 = torch.randn(2, 3, 30, 30, device=dev).half()
-    assert torch.equal(mod_s(x3), F.conv2d(x3, mod_s.weight, mod_s.bias, 2, 3)) and mod_s._cache is None
+    # so does a strided first layer with 5 to 8 input channels, or in fp32 (the reference sends every strided layer
+    # there); with at most 4 channels in a 16-bit type the engine has a kernel of its own (test_gpu_direct.py)
+    mod_s = pkg.WinoConv2d(6, 16, 7, 2, 3, dtype=torch.float16, device=dev)
+    x6 = torch.randn(2, 6, 30, 30, device=dev).half()
+    assert torch.equal(mod_s(x6), F.conv2d(x6, mod_s.weight, mod_s.bias, 2, 3)) and mod_s._cache is None
+    mod_f = pkg.WinoConv2d(3, 16, 7, 2, 3, device=dev)
+    x3 = torch.randn(2, 3, 30, 30, device=dev)
+    assert torch.equal(mod_f(x3), F.conv2d(x3, mod_f.weight, mod_f.bias, 2, 3)) and mod_f._cache is None
 
 
 def test_winoconv2d_module_follows_the_plan_form_when_the_batch_size_changes(dev):

@@ -182,3 +182,73 @@ def test_strided_input_gradient_through_the_kernel_row_tiles(dev, gemm_override)
     dx = engine.conv_backward_input(dy.half().to(dev), w.half().to(dev), (18, 20), 2, 3, 2)
     assert float(x.grad.abs().max()) < 2048
     assert torch.equal(dx.cpu().double(), x.grad)
+
+
+FIRST_CASES = [
+    # x shape, w shape, pad: strided first layers (at most 4 channels, stride 2, 3 / 5 / 7 kernel rows, at most 8 columns)
+    ((2, 3, 32, 32), (64, 3, 7, 7), 3), ((1, 3, 45, 51), (16, 3, 7, 7), 3), ((3, 1, 20, 33), (8, 1, 3, 3), 1),
+    ((2, 4, 37, 18), (72, 4, 5, 8), (2, 3)), ((2, 2, 16, 16), (136, 2, 3, 5), (0, 2)), ((5, 3, 64, 64), (64, 3, 7, 7), 3),
+    ((1, 3, 7, 9), (8, 3, 7, 7), 3), ((2, 3, 33, 34), (24, 3, 5, 5), 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", FIRST_CASES)
+def test_strided_first_layers_are_exact_on_small_integers(dev, dtype, case, host_layer):
+    """first_strided_kernel (csrc/direct_first.hip), the library's own choice for these layers: bit-equal to direct
+    convolution on small integers, bias included, to the oracle, from channel-last and from channel-first memory."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(8)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = torch.randint(-2, 3, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    ref = F.conv2d(x, w, b, stride=2, padding=pad)
+    assert float(ref.abs().max()) < {torch.float16: 2048, torch.bfloat16: 256}[dtype]
+    assert engine.make_desc(xs, ws, dtype, 2, pad, 4, stacked=None).direct == 1
+    xd, wd, bd = x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev)
+    y = engine.conv_forward(xd, wd, bd, 2, pad, 4)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert torch.equal(y.cpu(), ref.float().to(dtype))
+    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, 2, pad, DISC[dtype]))
+    ycl = engine.conv_forward(xd.contiguous(memory_format=torch.channels_last), wd, bd, 2, pad, 4)
+    assert torch.equal(ycl, y)
+    U = engine.transform_filter(wd, xs, 2, pad, 4)
+    assert tuple(U.shape) == (ws[0], ws[2], 8, 4)
+    assert torch.equal(U[:, :, :ws[3], :ws[1]], wd.permute(0, 2, 3, 1)) and float(U[:, :, ws[3]:].abs().sum()) == 0
+    assert torch.equal(engine.conv_forward(xd, wd, bd, 2, pad, 4, U=U), y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_resnet_first_layer_against_fp64_and_through_the_module(dev, dtype):
+    """N=8, 3 -> 64, 7x7, stride 2, 224x224: against fp64 convolution and the oracle on normal data; WinoConv2d keeps the
+    layer in the engine in 16-bit types and hands it to torch in fp32."""
+    import pytorch_winoconv_amd as pkg
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(8, 3, 224, 224, generator=g).to(dtype)
+    w = (torch.randn(64, 3, 7, 7, generator=g) * (2.0 / 147) ** 0.5).to(dtype)
+    ref = F.conv2d(x.double(), w.double(), None, stride=2, padding=3)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, 2, 3, 4)
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.2e-2}[dtype]
+    assert _rel(y, ref) <= tol
+    assert _rel(y[:1], ow.direct_conv(x[:1], w, None, 2, 3, DISC[dtype])) <= tol
+    mod = pkg.WinoConv2d(3, 64, 7, 2, 3, bias=False, dtype=dtype, device=dev)
+    with torch.no_grad():
+        mod.weight.copy_(w.to(dev))
+    assert torch.equal(mod(x.to(dev)), y) and mod._cache is not None
+    mod32 = pkg.WinoConv2d(3, 64, 7, 2, 3, bias=False, device=dev)
+    assert mod32(x.float().to(dev)).dtype == torch.float32 and mod32._cache is None
+
+
+def test_first_layer_module_trains(dev):
+    """Gradients of a strided first layer through the module: the weight gradient against fp64 autograd."""
+    import pytorch_winoconv_amd as pkg
+    torch.manual_seed(10)
+    mod = pkg.WinoConv2d(3, 16, 7, 2, 3, dtype=torch.float16, device=dev)
+    x = torch.randn(4, 3, 40, 40, device=dev).half()
+    y = mod(x)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    w64 = mod.weight.detach().double().cpu().requires_grad_(True)
+    b64 = mod.bias.detach().double().cpu().requires_grad_(True)
+    F.conv2d(x.double().cpu(), w64, b64, stride=2, padding=3).backward(dy.double().cpu())
+    assert _rel(mod.weight.grad, w64.grad) <= 2e-2 and _rel(mod.bias.grad, b64.grad) <= 2e-2
