@@ -360,6 +360,60 @@ def run_layouts(steps=50):
     return out
 
 
+def run_chunk_residency(iters=40):
+    """The three kernels of the metric layer on chunks of its batch, with V and M in the same buffers every iteration
+    (a chunk's V and M then sit in the 256 MB last-level cache when the next kernel reads them) and with V and M rotated
+    over more than 700 MB of buffers (served by HBM): us per chunk and per 64 images.  x and y always rotate over three
+    batches.  What a forward pass blocked per image chunk could gain from cache residency."""
+    import torch
+    from pytorch_winoconv_amd import _lib, engine
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    xs = [torch.randn(N, H, W, C, generator=g).half().to(dev) for _ in range(3)]
+    ys = [torch.empty(N, H, W, K, dtype=torch.float16, device=dev) for _ in range(3)]
+    w = (torch.randn(K, C, R, R, generator=g) * (2.0 / (C * R * R)) ** 0.5).half().to(dev)
+    out = []
+    for nc in (64, 16, 8, 4):
+        desc = engine.make_desc((nc, C, H, W), w.shape, torch.float16, 1, PAD, M_TILE)
+        plan = engine.plan_conv(desc)
+        U = engine.filter_transform(desc, plan, w)
+        _, grid = engine.out_dims(desc)
+        P, T = nc * grid[1] * grid[2], plan.t_total
+        Cp, ldm = lib.wc_padded_channels(C), lib.wc_padded_channels8(K)
+        st = engine._stream(xs[0])
+        for mode in ("hot", "cold"):
+            nset = 1 if mode == "hot" else max(2, int(700e6 // (2 * T * P * Cp * 2)) + 1)
+            Vs = [torch.empty(T, P, Cp, dtype=torch.float16, device=dev) for _ in range(nset)]
+            Ms = [torch.empty(T, P, ldm, dtype=torch.float16, device=dev) for _ in range(nset)]
+            ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(iters)]
+
+            def one(i, e=None):
+                V, Mb = Vs[i % nset], Ms[i % nset]
+                b0 = (i * nc) % N
+                xi, yi = xs[i % 3][b0:b0 + nc], ys[i % 3][b0:b0 + nc]
+                if e: e[0].record()
+                _lib.check(lib.wc_input_transform(ctypes.byref(desc), ctypes.byref(plan), engine._ptr(xi), nc, engine._ptr(V), st))
+                if e: e[1].record()
+                _lib.check(lib.wc_batched_gemm(engine._ptr(V), engine._ptr(U), engine._ptr(Mb), T, P, Cp, K, ldm, desc.dtype, st))
+                if e: e[2].record()
+                _lib.check(lib.wc_output_transform(ctypes.byref(desc), ctypes.byref(plan), engine._ptr(Mb), None, nc, engine._ptr(yi), st))
+                if e: e[3].record()
+            t0, i = time.perf_counter(), 0
+            while time.perf_counter() - t0 < 0.3:
+                one(i); i += 1
+            torch.cuda.synchronize()
+            for j in range(iters):
+                one(i + j, ev[j])
+            torch.cuda.synchronize()
+            us = [sum(e[k].elapsed_time(e[k + 1]) for e in ev) / iters * 1e3 for k in range(3)]
+            out.append({"chunk_images": nc, "V_M": mode, "buffer_sets": nset,
+                        "us_per_chunk": {"input_transform": round(us[0], 1), "batched_gemm": round(us[1], 1), "output_transform": round(us[2], 1)},
+                        "us_per_64_images": round(sum(us) * N / nc, 1)})
+            del Vs, Ms
+    return out
+
+
 def run_split_concat(steps=20):
     """Tile split / concat (bit-exact copies) at the metric layer's shape: us per call and HBM GB/s
     of the algorithmic bytes (input once + tiles once; tiles once + output once)."""
@@ -424,6 +478,9 @@ def main():
                     help="also time the host side of a small layer (c1) through the compiled host layer and through ctypes")
     ap.add_argument("--layouts", action="store_true",
                     help="also time small and large layers with channel-last and channel-first tensors")
+    ap.add_argument("--chunk-residency", action="store_true",
+                    help="also time the three kernels of the metric layer on chunks of 64 / 16 / 8 / 4 images with V and M "
+                         "kept in one set of buffers (last-level cache resident) and rotated over 700 MB (from HBM)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 128 MiB device-to-device copies before the timed region "
                          "(the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -613,6 +670,8 @@ def main():
         result["split_concat"] = run_split_concat()
     if args.layouts:
         result["layouts_ms"] = run_layouts()
+    if args.chunk_residency:
+        result["chunk_residency"] = run_chunk_residency()
     if args.host_overhead:
         result["host_overhead_c1"] = run_host_overhead()
     if not args.no_cpu:
