@@ -137,7 +137,9 @@ const char* wc_last_error(void);
 /* Test hook, no counterpart in the reference: forces tile shape `config` (an index into the
  * library's list of shapes; -1 = choose by problem size) on wc_batched_gemm, and for plans that
  * share one transformed input the kernel with one operand tile per piece (rows_mode 0), the
- * choice by size (1, the default) or one tile per run of pieces wherever the plan has runs (2).
+ * choice by size (1, the default), one tile per run of pieces wherever the plan has runs (2), or
+ * the persistent kernel with one tile per run fed by LDS-DMA wherever it runs (3: runs of 2 to 5
+ * pieces, else as 1).
  * config 8 / 9: the one-kernel F(2x2,3x3) path with workgroups of 64 / 32 output channels whatever
  * the number of tiles (9 only where the channel count allows it).
  * Works only in a process started with WINOCONV_TEST_HOOKS=1 in its environment (WC_ERR_UNSUPPORTED

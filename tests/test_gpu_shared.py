@@ -125,6 +125,45 @@ def test_one_operand_tile_per_run_is_exact_on_small_integers(dev, case, gemm_ove
     test_exact_on_small_integers(dev, case)
 
 
+@pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
+def test_dma_fed_tile_per_run_is_exact_on_small_integers(dev, case, gemm_override):
+    """The 512 x 128 tile fed by LDS-DMA (runs of two to five pieces, 16-bit types; chosen by size, here forced so
+    that partial tiles in both directions, 3-D plane jumps and tiles that end inside V's tail reach it)."""
+    gemm_override(rows_mode=3)
+    test_exact_on_small_integers(dev, case)
+
+
+DMA_CASES = [
+    # x shape, w shape, pad, tile: more than one 512-row tile, 128-channel blocks that end early, every run length
+    ((2, 64, 40, 36), (136, 64, 7, 7), 3, 2), ((1, 96, 50, 47), (128, 96, 5, 5), 2, 2), ((1, 32, 66, 70), (200, 32, 9, 10), 4, 2),
+    ((2, 64, 40, 36), (96, 64, 7, 7), 3, 3), ((1, 32, 80, 80), (64, 32, 5, 5), 2, 3), ((1, 32, 14, 20, 22), (40, 32, 5, 5, 5), 2, 2),
+    ((1, 64, 45, 45), (256, 64, 3, 3), 1, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", DMA_CASES)
+def test_dma_fed_tile_per_run_equals_the_register_staged_one(dev, dtype, case, gemm_override):
+    """Both kernels add the pieces of a run and the channel blocks in the same order: bit-identical outputs; and
+    against fp64 convolution."""
+    xs, ws, pad, m = case
+    g = torch.Generator().manual_seed(33)
+    x = torch.randn(*xs, generator=g).to(dtype)
+    fan = 1
+    for v in ws[1:]:
+        fan *= v
+    w = (torch.randn(*ws, generator=g) * (2.0 / fan) ** 0.5).to(dtype)
+    b = torch.randn(ws[0], generator=g).to(dtype)
+    ref = _conv(x.double(), w.double(), b.double(), pad)
+    gemm_override(rows_mode=2)
+    y2 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, m, stacked=2)
+    gemm_override(rows_mode=3)
+    y3 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, m, stacked=2)
+    assert torch.equal(y2, y3)
+    tol = {2: (3e-3, 2e-2), 3: (1e-2, 5e-2)}[m]             # F(3,3) evaluates at 2 as well: 3.1e-3 in fp16, 2.6e-2 in bf16
+    assert _rel(y3, ref) <= tol[dtype == torch.bfloat16]
+
+
 TILE3 = [c for c in CASES if len(c[0]) == 4 and min(c[1][2:]) >= 3 and max(c[1][2:]) >= 4]
 
 
@@ -221,6 +260,12 @@ def test_random_shapes(dev, case):
 @pytest.mark.parametrize("case", RANDOM[::2], ids=[str(i) for i in range(0, len(RANDOM), 2)])
 def test_random_shapes_with_one_operand_tile_per_run(dev, case, gemm_override):
     gemm_override(rows_mode=2)
+    test_random_shapes(dev, case)
+
+
+@pytest.mark.parametrize("case", RANDOM[1::2], ids=[str(i) for i in range(1, len(RANDOM), 2)])
+def test_random_shapes_with_the_dma_fed_tile_per_run(dev, case, gemm_override):
+    gemm_override(rows_mode=3)
     test_random_shapes(dev, case)
 
 
