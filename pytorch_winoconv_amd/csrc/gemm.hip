@@ -832,6 +832,18 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(Cp > 0 && Cp % 32 == 0, "wc_batched_gemm: reduction extent %d is not a multiple of 32", Cp);
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "wc_batched_gemm: row stride %d (needs >= K, multiple of 8)", ldm);
   WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32 || dtype == WC_BF16, "wc_batched_gemm: dtype %d", dtype);
+  // Persistent 256 x 256 tiles (gemm_persistent.hip) where whole layers measured faster with them than with every
+  // tile below (fp16, N = 64: 512 -> 512 channels at 28 x 28 0.148 ms against 0.154, 512 -> 256 at 56 x 56 0.349 against
+  // 0.375): reductions of 512 and more channels over at least three and a half rounds of tiles, the last round mostly
+  // full.  At 256 channels the product alone is 10 % faster on operands that come from HBM, but not behind an input
+  // transform that has just written them (0.234 ms either way at the 256-channel 56 x 56 layer), and smaller problems
+  // lose.  wc_test_gemm_override(10, .) takes the kernel wherever it runs.
+  if (gemm_persistent_fits(T_, P, Cp, K, dtype)) {
+    const int force = test_gemm_config();
+    const long long tiles = (long long)ceil_div(P, 256) * (K / 256) * T_, rounds = ceil_div_ll(tiles, kCus);
+    const bool by_size = Cp >= 512 && tiles >= 896 && tiles * 100 >= rounds * kCus * 85;
+    if (force == 10 || (force < 0 && by_size)) return gemm_persistent(V, U, M, T_, P, Cp, K, ldm, dtype, stream);
+  }
   GemmConfig c = dispatch_dtype(dtype, [&](auto t) { return choose<decltype(t)>(T_, P, K, Cp); });
   GemmArgs g;
   g.V = V; g.U = U; g.M = M;

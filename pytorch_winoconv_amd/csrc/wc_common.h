@@ -119,6 +119,9 @@ inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream);
 
+// wc_batched_gemm on persistent 256 x 256 tiles fed by LDS-DMA (gemm_persistent.hip): 16-bit types, K a multiple of 256
+bool gemm_persistent_fits(int T, int P, int Cp, int K, int dtype);
+int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, void* stream);
 // The same product on tiles of 512 x 128 fed by LDS-DMA (gemm_rows_dma.hip): runs of 2 to 5 pieces
 bool gemm_rows_dma_fits(SharedShift sh, int P, int Cp, int K, int dtype);
 int gemm_rows_dma(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm, int dtype,

@@ -201,6 +201,55 @@ def test_batched_gemm_long_reduction_tile(dev, dtype, gemm_override):
     assert torch.equal(M[:, :, :K], M0[:, :, :K])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,P,C,K", [
+    (3, 1000, 96, 256),        # three reduction steps (the fewest), a partial tile of rows
+    (5, 257, 256, 512),        # one row into the second tile, two tiles of channels
+    (2, 4096, 160, 256),       # whole tiles
+    (40, 300, 128, 256),       # more tiles than workgroups per XCD in a range that does not divide evenly
+    (1, 31, 512, 256),         # fewer tiles than workgroups: most return at once
+])
+def test_batched_gemm_persistent_tiles(dev, dtype, T, P, C, K, gemm_override):
+    """The persistent 256 x 256 kernel (chosen by size for long reductions over many tiles; forced here through
+    wc_test_gemm_override so that small shapes reach it): against an fp64 product, and bit for bit against the
+    256 x 128 tile of gemm_kernel, which adds the same products in the same order.  Rows of M beyond K are not
+    written by either."""
+    g = torch.Generator().manual_seed(6)
+    V = torch.randn(T, P, C, generator=g).to(dtype).to(dev)
+    U = (torch.randn(T, K, C, generator=g) / C ** 0.5).to(dtype).to(dev)
+    gemm_override(config=10)
+    M = engine.batched_gemm(V, U)
+    want = torch.bmm(V.double(), U.double().transpose(1, 2))
+    assert _rel(M[:, :, :K], want) <= (2e-3 if dtype == torch.float16 else 8e-3)
+    gemm_override(config=0)
+    M0 = engine.batched_gemm(V, U)
+    assert torch.equal(M, M0)
+
+
+def test_batched_gemm_persistent_tiles_integer_exact(dev, gemm_override):
+    g = torch.Generator().manual_seed(7)
+    V = torch.randint(-4, 5, (7, 700, 96), generator=g).half()
+    U = torch.randint(-3, 4, (7, 256, 96), generator=g).half()
+    want = torch.bmm(V.double(), U.double().transpose(1, 2))
+    gemm_override(config=10)
+    M = engine.batched_gemm(V.to(dev), U.to(dev))
+    assert torch.equal(M.double().cpu(), want)
+
+
+def test_batched_gemm_persistent_tiles_by_size(dev):
+    """A long reduction over three and a half rounds of tiles (the F(4x4,3x3) product of a 512 -> 256 channel layer)
+    takes the persistent kernel by itself: first and last batches against fp64."""
+    g = torch.Generator().manual_seed(8)
+    T, P, C, K = 36, 6500, 512, 256
+    V = torch.randn(T, P, C, generator=g).half().to(dev)
+    U = (torch.randn(T, K, C, generator=g) / C ** 0.5).half().to(dev)
+    M = engine.batched_gemm(V, U)
+    want = torch.bmm(V[:4].double(), U[:4].double().transpose(1, 2))
+    assert _rel(M[:4], want) <= 2e-3
+    want = torch.bmm(V[-2:].double(), U[-2:].double().transpose(1, 2))
+    assert _rel(M[-2:], want) <= 2e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_batched_gemm_integer_exact(dev, dtype):
     g = torch.Generator().manual_seed(4)
