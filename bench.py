@@ -133,6 +133,7 @@ SUITE = [
     ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 shared input F(2,2)^3", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16"),
     ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 F(2,r)^3 stacked", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16-stacked"),
     ("metric fp16 N64 C256 56x56 F(2,3)", (64, 256, 56, 56), (256, 256, 3, 3), 1, 1, 2, "f16"),
+    ("fp16 N64 C512 28x28 F(4,3) (batched GEMM on persistent 256x256 tiles)", (64, 512, 28, 28), (512, 512, 3, 3), 1, 1, 4, "f16"),
 ]
 VGG16 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),
          (256, 256, 56), (256, 512, 28), (512, 512, 28), (512, 512, 28), (512, 512, 14), (512, 512, 14),
