@@ -138,6 +138,8 @@ DMA_CASES = [
     ((2, 64, 40, 36), (136, 64, 7, 7), 3, 2), ((1, 96, 50, 47), (128, 96, 5, 5), 2, 2), ((1, 32, 66, 70), (200, 32, 9, 10), 4, 2),
     ((2, 64, 40, 36), (96, 64, 7, 7), 3, 3), ((1, 32, 80, 80), (64, 32, 5, 5), 2, 3), ((1, 32, 14, 20, 22), (40, 32, 5, 5, 5), 2, 2),
     ((1, 64, 45, 45), (256, 64, 3, 3), 1, 2),
+    # more tiles than workgroups: a workgroup walks over two or three tiles of its XCD's range
+    ((2, 32, 160, 160), (136, 32, 5, 5), 2, 3), ((1, 32, 200, 190), (128, 32, 7, 7), 3, 2),
 ]
 
 

@@ -208,6 +208,8 @@ def test_batched_gemm_long_reduction_tile(dev, dtype, gemm_override):
     (2, 4096, 160, 256),       # whole tiles
     (40, 300, 128, 256),       # more tiles than workgroups per XCD in a range that does not divide evenly
     (1, 31, 512, 256),         # fewer tiles than workgroups: most return at once
+    (60, 1300, 96, 256),       # 360 tiles: some workgroups walk over two
+    (41, 1100, 128, 512),      # 410 tiles, ranges of 51 and 52 tiles per XCD
 ])
 def test_batched_gemm_persistent_tiles(dev, dtype, T, P, C, K, gemm_override):
     """The persistent 256 x 256 kernel (chosen by size for long reductions over many tiles; forced here through
