@@ -220,12 +220,14 @@ def test_winoconv3d_module(dev):
     assert torch.equal(mod3(x3), F.conv3d(x3, mod3.weight, mod3.bias, 1, 1)) and mod3._cache is None
 
 
-@pytest.mark.parametrize("ws,m,stacked", [
-    ((48, 32, 5, 5), 4, 0),        # DWM pieces, four kernels
-    ((48, 32, 5, 5), 2, 2),        # two-tap pieces sharing one transformed input (shifted GEMM operand)
-    ((48, 32, 3, 3), 2, 0),        # thin 16-bit 3x3 layer: filter transform + the one fused kernel
+@pytest.mark.parametrize("ws,m,stacked,force", [
+    ((48, 32, 5, 5), 4, 0, None),        # DWM pieces, four kernels
+    ((48, 32, 5, 5), 2, 2, None),        # two-tap pieces sharing one transformed input (shifted GEMM operand)
+    ((48, 32, 3, 3), 2, 0, None),        # thin 16-bit 3x3 layer: filter transform + the one fused kernel
+    ((48, 32, 5, 5), 2, 2, (-1, 3)),     # ... the shifted product on its persistent LDS-DMA kernel
+    ((256, 96, 3, 3), 4, 0, (10, 1)),    # the batched GEMM on its persistent LDS-DMA kernel
 ])
-def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked):
+def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked, force, gemm_override):
     """The library allocates nothing, never synchronises and takes its stream from the caller, so a
     whole forward pass can be captured once and replayed.  The graph is replayed three times with new
     input contents, eager work and synchronisation between the replays, and every replay must equal
@@ -233,7 +235,9 @@ def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked):
     import ctypes
     from pytorch_winoconv_amd import _lib
     lib = _lib.load()
-    xs = (2, 32, 20, 20)
+    if force:
+        gemm_override(*force)
+    xs = (2, ws[1], 20, 20)
     pad = ws[2] // 2
     g = torch.Generator().manual_seed(11)
     x = torch.randn(*xs, generator=g).half().to(dev).contiguous(memory_format=torch.channels_last)
@@ -243,7 +247,7 @@ def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked):
     _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
     wsp = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
     x_cl = pkg.engine.channel_last(x)
-    y = torch.empty(2, 20, 20, 48, dtype=torch.float16, device=dev)
+    y = torch.empty(2, 20, 20, ws[0], dtype=torch.float16, device=dev)
     strides = pkg.engine._w_strides(w)
 
     def forward():
