@@ -128,6 +128,7 @@ SUITE = [
     ("c4 fp16 N32 C128 112x112 5x5 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 5, 5), 1, 2, 4, "f16-pieces"),
     ("c4 fp16 N32 C128 112x112 7x7 s1 DWM F(4,r) piece by piece", (32, 128, 112, 112), (128, 128, 7, 7), 1, 3, 4, "f16-pieces"),
     ("first layer fp16 N32 3->64 224x224 7x7 s2 (the direct form's first-layer kernel)", (32, 3, 224, 224), (64, 3, 7, 7), 2, 3, 4, "f16"),
+    ("3-D first layer fp16 N8 3->64 16x112x112 3x3x3 (the direct form's 3-D first-layer kernel)", (8, 3, 16, 112, 112), (64, 3, 3, 3, 3), 1, 1, 2, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)^3", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 2, "f16"),
     ("c5 fp16 N8 C128 16x56x56 3x3x3 F(2,3)xF(4,3)^2", (8, 128, 16, 56, 56), (128, 128, 3, 3, 3), 1, 1, 4, "f16"),
     ("3-D DWM fp16 N4 C64 16x28x28 5x5x5 shared input F(2,2)^3", (4, 64, 16, 28, 28), (64, 64, 5, 5, 5), 1, 2, 2, "f16"),

@@ -124,7 +124,9 @@ typedef struct {
                     *    reductions always, longer ones where the output fills the chip) and for fp32 3x3 layers at
                     *    stride 2 over at most 128 channels: strides the reference does not implement
                     *    (src/winograd_conv.cpp:122-126) and where Winograd tiles on the parity phases save few or no
-                    *    multiplications.  wc_conv_forward, wc_filter_transform,
+                    *    multiplications; and for first layers with at most 4 channels in a 16-bit type - 2-D at stride 2
+                    *    (3 / 5 / 7 kernel rows of at most 8 taps, U (K, kH, 8, 4)) and 3-D 3x3x3 at stride 1 (rows of at
+                    *    most 4 taps, U (K, 9, 4, 4)) - which have kernels of their own.  wc_conv_forward, wc_filter_transform,
                     *    wc_conv_workspace_bytes and wc_conv_u_elems honour it; the other stage functions do not apply. */
 } wc_conv_desc;
 

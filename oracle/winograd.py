@@ -30,6 +30,8 @@ transform_kernels_3d.cu:4987).
   "bf16"  the same contract with bfloat16 storage (the reference has no bfloat16 path).
 """
 import math
+import itertools
+
 import torch
 
 from . import cook_toom
@@ -272,21 +274,24 @@ def direct_conv(x, w, bias=None, stride=1, padding=0, discipline="fp32"):
     are 1, so y[b, k, oy, ox] = sum over taps (ky, kx) and channels of x[b, c, stride oy + ky - pad, stride ox + kx - pad]
     w[k, c, ky, kx] with nothing transformed: the products are added tap by tap (ky outermost, the order the engine's
     product walks its reduction axis) in the arithmetic type of the discipline, the bias is added to the sum, and the
-    result is rounded once to the storage type.  2-D.  The reference has no such form and no stride 2 at all
-    (src/winograd_conv.cpp:122-126); the definition of the convolution itself (torch's conv2d in fp64) pins it."""
+    result is rounded once to the storage type.  2-D, or 3-D with the kernel planes outermost.  The reference has no such
+    form and no stride 2 at all (src/winograd_conv.cpp:122-126); the definition of the convolution itself (torch's
+    conv2d / conv3d in fp64) pins it."""
     mt, st = _MATH[discipline], _STORE[discipline]
-    B, C, H, W = x.shape
-    K, _, kh, kw = w.shape
-    ph, pw = (padding, padding) if isinstance(padding, int) else tuple(padding)
-    oH, oW = out_dims((H, W), (kh, kw), (ph, pw), stride)
-    xp = torch.zeros(B, C, H + 2 * ph + stride, W + 2 * pw + stride, dtype=mt)
-    xp[:, :, ph:ph + H, pw:pw + W] = x.to(st).to(mt)
+    nd = x.dim() - 2
+    B, C = x.shape[:2]
+    K = w.shape[0]
+    sp, ks = tuple(x.shape[2:]), tuple(w.shape[2:])
+    pads = (padding,) * nd if isinstance(padding, int) else tuple(padding)
+    outs = out_dims(sp, ks, pads, stride)
+    xp = torch.zeros(B, C, *[n + 2 * p + stride for n, p in zip(sp, pads)], dtype=mt)
+    xp[(slice(None), slice(None)) + tuple(slice(p, p + n) for n, p in zip(sp, pads))] = x.to(st).to(mt)
     wm = w.to(st).to(mt)
-    acc = torch.zeros(B, K, oH, oW, dtype=mt)
-    for ky in range(kh):
-        for kx in range(kw):
-            win = xp[:, :, ky:ky + stride * (oH - 1) + 1:stride, kx:kx + stride * (oW - 1) + 1:stride]
-            acc += torch.einsum("bchw,kc->bkhw", win, wm[:, :, ky, kx])
+    acc = torch.zeros(B, K, *outs, dtype=mt)
+    letters = "hw" if nd == 2 else "dhw"
+    for tap in itertools.product(*[range(k) for k in ks]):
+        win = xp[(slice(None), slice(None)) + tuple(slice(t, t + stride * (o - 1) + 1, stride) for t, o in zip(tap, outs))]
+        acc += torch.einsum("bc%s,kc->bk%s" % (letters, letters), win, wm[(slice(None), slice(None)) + tap])
     if bias is not None:
-        acc += bias.to(st).to(mt).view(1, K, 1, 1)
+        acc += bias.to(st).to(mt).view(1, K, *([1] * nd))
     return acc.to(st)

@@ -99,11 +99,16 @@ class _WinoConvNd(nn.Module):
                      and len(set(self.stride)) == 1 and self.groups == 1 and set(self.dilation) == {1})
             if not first:
                 return False
-        # ... and so do 3-D first layers with at most 4 input channels, for which there is no fused kernel like the
-        # 2-D one: F(2,3)^3 on 3 channels padded to 32 makes V eighty times the input (N=2, 3 -> 64, 16x112x112:
-        # 0.27 ms in fp16 and 0.52 ms in fp32 against 0.12 and 0.11 ms)
+        # ... and so do 3-D first layers with at most 4 input channels: F(2,3)^3 on 3 channels padded to 32 makes V eighty
+        # times the input (N=2, 3 -> 64, 16x112x112: 0.27 ms in fp16 and 0.52 ms in fp32 against 0.12 and 0.11 ms) -
+        # except 3x3x3 layers at stride 1 in a 16-bit type, for which the direct form has a kernel (N=8: 0.05 ms against
+        # 0.41-0.57 ms)
         if self.nd == 3 and self.in_channels <= 4:
-            return False
+            first3d = (x.dtype in (torch.float16, torch.bfloat16) and tuple(self.kernel_size) == (3, 3, 3)
+                       and set(self.stride) == {1} and self.out_channels % 8 == 0 and self.groups == 1
+                       and set(self.dilation) == {1})
+            if not first3d:
+                return False
         return (self.groups == 1 and set(self.dilation) == {1} and len(set(self.stride)) == 1
                 and self.stride[0] in (1, 2) and max(self.kernel_size) <= 10)
 

@@ -119,7 +119,7 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
   // through a channel-last copy of one chunk (the one-kernel path: of the whole batch)
   L->x_direct = d->x_layout == 1 && ((!L->thin && !L->direct && input_transform_nchw_fits(d, &L->plan)) ||
-                                     (L->direct && direct_first_fits(d_in)));      // ... and so does the first-layer kernel
+                                     (L->direct && (direct_first_fits(d_in) || direct_first3d_fits(d_in))));      // ... and so do the first-layer kernels
   const size_t images = L->thin || L->direct ? d->N : chunk;
   const size_t x_image = (size_t)d->in[0] * d->in[1] * d->in[2] * d->C * L->es;
   const size_t y_image = (size_t)L->out[0] * L->out[1] * L->out[2] * d->K * L->es;

@@ -39,6 +39,7 @@ __global__ __launch_bounds__(256) void direct_filter_kernel(DirectFilterArgs a) 
 }
 
 bool direct_conv_fits(const wc_conv_desc* d) {
+  if (direct_first3d_fits(d)) return true;        // 3-D first layers: the only 3-D problems with a direct form (direct_first3d.hip)
   if (d->ndim != 2) return false;
   if (direct_first_fits(d)) return true;          // strided first layers: their own kernel and filter layout (direct_first.hip)
   if (d->C % (d->dtype == WC_F32 ? 16 : 32) != 0 || d->K % 8 != 0) return false;   // whole reduction blocks along C, 16-byte stores along K
@@ -52,11 +53,13 @@ bool direct_conv_fits(const wc_conv_desc* d) {
 }
 
 size_t direct_u_elems(const wc_conv_desc* d) {
+  if (direct_first3d_fits(d)) return direct_first3d_u_elems(d);
   return direct_first_fits(d) ? direct_first_u_elems(d) : (size_t)d->K * d->kernel[1] * d->kernel[2] * d->C;
 }
 
 int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream) {
   WC_CHECK_ARG(w && w_strides && U, "direct filter copy: null pointer");
+  if (direct_first3d_fits(d)) return direct_first3d_filter(d, w, w_strides, U, stream);
   if (direct_first_fits(d)) return direct_first_filter(d, w, w_strides, U, stream);
   DirectFilterArgs a;
   a.w = w; a.U = U;
@@ -73,12 +76,13 @@ int direct_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[
 
 int direct_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y, void* stream) {
   WC_CHECK_ARG(direct_conv_fits(d), "direct convolution: 2-D, input channels a multiple of 32 (fp32: 16), output "
-               "channels a multiple of 8");
+               "channels a multiple of 8 (or a first layer with at most 4 channels in a 16-bit type: 2-D at stride 2, 3-D 3x3x3 at stride 1)");
   int out[3], grid[3];
   wc_conv_desc e = *d;
   e.direct = 0; e.stacked = 0; e.m = 2;
   int rc = wc_conv_out_dims(&e, out, grid);
   if (rc) return rc;
+  if (direct_first3d_fits(d)) return direct_first3d_conv(d, x, n_images, U, bias, y, out, stream);
   if (direct_first_fits(d)) return direct_first_conv(d, x, n_images, U, bias, y, out[1], out[2], stream);
   return gemm_direct_conv(x, U, bias, y, n_images, d->in[1], d->in[2], d->C, d->K, d->kernel[1], d->kernel[2], d->stride,
                           d->pad[1], d->pad[2], out[1], out[2], d->dtype, stream);

@@ -372,6 +372,8 @@ static int auto_stacked(const wc_conv_desc* d) {
 //  * A kernel of one tap at either stride, every type: the tile F(m,1) has nothing to save and its transforms are
 //    copies (fp16 N=64, 64 -> 256 channels, 56x56: three kernels 78 us).
 static bool direct_preferred(const wc_conv_desc* d) {
+  // 3-D first layers (direct_first3d.hip; N=8, 3 -> 64, 16x112x112 in fp16: the Winograd plan 1.05 ms)
+  if (direct_first3d_fits(d)) return true;
   const int taps = d->kernel[1] * d->kernel[2];
   if (taps == 1) return true;
   if (d->stride != 2) return false;

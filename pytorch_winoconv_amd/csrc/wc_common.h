@@ -147,6 +147,13 @@ size_t direct_first_u_elems(const wc_conv_desc* d);
 int direct_first_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
 int direct_first_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y,
                       int oH, int oW, void* stream);
+// 3-D first layers (direct_first3d.hip): at most 4 input channels, a 3x3x3 kernel (rows of at most 4 taps) at stride 1,
+// 16-bit types; U is (K, 9, 4, 4)
+bool direct_first3d_fits(const wc_conv_desc* d);
+size_t direct_first3d_u_elems(const wc_conv_desc* d);
+int direct_first3d_filter(const wc_conv_desc* d, const void* w, const int64_t w_strides[5], void* U, void* stream);
+int direct_first3d_conv(const wc_conv_desc* d, const void* x, int n_images, const void* U, const void* bias, void* y,
+                        const int out[3], void* stream);
 // o_step > 0: row (b, oy, ox) of the result goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of image b of an
 // (o_H, o_W) tensor instead of to row b oH oW + oy oW + ox
 int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, int N, int H, int W, int C, int K,

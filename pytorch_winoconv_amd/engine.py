@@ -334,7 +334,9 @@ def transform_filter(w, x_shape, stride=1, padding=0, m=2, whole_kernel=False, s
         n = ctypes.c_size_t()
         check(_lib.load().wc_conv_u_elems(ctypes.byref(desc), ctypes.byref(n)))
         shape = (desc.K, desc.kernel[1], desc.kernel[2], desc.C)
-        if n.value != shape[0] * shape[1] * shape[2] * shape[3]:
+        if desc.ndim == 3:
+            shape = (desc.K, desc.kernel[0] * desc.kernel[1], 4, 4)      # 3-D first layers: rows of 4 taps of 4 channels
+        elif n.value != shape[0] * shape[1] * shape[2] * shape[3]:
             shape = (desc.K, desc.kernel[1], 8, 4)
         U = torch.empty(shape, dtype=w.dtype, device=w.device)
         plan = Plan()

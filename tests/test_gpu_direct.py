@@ -252,3 +252,63 @@ def test_first_layer_module_trains(dev):
     b64 = mod.bias.detach().double().cpu().requires_grad_(True)
     F.conv2d(x.double().cpu(), w64, b64, stride=2, padding=3).backward(dy.double().cpu())
     assert _rel(mod.weight.grad, w64.grad) <= 2e-2 and _rel(mod.bias.grad, b64.grad) <= 2e-2
+
+
+FIRST3D_CASES = [
+    # x shape, w shape, pad: 3-D first layers (at most 4 channels, 3x3x3 at stride 1, rows of at most 4 taps)
+    ((2, 3, 6, 20, 21), (64, 3, 3, 3, 3), 1), ((1, 3, 4, 33, 18), (16, 3, 3, 3, 3), (1, 0, 1)), ((1, 1, 5, 16, 16), (8, 1, 3, 3, 3), 1),
+    ((2, 4, 3, 9, 35), (72, 4, 3, 3, 4), (0, 1, 2)), ((1, 2, 7, 17, 17), (136, 2, 3, 3, 2), (1, 1, 0)), ((3, 3, 8, 40, 40), (32, 3, 3, 3, 3), 1),
+    ((1, 3, 3, 3, 3), (8, 3, 3, 3, 3), 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", FIRST3D_CASES)
+def test_3d_first_layers_are_exact_on_small_integers(dev, dtype, case, host_layer):
+    """first3d_kernel (csrc/direct_first3d.hip), the library's own choice for these layers: bit-equal to direct
+    convolution on small integers, bias included, to the oracle, from channel-last and from channel-first memory."""
+    xs, ws, pad = case
+    g = torch.Generator().manual_seed(18)
+    x = torch.randint(-3, 4, xs, generator=g).double()
+    w = torch.randint(-2, 3, ws, generator=g).double()
+    b = torch.randint(-8, 9, (ws[0],), generator=g).double()
+    ref = F.conv3d(x, w, b, stride=1, padding=pad)
+    assert float(ref.abs().max()) < {torch.float16: 2048, torch.bfloat16: 256}[dtype]
+    assert engine.make_desc(xs, ws, dtype, 1, pad, 2, stacked=None).direct == 1
+    xd, wd, bd = x.to(dtype).to(dev), w.to(dtype).to(dev), b.to(dtype).to(dev)
+    y = engine.conv_forward(xd, wd, bd, 1, pad, 2)
+    assert tuple(y.shape) == tuple(ref.shape)
+    assert torch.equal(y.cpu(), ref.float().to(dtype))
+    assert torch.equal(y.cpu(), ow.direct_conv(x, w, b, 1, pad, DISC[dtype]))
+    ycl = engine.conv_forward(xd.contiguous(memory_format=torch.channels_last_3d), wd, bd, 1, pad, 2)
+    assert torch.equal(ycl, y)
+    U = engine.transform_filter(wd, xs, 1, pad, 2)
+    assert tuple(U.shape) == (ws[0], 9, 4, 4)
+    assert torch.equal(U[:, :, :ws[4], :ws[1]], wd.permute(0, 2, 3, 4, 1).reshape(ws[0], 9, ws[4], ws[1]))
+    assert float(U[:, :, ws[4]:].abs().sum()) == 0 and float(U[:, :, :, ws[1]:].abs().sum()) == 0
+    assert torch.equal(engine.conv_forward(xd, wd, bd, 1, pad, 2, U=U), y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_3d_first_layer_against_fp64_and_through_the_module(dev, dtype):
+    """N=2, 3 -> 64, 3x3x3 on 8 x 56 x 56 clips: against fp64 convolution and the oracle on normal data, values beside the
+    window that are not finite do not leak into it, and WinoConv3d keeps the layer in the engine in 16-bit types."""
+    import pytorch_winoconv_amd as pkg
+    g = torch.Generator().manual_seed(19)
+    x = torch.randn(2, 3, 8, 56, 56, generator=g).to(dtype)
+    w = (torch.randn(64, 3, 3, 3, 3, generator=g) * (2.0 / 81) ** 0.5).to(dtype)
+    ref = F.conv3d(x.double(), w.double(), None, stride=1, padding=1)
+    y = engine.conv_forward(x.to(dev), w.to(dev), None, 1, 1, 2)
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.2e-2}[dtype]
+    assert _rel(y, ref) <= tol
+    assert _rel(y[:1, :, :2], ow.direct_conv(x[:1, :, :3], w, None, 1, 1, DISC[dtype])[:, :, :2]) <= tol
+    # an infinity one pixel to the right of a window (the fourth, padded tap of a row) stays out of it
+    xi = x.clone()
+    xi[0, :, 4, 20, 30] = float("inf")
+    yi = engine.conv_forward(xi.to(dev), w.to(dev), None, 1, 1, 2)
+    assert torch.isfinite(yi[0, :, 4, 20, :29]).all() and torch.equal(yi[0, :, 4, 20, :29], y[0, :, 4, 20, :29])
+    mod = pkg.WinoConv3d(3, 64, 3, 1, 1, bias=False, dtype=dtype, device=dev)
+    with torch.no_grad():
+        mod.weight.copy_(w.to(dev))
+    ym = mod(x.to(dev))
+    assert mod._cache is not None and torch.equal(ym, y)

@@ -26,3 +26,20 @@ def test_direct_form_is_the_convolution(xs, ws, stride, pad):
     # the same sum as the decomposed forms of the oracle
     yd = ow.dwm_conv(x, w, b, stride, pad, 2, "fp32")
     assert float((y32 - yd).abs().max() / ref.abs().max()) < 1e-5
+
+
+CASES_3D = [((2, 3, 5, 8, 9), (4, 3, 3, 3, 3), 1, 1), ((1, 4, 6, 7, 7), (5, 4, 3, 3, 2), 1, (1, 0, 1)), ((1, 2, 4, 6, 5), (3, 2, 2, 3, 3), 2, 1)]
+
+
+@pytest.mark.parametrize("xs,ws,stride,pad", CASES_3D)
+def test_direct_form_is_the_convolution_in_3d(xs, ws, stride, pad):
+    """The same restatement with the kernel planes outermost: torch's conv3d in fp64, and bit for bit on integers."""
+    g = torch.Generator().manual_seed(1)
+    x, w, b = torch.randn(*xs, generator=g), torch.randn(*ws, generator=g), torch.randn(ws[0], generator=g)
+    ref = F.conv3d(x.double(), w.double(), b.double(), stride=stride, padding=pad)
+    y = ow.direct_conv(x, w, b, stride, pad, "fp64")
+    assert y.shape == ref.shape and float((y - ref).abs().max()) < 1e-12
+    xi, wi = torch.randint(-3, 4, xs, generator=g).double(), torch.randint(-2, 3, ws, generator=g).double()
+    for disc in ("fp32", "fp16", "bf16"):
+        yi = ow.direct_conv(xi, wi, None, stride, pad, disc)
+        assert torch.equal(yi.double(), F.conv3d(xi, wi, stride=stride, padding=pad))
