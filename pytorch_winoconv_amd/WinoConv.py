@@ -101,7 +101,7 @@ class _WinoConvNd(nn.Module):
                 return False
         # ... and so do 3-D first layers with at most 4 input channels: F(2,3)^3 on 3 channels padded to 32 makes V eighty
         # times the input (N=2, 3 -> 64, 16x112x112: 0.27 ms in fp16 and 0.52 ms in fp32 against 0.12 and 0.11 ms) -
-        # except 3x3x3 layers at stride 1 in a 16-bit type, for which the direct form has a kernel (N=8: 0.05 ms against
+        # except 3x3x3 layers at stride 1 in a 16-bit type, for which the direct form has a kernel (N=8: 0.06 ms against
         # 0.41-0.57 ms)
         if self.nd == 3 and self.in_channels <= 4:
             first3d = (x.dtype in (torch.float16, torch.bfloat16) and tuple(self.kernel_size) == (3, 3, 3)

@@ -12,7 +12,7 @@
 // over tiles persistently.  Per tile the input patch (3 planes of 18 rows of 19 pixels) goes global -> registers ->
 // LDS with the channels padded to 4 (zero outside the image; patches are requested two tiles ahead, into two sets of
 // registers, and LDS holds two patches); the filter fragments of the workgroup's 64 output channels (9 rows x 2
-// channel blocks) stay in registers; 36 `v_mfma_f32_32x32x16` per wavefront and tile; the result leaves through LDS as
+// channel blocks) stay in LDS; 36 `v_mfma_f32_32x32x16` per wavefront and tile; the result leaves through LDS as
 // whole 128-byte pixel rows with the bias added before the one rounding.  The taps a kernel row does not have meet
 // zeros on both sides (the filter's padding, and the fragment's half for them is cleared: a pixel beside the window
 // may hold anything, infinities included).  x may be channel-last or channel-first (five element strides).
@@ -50,7 +50,7 @@ struct First3dArgs {
 };
 
 template <typename T, int KD, int KH>
-__global__ __launch_bounds__(256, 2) void first3d_kernel(First3dArgs a) {
+__global__ __launch_bounds__(256, 3) void first3d_kernel(First3dArgs a) {
   using MF = MfmaG<T>;
   using Frag = typename MF::Frag;
   constexpr int R = KD * KH;                               // kernel rows = MFMA steps
@@ -59,23 +59,25 @@ __global__ __launch_bounds__(256, 2) void first3d_kernel(First3dArgs a) {
   constexpr int PATCH = KD * PLANE;
   constexpr int NPIX = KD * PH * kPatchW;                  // pixels a patch loads
   constexpr int NL = (NPIX + 255) / 256;                   // pixels per thread
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * PATCH + 4 * 32 * 128];
+  constexpr int UBYTES = 2 * R * 64 * 16;                  // the filter fragments of 64 output channels: (block, row, lane) x 16 bytes
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * PATCH + 4 * 32 * 128 + UBYTES];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int k0 = blockIdx.y * 64;
   const uint16_t* xb = static_cast<const uint16_t*>(a.x);
 
-  // filter fragments of this lane's two output channels (k0 + l32, k0 + 32 + l32): U is (K, R, 4 taps, 4 channels), a
-  // lane's 8 elements being taps 2 lhi and 2 lhi + 1
-  Frag uf[2][R];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int k = min(k0 + 32 * j + l32, a.K - 1);
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      uf[j][r] = *reinterpret_cast<const Frag*>(static_cast<const T*>(a.U) + ((long long)k * R + r) * 16 + lhi * 8);
+  // filter fragments of the workgroup's 64 output channels, in LDS in the order the lanes read them (block j, row r,
+  // lane: the 16 bytes of output channel k0 + 32 j + l32, taps 2 lhi and 2 lhi + 1 of U (K, R, 4 taps, 4 channels));
+  // in registers they would cost 8 R registers and a wavefront per SIMD
+  unsigned char* ulds = lds + 2 * PATCH + 4 * 32 * 128;
+  for (int q = tid; q < 2 * R * 64; q += 256) {
+    const int ln = q & 63, r = (q >> 6) % R, j = q / (64 * R);
+    const int k = min(k0 + 32 * j + (ln & 31), a.K - 1);
+    *reinterpret_cast<u32x4*>(ulds + q * 16) =
+        *reinterpret_cast<const u32x4*>(static_cast<const T*>(a.U) + ((long long)k * R + r) * 16 + (ln >> 5) * 8);
   }
+  const unsigned char* ufrag = ulds + lane * 16;
 
   // patch pixels of this thread: q = tid + 256 n -> (plane, row, column)
   int pz[NL], prow[NL], pcol[NL];
@@ -159,7 +161,9 @@ __global__ __launch_bounds__(256, 2) void first3d_kernel(First3dArgs a) {
     for (int kz = 0; kz < KD; ++kz)
 #pragma unroll
       for (int ky = 0; ky < KH; ++ky) {
-        Frag vf[2];
+        Frag vf[2], uf[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) uf[j] = *reinterpret_cast<const Frag*>(ufrag + (j * R + kz * KH + ky) * (64 * 16));
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
           const unsigned char* p = patch + kz * PLANE + ky * kPitch * 8 + frag_off[i];
@@ -172,7 +176,7 @@ __global__ __launch_bounds__(256, 2) void first3d_kernel(First3dArgs a) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = MF::run(uf[j][kz * KH + ky], vf[i], acc[i][j]);
+          for (int j = 0; j < 2; ++j) acc[i][j] = MF::run(uf[j], vf[i], acc[i][j]);
       }
     // epilogue: 32 pixels x 64 channels per block row through this wavefront's staging block (128-byte rows, the
     // 16-byte chunks of a row swizzled by the row), then whole pixel rows to y
@@ -283,8 +287,8 @@ int direct_first3d_conv(const wc_conv_desc* d, const void* x, int n_images, cons
   a.n_tiles = (int)tiles;
   auto fn = d->dtype == WC_F16 ? &first3d_kernel<half_t, 3, 3> : &first3d_kernel<bf16_t, 3, 3>;
   const int k_blocks = ceil_div(d->K, 64);
-  // persistent workgroups: two per CU, fewer where the tiles do not fill them
-  int grid = 2 * kCus / k_blocks;
+  // persistent workgroups: three per CU, fewer where the tiles do not fill them
+  int grid = 3 * kCus / k_blocks;
   if (grid < 1) grid = 1;
   if (grid > a.n_tiles) grid = a.n_tiles;
   hipLaunchKernelGGL(fn, dim3((unsigned)grid, (unsigned)k_blocks), dim3(256), 0, as_stream(stream), a);
