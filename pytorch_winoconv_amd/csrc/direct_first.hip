@@ -11,13 +11,13 @@
 //
 // A workgroup (four wavefronts) owns tiles of 16 x 16 output pixels x 64 output channels and walks over tiles
 // persistently.  Per tile the input patch (2 x 15 + kh rows of 2 x 15 + 8 pixels) goes global -> registers -> LDS with
-// the channels padded to 4 (zero outside the image; the patch of the next tile is requested before this tile is
-// multiplied and LDS holds two patches); the filter fragments of a wavefront's 64 output channels (kh x 2 x 2
+// the channels padded to 4 (zero outside the image; patches are requested two tiles ahead, into two sets of registers,
+// and LDS holds two patches); the filter fragments of a wavefront's 64 output channels (kh x 2 x 2
 // fragments) stay in registers for the life of the workgroup; 8 kh `v_mfma_f32_32x32x16` per wavefront and tile; the
 // result leaves through LDS as whole 128-byte pixel rows with the bias added before the one rounding.  x is read once
 // (plus the halo of the tiles), y written once, nothing else touches memory.  x may be channel-last or channel-first
 // (wc_conv_desc.x_layout): the patch loader takes the four element strides, so a torch tensor in its default layout
-// needs no copy (N=32, 3 -> 64, 224x224: 0.031 ms either way; a channel-last copy of x first costs 0.04 ms more).
+// needs no copy (N=32, 3 -> 64, 224x224: 0.026 ms either way; a channel-last copy of x first costs 0.04 ms more).
 #include "wc_common.h"
 
 namespace wc {
@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256, 2) void first_strided_kernel(FirstArgs a) {
     prow[n] = q < NPIX ? q / kPatchW : -1;
     pcol[n] = q - (q / kPatchW) * kPatchW;
   }
-  uint16_t pv[NL][4];
-  auto load_patch = [&](int tile) {
+  uint16_t pva[NL][4], pvb[NL][4];             // the patches of the next two tiles, on their way
+  auto load_patch = [&](int tile, uint16_t (&pv)[NL][4]) {
     const int tx = tile % a.tiles_x, ty = (tile / a.tiles_x) % a.tiles_y, b = tile / (a.tiles_x * a.tiles_y);
     const int iy0 = 2 * ty * kTile - a.pad_h, ix0 = 2 * tx * kTile - a.pad_w;
 #pragma unroll
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256, 2) void first_strided_kernel(FirstArgs a) {
       }
     }
   };
-  auto store_patch = [&](int buf) {
+  auto store_patch = [&](int buf, const uint16_t (&pv)[NL][4]) {
 #pragma unroll
     for (int n = 0; n < NL; ++n) {
       if (prow[n] < 0) continue;
@@ -126,13 +126,16 @@ __global__ __launch_bounds__(256, 2) void first_strided_kernel(FirstArgs a) {
 
   int tile = blockIdx.x;
   if (tile >= a.n_tiles) return;
-  load_patch(tile);
+  load_patch(tile, pva);
+  if (tile + (int)gridDim.x < a.n_tiles) load_patch(tile + gridDim.x, pvb);
   int buf = 0;
-  for (; tile < a.n_tiles; tile += gridDim.x) {
-    store_patch(buf);
+  // one tile; `mine`: the registers its patch arrived in, refilled with the patch of the tile after next (the memory
+  // latency under load is longer than one tile's work: with one tile ahead every tile waited for its patch)
+  auto do_tile = [&](int tile, uint16_t (&mine)[NL][4]) {
+    store_patch(buf, mine);
     __syncthreads();                                    // the patch is complete; the other buffer is free (its tile is done)
-    const int next = tile + gridDim.x;
-    if (next < a.n_tiles) load_patch(next);
+    const int next = tile + 2 * gridDim.x;
+    if (next < a.n_tiles) load_patch(next, mine);
     f32x16 acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -187,6 +190,10 @@ __global__ __launch_bounds__(256, 2) void first_strided_kernel(FirstArgs a) {
       }
     }
     buf ^= 1;
+  };
+  for (; tile < a.n_tiles; tile += 2 * gridDim.x) {
+    do_tile(tile, pva);
+    if (tile + (int)gridDim.x < a.n_tiles) do_tile(tile + gridDim.x, pvb);
   }
 }
 
