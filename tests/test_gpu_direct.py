@@ -312,3 +312,24 @@ def test_3d_first_layer_against_fp64_and_through_the_module(dev, dtype):
         mod.weight.copy_(w.to(dev))
     ym = mod(x.to(dev))
     assert mod._cache is not None and torch.equal(ym, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_3d_first_layer_module_trains(dev, dtype):
+    """Gradients of a WinoConv3d first layer (forward on first3d_kernel, gradients in the transform domain) against fp64
+    autograd of the same layer."""
+    import pytorch_winoconv_amd as pkg
+    g = torch.Generator().manual_seed(20)
+    mod = pkg.WinoConv3d(3, 16, 3, 1, 1, bias=True, dtype=dtype, device=dev)
+    x = torch.randn(2, 3, 6, 20, 22, generator=g).to(dtype).to(dev).requires_grad_(True)
+    y = mod(x)
+    dy = torch.randn(y.shape, generator=g).to(dtype).to(dev)
+    y.backward(dy)
+    xr = x.detach().double().requires_grad_(True)
+    wr = mod.weight.detach().double().requires_grad_(True)
+    br = mod.bias.detach().double().requires_grad_(True)
+    F.conv3d(xr, wr, br, 1, 1).backward(dy.double())
+    tol = {torch.float16: 4e-3, torch.bfloat16: 3e-2}[dtype]
+    assert mod._cache is not None
+    assert _rel(mod.weight.grad.detach(), wr.grad) <= tol and _rel(mod.bias.grad.detach(), br.grad) <= tol
+    assert _rel(x.grad.detach(), xr.grad) <= tol
