@@ -58,7 +58,13 @@ struct Layout {
   bool direct;                        // the direct form: the product reads x itself, V and M are not needed
   bool x_direct;                      // channel-first x is read by the input transform itself
   size_t xcl_bytes, ycl_bytes;        // channel-last scratch copies of a chunk of x / of y (0 if not needed)
-  size_t need() const { return (thin || direct ? u_bytes : u_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
+  // 3-D F(2,3)^3 plans in 16-bit types: the width half of the output transform is folded into the product
+  // (batched_gemm_fold_w, gemm.hip): M holds 32 elements per tile instead of 64, the workspace also the folded filter
+  bool fold;
+  size_t fold_bytes;
+  wc_conv_desc fold_desc;             // what the output transform then sees: a kernel one tap wide, the same output
+  wc_plan fold_plan;
+  size_t need() const { return (thin || direct ? u_bytes : u_bytes + fold_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
 };
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -116,6 +122,29 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   L->v_bytes = round256((size_t)T * (Pc + (L->shared ? L->shift.tail : 0)) * L->vrow * L->es);
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
   L->thin = !L->direct && !d->unfused && thin_conv_fits(d, &L->plan);
+  L->fold = false; L->fold_bytes = 0;
+  {
+    const wc_plan& pl = L->plan;
+    const bool cube = !L->direct && !L->shared && !d->whole_kernel && d->ndim == 3 && pl.n_pieces == 1 &&
+                      pl.tap_step == 1 && pl.m[0] == 2 && pl.m[1] == 2 && pl.m[2] == 2 && pl.piece[0].r[0] == 3 &&
+                      pl.piece[0].r[1] == 3 && pl.piece[0].r[2] == 3 && (d->dtype == WC_F16 || d->dtype == WC_BF16);
+    // where the product waits for memory (at most 128 channels) and the problem is large enough for the smaller M to
+    // matter (fp16 N=8 16x56x56: 128 -> 128 channels 0.604 against 0.712 ms, 64 -> 128 0.394 | 0.590, 32 -> 32 0.575 |
+    // 0.705; 256 -> 256 on 8x28x28 0.118 | 0.107, 512 -> 512 on 8x14x14 0.15 | 0.076: half more multiplications where they
+    // are what the product waits for; 128 -> 128 on one 8x28x28 clip 0.034 | 0.031).  wc_test_gemm_override(11, .)
+    // switches it off, (12, .) on for every such plan.
+    const int force = test_gemm_config();
+    if (cube && force != 11 && (force == 12 || (L->Cp <= 128 && Pc >= 4096))) {
+      wc_conv_desc f = *d;
+      f.kernel[2] = 1; f.pad[2] = 0; f.in[2] = L->out[2]; f.x_layout = 0; f.y_layout = 0;
+      if (wc_plan_conv(&f, &L->fold_plan) == WC_OK && L->fold_plan.t_total == 32) {
+        L->fold = true;
+        L->fold_desc = f;
+        L->fold_bytes = round256((size_t)32 * d->K * 3 * L->Cp * L->es);
+        L->m_bytes = round256((size_t)32 * Pc * L->ldm * L->es);
+      }
+    }
+  }
   // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
   // through a channel-last copy of one chunk (the one-kernel path: of the whole batch)
   L->x_direct = d->x_layout == 1 && ((!L->thin && !L->direct && input_transform_nchw_fits(d, &L->plan)) ||
@@ -230,7 +259,7 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
                  d->ndim, dt[d->dtype], d->N, d->C, d->K, d->in[0], d->in[1], d->in[2], d->kernel[0], d->kernel[1], d->kernel[2],
                  d->stride, d->pad[0], d->pad[1], d->pad[2], L.plan.m[0], L.plan.m[1], L.plan.m[2], L.plan.n_pieces, L.plan.t_total,
                  d->stacked, d->whole_kernel ? " whole-kernel tile" : "",
-                 L.direct ? "direct form: the product reads x" : L.thin ? "one fused kernel" : (L.shared ? "input transform, shifted batched GEMM, output transform"
+                 L.direct ? "direct form: the product reads x" : L.thin ? "one fused kernel" : L.fold ? "input transform, batched GEMM with the width half of the output transform folded in, output transform" : (L.shared ? "input transform, shifted batched GEMM, output transform"
                                                          : "input transform, batched GEMM, output transform"),
                  L.thin || L.direct ? d->N : L.chunk, L.tiles_per_image, need, L.u_bytes, L.thin || L.direct ? (size_t)0 : L.v_bytes,
                  L.thin || L.direct ? (size_t)0 : L.m_bytes, L.xcl_bytes, L.ycl_bytes,
@@ -239,9 +268,11 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
   }
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   void* Uws = ws;
-  void* V = ws + L.u_bytes;
-  void* M = ws + L.u_bytes + L.v_bytes;
-  unsigned char* tail = ws + (L.thin || L.direct ? L.u_bytes : L.u_bytes + L.v_bytes + L.m_bytes);
+  void* Ufold = ws + L.u_bytes;
+  void* V = ws + L.u_bytes + L.fold_bytes;
+  void* M = ws + L.u_bytes + L.fold_bytes + L.v_bytes;
+  unsigned char* tail = ws + (L.thin || L.direct ? L.u_bytes : L.u_bytes + L.fold_bytes + L.v_bytes + L.m_bytes);
+  bool folded = false;
   void* Xcl = tail;                       // channel-last copies of channel-first tensors, one chunk each
   void* Ycl = tail + L.xcl_bytes;
   StageTimer timer(stage_ms != nullptr, stream);
@@ -288,12 +319,25 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
       });
       if (rc) return rc;
       filter_with_input = false;
+      if (L.fold && !folded) {          // (after the launch that may have transformed the filter beside the input)
+        rc = timer.run(WC_STAGE_FILTER, [&] { return fold_filter_w(U, Ufold, d->K, L.Cp, d->dtype, stream); });
+        if (rc) return rc;
+        folded = true;
+      }
       rc = timer.run(WC_STAGE_PRODUCT, [&] {
+        if (L.fold) return batched_gemm_fold_w(V, Ufold, M, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
         return L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
                         : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
       });
       if (rc) return rc;
-      rc = timer.run(WC_STAGE_OUTPUT, [&] { return wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream); });
+      rc = timer.run(WC_STAGE_OUTPUT, [&] {
+        if (L.fold) {
+          wc_conv_desc fd = L.fold_desc;
+          fd.N = dcl.N;
+          return wc_output_transform(&fd, &L.fold_plan, M, bias, n, ydst, stream);
+        }
+        return wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream);
+      });
       if (rc) return rc;
     }
     if (L.ycl_bytes) {

@@ -86,6 +86,11 @@ struct GemmArgs {
   // parity class of its pixels): row (b, oy, ox) of the product goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of
   // image b of an (o_H, o_W) tensor; o_step == 0: rows are written one after the other
   int o_step, o_y0, o_x0, o_H, o_W;
+  // shifted operand only: batches in pairs (batched_gemm_fold_w).  Batch 2 g + j of the launch is the pair member j of
+  // group g, at g sV + j sV2 (and likewise in U and M), and the two members of a group are neighbouring workgroups: they
+  // share most of their V rows, which the second then finds in L2
+  int pair;
+  long long sV2, sU2, sM2;
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -118,13 +123,16 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
 
   const int blk = xcd_remap(blockIdx.x, g.per_xcd);
   if (blk >= g.n_blocks) return;
-  const int kt_ = blk % g.tiles_k;
-  const int pt = (blk / g.tiles_k) % g.tiles_p;
-  const int t = blk / (g.tiles_k * g.tiles_p);
+  const bool pair = SHIFT && !DIRECT && g.pair;
+  const int member = pair ? blk & 1 : 0;
+  const int rest = pair ? blk >> 1 : blk;
+  const int kt_ = rest % g.tiles_k;
+  const int pt = (rest / g.tiles_k) % g.tiles_p;
+  const int t = rest / (g.tiles_k * g.tiles_p);
   const int p0 = pt * BM, k0 = kt_ * BN;
 
-  const T* Vt = static_cast<const T*>(g.V) + (long long)t * g.sV;
-  const T* Ut = static_cast<const T*>(g.U) + (long long)t * g.sU;
+  const T* Vt = static_cast<const T*>(g.V) + (long long)t * g.sV + (pair ? member * g.sV2 : 0);
+  const T* Ut = static_cast<const T*>(g.U) + (long long)t * g.sU + (pair ? member * g.sU2 : 0);
 
   const int tid = threadIdx.x;
   const int lrow = tid / CPR, lpart = tid % CPR;
@@ -254,7 +262,7 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   constexpr int CS = BN + EPC;                     // padded row of the staged output tile
   constexpr int SROWS = 32 * NWP * EI;             // staged rows per pass: NWP wavefront rows x EI x 32
   T* cs = lds;   // operand stages are free after the last barrier; the launch sizes LDS for both uses
-  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
+  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM + (pair ? member * g.sM2 : 0);
   constexpr int CPRO = BN / EPC;                   // 16-byte chunks per output row
   constexpr int RPPO = NT / CPRO;                  // rows per pass
   static_assert(NT % CPRO == 0 && SROWS % RPPO == 0, "output tile shape");
@@ -725,7 +733,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   g.plane_runs = sh.n_runs;
   g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
-  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0; g.pair = 0; g.sV2 = g.sU2 = g.sM2 = 0;
   g.n_run = sh.n_run; g.total_runs = sh.n_planes * sh.n_runs;
   g.run_rows = sh.run_rows; g.plane_extra = sh.plane_rows - sh.n_runs * sh.run_rows;
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
@@ -737,6 +745,74 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
   hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
   WC_CHECK_LAUNCH(rows ? "gemm_rows_kernel" : "gemm_kernel (shifted operand)");
+  return WC_OK;
+}
+
+// ---- the width half of the output transform folded into the product (3-D F(2,3)^3 plans) -------------------------------
+// A^T of F(2,3) along the width only adds and subtracts: y0 = m0 + m1 + m2, y1 = m1 - m2 - m3 over the four width elements
+// of a (depth, height) element pair g.  Each is ONE product over a three times longer reduction: y0[g] = [V0 | V1 | V2] x
+// [U0 | U1 | U2]^T, y1[g] = [V1 | V2 | V3] x [U1 | -U2 | -U3]^T - the shifted operand of gemm_kernel<SHIFT> whose V pointer
+// jumps on by one element plane after every Cp channels.  M then has 32 elements per tile instead of 64, written once
+// and read once by the output transform (kinds F(2,3), F(2,3), F(2,1): nothing left to do along the width), for half more
+// multiplications in a product that waits for memory.  Uf (2, 16, K, 3 Cp) from fold_filter_w; Mf (32, P, ldm) with
+// element index 2 g + (0 | 1).
+template <typename T>
+__global__ __launch_bounds__(256) void fold_filter_kernel(const T* __restrict__ U, T* __restrict__ Uf, int K, int Cp, long long total) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int cv = Cp / 8;
+  const int c8 = (int)(idx % cv);
+  long long q = idx / cv;
+  const int piece = (int)(q % 3); q /= 3;
+  const int k = (int)(q % K); q /= K;
+  const int g = (int)(q % 16);
+  const int j2 = (int)(q / 16);
+  Chunk16 v = *reinterpret_cast<const Chunk16*>(U + ((long long)(4 * g + j2 + piece) * K + k) * Cp + c8 * 8);
+  if (j2 == 1 && piece >= 1) {                           // minus: the sign bits of the eight 16-bit values
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] ^= 0x80008000u;
+  }
+  *reinterpret_cast<Chunk16*>(Uf + (((long long)(j2 * 16 + g) * K + k) * 3 + piece) * Cp + c8 * 8) = v;
+}
+
+int fold_filter_w(const void* U, void* Uf, int K, int Cp, int dtype, void* stream) {
+  WC_CHECK_ARG(U && Uf && K > 0 && Cp > 0 && Cp % 32 == 0 && (dtype == WC_F16 || dtype == WC_BF16), "fold_filter_w: K %d, Cp %d", K, Cp);
+  const long long total = 2ll * 16 * K * 3 * (Cp / 8);
+  const unsigned blocks = (unsigned)ceil_div_ll(total, 256);
+  hipLaunchKernelGGL(fold_filter_kernel<half_t>, dim3(blocks), dim3(256), 0, as_stream(stream), static_cast<const half_t*>(U),
+                     static_cast<half_t*>(Uf), K, Cp, total);      // bit pattern only: one instance serves both 16-bit types
+  WC_CHECK_LAUNCH("fold_filter_kernel");
+  return WC_OK;
+}
+
+int batched_gemm_fold_w(const void* V, const void* Uf, void* Mf, int P, int Cp, int K, int ldm, int dtype, void* stream) {
+  WC_CHECK_ARG(V && Uf && Mf, "batched_gemm_fold_w: null pointer");
+  WC_CHECK_ARG(P > 0 && K > 0 && Cp > 0 && Cp % 32 == 0 && ldm >= K && ldm % 8 == 0, "batched_gemm_fold_w: P %d, K %d, Cp %d, ldm %d", P, K, Cp, ldm);
+  if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_fold_w: 16-bit types only");
+  const GemmConfig c = dtype == WC_F16 ? choose_shifted<half_t>(16, P, K) : choose_shifted<bf16_t>(16, P, K);
+  const long long plane = (long long)P * Cp;
+  GemmArgs g;
+  g.P = P; g.K = K; g.ldm = ldm;
+  g.Cp = 3 * Cp;                                         // reduction length = row length of Uf
+  g.ldv = Cp;
+  g.run_blocks = Cp / c.bk;                              // after the channels of one element: on to the next element plane
+  g.jump = plane - Cp;
+  g.plane_runs = 1 << 30; g.jump2 = 0;
+  g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0; g.pair = 0; g.sV2 = g.sU2 = g.sM2 = 0;
+  g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
+  g.sV = 4 * plane; g.sU = (long long)K * g.Cp; g.sM = 2ll * P * ldm;
+  g.pair = 1; g.sV2 = plane; g.sU2 = 16 * g.sU; g.sM2 = (long long)P * ldm;
+  g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 32;
+  const long long blocks = (long long)g.tiles_p * g.tiles_k * 32;
+  WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_fold_w: problem too large");
+  g.n_blocks = (int)blocks;
+  g.per_xcd = ceil_div((int)blocks, kXcds);
+  g.per_xcd += g.per_xcd & 1;                            // the two members of a pair on one XCD
+  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
+  g.V = V; g.U = Uf; g.M = Mf;
+  hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
+  WC_CHECK_LAUNCH("gemm_kernel (element planes along the reduction)");
   return WC_OK;
 }
 
@@ -810,7 +886,7 @@ int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, in
   g.H = H; g.W = W; g.oH = oH; g.oW = oW; g.conv_stride = stride; g.pad_h = pad_h; g.pad_w = pad_w;
   g.kw = kw; g.cblocks = C / c.bk;
   g.o_step = o_step; g.o_y0 = o_y0; g.o_x0 = o_x0; g.o_H = o_H; g.o_W = o_W;
-  g.sV = 0; g.sU = 0; g.sM = 0;
+  g.sV = 0; g.sU = 0; g.sM = 0; g.pair = 0; g.sV2 = g.sU2 = g.sM2 = 0;
   g.tiles_p = ceil_div((int)P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 1;
   const long long blocks = (long long)g.tiles_p * g.tiles_k;
   g.n_blocks = (int)blocks;
@@ -852,7 +928,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
   g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
-  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0; g.pair = 0; g.sV2 = g.sU2 = g.sM2 = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

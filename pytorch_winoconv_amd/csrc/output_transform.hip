@@ -323,6 +323,9 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
   if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23)
     return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 2>
                     : &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 1>;
+  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_21)        // F(2,3)^3 with the width half done by the product
+    return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_21, 2>
+                    : &output_transform_kernel<T, KIND_23, KIND_23, KIND_21, 1>;
   if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43)
     return vec == 4 ? &output_transform_3d_m4_kernel<T, 2> : &output_transform_3d_m4_kernel<T, 1>;
   // whole-kernel tiles F(2,r) x F(2,r), r = 4..7

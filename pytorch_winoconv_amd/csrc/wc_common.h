@@ -119,6 +119,10 @@ inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream);
 
+// The width half of the output transform of 3-D F(2,3)^3 plans folded into the product (gemm.hip): U (64, K, Cp) ->
+// Uf (2, 16, K, 3 Cp), and the product V (64, P, Cp) x Uf -> Mf (32, P, ldm)
+int fold_filter_w(const void* U, void* Uf, int K, int Cp, int dtype, void* stream);
+int batched_gemm_fold_w(const void* V, const void* Uf, void* Mf, int P, int Cp, int K, int ldm, int dtype, void* stream);
 // wc_batched_gemm on persistent 256 x 256 tiles fed by LDS-DMA (gemm_persistent.hip): 16-bit types, K a multiple of 256
 bool gemm_persistent_fits(int T, int P, int Cp, int K, int dtype);
 int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, void* stream);

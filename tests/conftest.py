@@ -34,10 +34,14 @@ def gemm_override():
     from pytorch_winoconv_amd import _lib
     lib = _lib.load()
 
+    from pytorch_winoconv_amd import engine
+
     def force(config=-1, rows_mode=1):
         _lib.check(lib.wc_test_gemm_override(config, rows_mode))
+        engine._SETUPS.clear()              # workspace sizes are kept per problem, and some settings change them
     yield force
     _lib.check(lib.wc_test_gemm_override(-1, 1))
+    engine._SETUPS.clear()
 
 
 @pytest.fixture(params=["compiled", "ctypes"])
