@@ -144,8 +144,8 @@ const char* wc_last_error(void);
  * pieces, else as 1).
  * config 10: wc_batched_gemm on persistent 256 x 256 tiles wherever that kernel runs (16-bit types, K a
  * multiple of 256, reductions of 96 and more).
- * config 11 / 12: 3-D F(2,3)^3 plans in 16-bit types never / always fold the width half of the output transform
- * into the product (by size otherwise).
+ * config 11 / 12: 3-D F(2,3)^3 plans in 16-bit types never / always take the width axis inside the product
+ * (transforms along depth and height only, the three width taps along the reduction; by size otherwise).
  * config 8 / 9: the one-kernel F(2x2,3x3) path with workgroups of 64 / 32 output channels whatever
  * the number of tiles (9 only where the channel count allows it).
  * Works only in a process started with WINOCONV_TEST_HOOKS=1 in its environment (WC_ERR_UNSUPPORTED

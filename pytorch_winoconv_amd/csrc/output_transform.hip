@@ -349,8 +349,23 @@ static OutMultiKernel pick_multi(bool flat, int m, int vec) {
 
 using namespace wc;
 
+namespace wc {
+int output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, const void* M, const void* bias, int n_images,
+                          void* y, int grid_w, void* stream);
+int output_transform_wide(const wc_conv_desc* d, const wc_plan* plan, const void* M, const void* bias, int n_images, void* y,
+                          int grid_w, void* stream) {
+  return output_transform_impl(d, plan, M, bias, n_images, y, grid_w, stream);
+}
+}  // namespace wc
+
 extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan_in, const void* M,
                                    const void* bias, int n_images, void* y, void* stream) {
+  return wc::output_transform_impl(d, plan_in, M, bias, n_images, y, 0, stream);
+}
+
+// grid_w: 0, or the width of the tile grid M was computed on (at least what the output needs)
+int wc::output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, const void* M, const void* bias,
+                              int n_images, void* y, int grid_w, void* stream) {
   WC_CHECK_ARG(d && plan_in && M && y, "wc_output_transform: null pointer");
   // a stacked plan has one set of products (the batched GEMM has added the pieces): the output
   // transform of a single piece with the shared tile
@@ -367,6 +382,10 @@ extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan_in
   int out[3], grid[3];
   int rc = wc_conv_out_dims(d, out, grid);
   if (rc) return rc;
+  if (grid_w) {
+    WC_CHECK_ARG(grid_w >= grid[2], "wc_output_transform: a tile grid %d wide for %d tiles", grid_w, grid[2]);
+    grid[2] = grid_w;
+  }
   WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_output_transform: bad plan");
   const int ldm = wc_padded_channels8(d->K);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];

@@ -1,8 +1,9 @@
-"""3-D F(2,3)^3 plans in 16-bit types with the width half of the output transform folded into the product
-(`batched_gemm_fold_w`, csrc/gemm.hip): y0 = m0 + m1 + m2 and y1 = m1 - m2 - m3 over the four width elements are each one
-product over a three times longer reduction, so M holds 32 elements per tile instead of 64.  The library takes the path
-by size; forced here (wc_test_gemm_override(12, .)) so that small shapes reach it.  Nothing the reference does (its 3-D
-path is F(2,3)^3 through three kernels: src/base_conv_launchers.cu); the convolution itself pins it."""
+"""3-D F(2,3)^3 plans in 16-bit types with the width axis taken inside the product (`batched_gemm_fold_w`,
+csrc/gemm.hip).  The input is transformed along depth and height only (V: 32 elements per tile of two columns, on a grid
+one tile wider than the output's), the three width taps lie side by side along the reduction, and the two output columns
+of a tile are two products on the same two element planes: M too holds 32 elements per tile instead of 64.  The library
+takes the path by size; forced here (wc_test_gemm_override(12, .)) so that small shapes reach it.  Nothing the reference
+does (its 3-D path is F(2,3)^3 through three kernels: src/base_conv_launchers.cu); the convolution itself pins it."""
 import pytest
 import torch
 import torch.nn.functional as F
@@ -69,8 +70,8 @@ def test_folded_product_is_exact_on_small_integers(dev, case, gemm_override):
 
 
 def test_the_library_folds_by_size(dev, gemm_override):
-    """At most 128 channels over at least 4096 tiles: the workspace of the folded path (M half as large, the folded
-    filter beside U) is what wc_conv_workspace_bytes reports; against fp64 on a slice."""
+    """Few channels over many tiles: the workspace of the folded path (V and M half as large, the folded filter beside
+    U) is what wc_conv_workspace_bytes reports; against fp64 on a slice."""
     import ctypes
     from pytorch_winoconv_amd import _lib
     lib = _lib.load()
@@ -89,7 +90,7 @@ def test_the_library_folds_by_size(dev, gemm_override):
     _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(d), ctypes.byref(nb)))
     gemm_override(config=11)
     _lib.check(lib.wc_conv_workspace_bytes(ctypes.byref(d), ctypes.byref(nb11)))
-    assert nb.value == nb11.value                                        # 256 channels: not folded
+    assert nb.value == nb11.value                                        # 256 channels over 1568 tiles: not folded
     gemm_override(config=-1)
     g = torch.Generator().manual_seed(33)
     x = torch.randn(*xs, generator=g).half()
