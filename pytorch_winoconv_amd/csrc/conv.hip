@@ -58,16 +58,13 @@ struct Layout {
   bool direct;                        // the direct form: the product reads x itself, V and M are not needed
   bool x_direct;                      // channel-first x is read by the input transform itself
   size_t xcl_bytes, ycl_bytes;        // channel-last scratch copies of a chunk of x / of y (0 if not needed)
-  // 3-D F(2,3)^3 plans in 16-bit types: the width axis is taken inside the product (batched_gemm_fold_w, gemm.hip).  V
-  // (depth and height transformed only) and M hold 32 elements per tile instead of 64, on a tile grid one tile wider
-  // than the output's; the workspace also holds the filter with the width taps side by side
+  // 3-D F(2,3)^3 plans in 16-bit types: the width axis is taken inside the product (fold_filter_w, gemm.hip).  V and M
+  // hold 16 elements per pixel column of a tile row (depth and height transformed only), half of what the plan's V and
+  // M hold; the workspace also holds the filter with the width taps side by side
   bool fold;
   size_t fold_bytes;
-  wc_conv_desc fold_in_desc;          // what the input transform sees: a kernel one tap wide, the same input
-  wc_conv_desc fold_desc;             // what the output transform sees: a kernel one tap wide, the same output
-  wc_plan fold_plan;
-  int fold_grid_w;                    // tiles along the width, of V and M
-  long long fold_tiles_per_image;     // (tiles_per_image where the plan is not folded)
+  SharedShift fold_shift;             // one run of three pieces, each one row of V further
+  long long fold_rows_per_image;      // rows of V and M: the pixel columns of all tile rows (tiles_per_image where the plan is not folded)
   size_t need() const { return (thin || direct ? u_bytes : u_bytes + fold_bytes + v_bytes + m_bytes) + xcl_bytes + ycl_bytes; }
 };
 
@@ -127,40 +124,32 @@ int make_layout(const wc_conv_desc* d_in, Layout* L) {
   L->m_bytes = round256((size_t)T * Pc * L->ldm * L->es);
   L->thin = !L->direct && !d->unfused && thin_conv_fits(d, &L->plan);
   L->fold = false; L->fold_bytes = 0;
-  L->fold_grid_w = 0; L->fold_tiles_per_image = L->tiles_per_image;
+  L->fold_rows_per_image = L->tiles_per_image;
   {
     const wc_plan& pl = L->plan;
     const bool cube = !L->direct && !L->shared && !d->whole_kernel && d->ndim == 3 && pl.n_pieces == 1 &&
                       pl.tap_step == 1 && pl.m[0] == 2 && pl.m[1] == 2 && pl.m[2] == 2 && pl.piece[0].r[0] == 3 &&
                       pl.piece[0].r[1] == 3 && pl.piece[0].r[2] == 3 && (d->dtype == WC_F16 || d->dtype == WC_BF16);
-    // Half the V and M traffic for half more multiplications, one more tile per grid row and one more launch: it pays
-    // where the pipeline waits for memory, the more channels the larger the problem has to be.  Measured fp16, ms
-    // folded | not: N=8 16x56x56 128 -> 128 channels 0.491 | 0.712, 64 -> 128 0.326 | 0.590, 64 -> 64 0.208 | 0.371;
-    // N=8 16x112x112 32 -> 32 0.463 | 0.712; one 8x28x28 clip 128 -> 128 0.028 | 0.031; 8x28x28 256 -> 256 N=16 0.335 | 0.418,
-    // N=4 0.097 | 0.106, 256 -> 512 N=2 0.095 | 0.094, 384 -> 384 N=8 0.345 | 0.372, 192 -> 192 N=4 unpadded 0.064 | 0.057;
-    // 8x14x14 384 -> 384 N=4 0.068 | 0.062, 512 -> 512 N=4 0.091 | 0.076; 8x14x14 64 -> 64 N=1 0.021 | 0.018.
+    // Half the V and M traffic for half more multiplications and one more launch: it pays where the pipeline waits
+    // for memory, the more channels the larger the problem has to be.  Measured fp16, ms folded | not: N=8 16x56x56
+    // 128 -> 128 channels 0.437 | 0.712, 64 -> 128 0.317 | 0.590, 64 -> 64 0.205 | 0.371; N=8 16x112x112 32 -> 32 0.455 | 0.712;
+    // one 8x28x28 clip 128 -> 128 0.027 | 0.031; 8x28x28 256 -> 256 N=16 0.284 | 0.415, N=4 0.093 | 0.105, 256 -> 512 N=2
+    // 0.091 | 0.094, 320 -> 320 N=4 0.138 | 0.156, 384 -> 384 N=8 0.291 | 0.367, 192 -> 192 N=4 unpadded 0.057 | 0.057;
+    // 8x14x14 384 -> 384 N=4 0.062 | 0.063, 512 -> 512 N=4 0.085 | 0.077, 512 -> 128 N=8 0.087 | 0.069; 4x14x14 512 -> 512
+    // N=16 0.151 | 0.130; 8x14x14 64 -> 64 N=1 0.017 | 0.016.
     // wc_test_gemm_override(11, .) switches it off, (12, .) on for every such plan.
     const int force = test_gemm_config();
-    const long long min_tiles = L->Cp <= 128 ? 512 : L->Cp <= 256 ? 3000 : L->Cp <= 384 ? 6000 : (1ll << 40);
+    const long long min_tiles = L->Cp <= 128 ? 512 : L->Cp <= 384 ? 3000 : (1ll << 40);
     if (cube && force != 11 && (force == 12 || Pc >= min_tiles)) {
-      wc_conv_desc fi = *d, fo = *d;
-      fi.kernel[2] = 1; fi.x_layout = 0; fi.y_layout = 0;
-      fo.kernel[2] = 1; fo.pad[2] = 0; fo.in[2] = L->out[2]; fo.x_layout = 0; fo.y_layout = 0;
-      int o3[3], g3[3];
-      wc_plan po;
-      if (wc_plan_conv(&fi, &L->fold_plan) == WC_OK && L->fold_plan.t_total == 32 && wc_plan_conv(&fo, &po) == WC_OK &&
-          po.t_total == 32 && wc_conv_out_dims(&fi, o3, g3) == WC_OK && g3[0] == L->grid[0] && g3[1] == L->grid[1] &&
-          g3[2] == L->grid[2] + 1) {
-        L->fold = true;
-        L->fold_in_desc = fi;
-        L->fold_desc = fo;
-        L->fold_grid_w = g3[2];
-        L->fold_tiles_per_image = (long long)g3[0] * g3[1] * g3[2];
-        const long long Pw = L->fold_tiles_per_image * chunk;
-        L->fold_bytes = round256((size_t)16 * d->K * 3 * L->Cp * L->es);
-        L->v_bytes = round256((size_t)(32 * Pw + 1) * L->Cp * L->es);       // one more row: the last tile's right neighbour
-        L->m_bytes = round256((size_t)32 * Pw * L->ldm * L->es);
-      }
+      const int Wx = columns_width(d);
+      L->fold = true;
+      L->fold_rows_per_image = (long long)L->grid[0] * L->grid[1] * Wx;
+      L->fold_shift.n_run = 3; L->fold_shift.n_runs = 1; L->fold_shift.n_planes = 1;
+      L->fold_shift.run_rows = Wx; L->fold_shift.plane_rows = Wx; L->fold_shift.tail = 2;
+      const long long Pw = L->fold_rows_per_image * chunk;
+      L->fold_bytes = round256((size_t)16 * d->K * 3 * L->Cp * L->es);
+      L->v_bytes = round256((size_t)16 * (Pw + 2) * L->Cp * L->es);
+      L->m_bytes = round256((size_t)16 * Pw * L->ldm * L->es);
     }
   }
   // channel-first tensors: the input transform of small single-piece plans reads x as it is; everything else goes
@@ -277,7 +266,7 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
                  d->ndim, dt[d->dtype], d->N, d->C, d->K, d->in[0], d->in[1], d->in[2], d->kernel[0], d->kernel[1], d->kernel[2],
                  d->stride, d->pad[0], d->pad[1], d->pad[2], L.plan.m[0], L.plan.m[1], L.plan.m[2], L.plan.n_pieces, L.plan.t_total,
                  d->stacked, d->whole_kernel ? " whole-kernel tile" : "",
-                 L.direct ? "direct form: the product reads x" : L.thin ? "one fused kernel" : L.fold ? "input transform (depth, height), batched GEMM with the width taps along its reduction, output transform" : (L.shared ? "input transform, shifted batched GEMM, output transform"
+                 L.direct ? "direct form: the product reads x" : L.thin ? "one fused kernel" : L.fold ? "input transform (depth, height), shifted batched GEMM with the width taps along its reduction, output transform" : (L.shared ? "input transform, shifted batched GEMM, output transform"
                                                          : "input transform, batched GEMM, output transform"),
                  L.thin || L.direct ? d->N : L.chunk, L.tiles_per_image, need, L.u_bytes, L.thin || L.direct ? (size_t)0 : L.v_bytes,
                  L.thin || L.direct ? (size_t)0 : L.m_bytes, L.xcl_bytes, L.ycl_bytes,
@@ -329,41 +318,33 @@ int forward_impl(const wc_conv_desc* d, const void* x, const void* w, const int6
       rc = timer.run(WC_STAGE_PRODUCT, [&] { return thin_conv_forward(&dcl, &L.plan, xin, U, bias, ydst, stream); });
       if (rc) return rc;
     } else {
-      const long long P = L.fold_tiles_per_image * n;
+      const long long P = L.fold_rows_per_image * n;
       WC_CHECK_ARG(P < (1ll << 31), "wc_conv_forward: chunk has too many tiles");
-      if (L.fold && filter_with_input) {     // the input transform below runs on another plan than the filter's
+      if (L.fold && filter_with_input) {     // the input transform below is not the plan's
         rc = wc_filter_transform(d, &L.plan, w, w_strides, Uws, stream);
         if (rc) return rc;
         filter_with_input = false;
       }
       rc = timer.run(WC_STAGE_INPUT, [&] {
-        if (L.fold) {
-          wc_conv_desc fi = L.fold_in_desc;
-          fi.N = dcl.N;
-          return wc_input_transform(&fi, &L.fold_plan, xin, n, V, stream);
-        }
+        if (L.fold) return input_transform_columns(&dcl, xin, n, V, stream);
         return filter_with_input ? input_filter_transform(&dcl, &L.plan, xin, n, V, w, w_strides, Uws, stream)
                                  : wc_input_transform(&dcl, &L.plan, xin, n, V, stream);
       });
       if (rc) return rc;
       filter_with_input = false;
-      if (L.fold && !folded) {          // (after the launch that may have transformed the filter beside the input)
+      if (L.fold && !folded) {
         rc = timer.run(WC_STAGE_FILTER, [&] { return fold_filter_w(U, Ufold, d->K, L.Cp, d->dtype, stream); });
         if (rc) return rc;
         folded = true;
       }
       rc = timer.run(WC_STAGE_PRODUCT, [&] {
-        if (L.fold) return batched_gemm_fold_w(V, Ufold, M, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
+        if (L.fold) return batched_gemm_shifted(V, Ufold, M, 16, (int)P, L.Cp, L.fold_shift, d->K, L.ldm, d->dtype, stream);
         return L.shared ? batched_gemm_shifted(V, U, M, L.plan.t_total, (int)P, L.vrow, L.shift, d->K, L.ldm, d->dtype, stream)
                         : wc_batched_gemm(V, U, M, L.plan.t_total, (int)P, L.Cp, d->K, L.ldm, d->dtype, stream);
       });
       if (rc) return rc;
       rc = timer.run(WC_STAGE_OUTPUT, [&] {
-        if (L.fold) {
-          wc_conv_desc fd = L.fold_desc;
-          fd.N = dcl.N;
-          return output_transform_wide(&fd, &L.fold_plan, M, bias, n, ydst, L.fold_grid_w, stream);
-        }
+        if (L.fold) return output_transform_columns(&dcl, M, bias, n, ydst, stream);
         return wc_output_transform(&dcl, &L.plan, M, bias, n, ydst, stream);
       });
       if (rc) return rc;

@@ -86,13 +86,6 @@ struct GemmArgs {
   // parity class of its pixels): row (b, oy, ox) of the product goes to pixel (o_step oy + o_y0, o_step ox + o_x0) of
   // image b of an (o_H, o_W) tensor; o_step == 0: rows are written one after the other
   int o_step, o_y0, o_x0, o_H, o_W;
-  // shifted operand only: batches in pairs (batched_gemm_fold_w).  Batch 2 g + j of the launch is the pair member j of
-  // group g, at g sV and g sU (in M: at g sM + j sM2); its reduction is three pieces of run_blocks blocks, piece i of
-  // member j reading V at vtab[j][i] elements beyond where the reduction index alone would; the two members of a group
-  // are neighbouring workgroups: they share most of their V rows, which the second then finds in L2
-  int pair;
-  long long sM2;
-  long long vtab[2][3];
 };
 
 typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));   // one 16-byte global/LDS access
@@ -125,12 +118,9 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
 
   const int blk = xcd_remap(blockIdx.x, g.per_xcd);
   if (blk >= g.n_blocks) return;
-  const bool pair = SHIFT && !DIRECT && g.pair;
-  const int member = pair ? blk & 1 : 0;
-  const int rest = pair ? blk >> 1 : blk;
-  const int kt_ = rest % g.tiles_k;
-  const int pt = (rest / g.tiles_k) % g.tiles_p;
-  const int t = rest / (g.tiles_k * g.tiles_p);
+  const int kt_ = blk % g.tiles_k;
+  const int pt = (blk / g.tiles_k) % g.tiles_p;
+  const int t = blk / (g.tiles_k * g.tiles_p);
   const int p0 = pt * BM, k0 = kt_ * BN;
 
   const T* Vt = static_cast<const T*>(g.V) + (long long)t * g.sV;
@@ -213,24 +203,18 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int nk = g.Cp / BK;
-  long long vshift = pair ? g.vtab[member][0] : 0;
+  long long vshift = 0;
   int run_left = SHIFT ? g.run_blocks : 0, plane_left = SHIFT ? g.plane_runs : 0;
-  int piece = 0;
-  gload(0, vshift);
+  gload(0, 0);
   lstore(0);
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     if constexpr (SHIFT) {
       if (--run_left == 0) {
+        vshift += g.jump;
         run_left = g.run_blocks;
-        if (pair) {
-          piece = piece < 2 ? piece + 1 : 2;
-          vshift = g.vtab[member][piece];
-        } else {
-          vshift += g.jump;
-          if (--plane_left == 0) { vshift += g.jump2; plane_left = g.plane_runs; }
-        }
+        if (--plane_left == 0) { vshift += g.jump2; plane_left = g.plane_runs; }
       }
     }
     if (kt + 1 < nk) gload(kt + 1, vshift);
@@ -270,7 +254,7 @@ __global__ __launch_bounds__(64 * NWP * NWK, (WM * WN <= 8 && NWP * NWK == 4 ? 2
   constexpr int CS = BN + EPC;                     // padded row of the staged output tile
   constexpr int SROWS = 32 * NWP * EI;             // staged rows per pass: NWP wavefront rows x EI x 32
   T* cs = lds;   // operand stages are free after the last barrier; the launch sizes LDS for both uses
-  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM + (pair ? member * g.sM2 : 0);
+  T* Mt = static_cast<T*>(g.M) + (long long)t * g.sM;
   constexpr int CPRO = BN / EPC;                   // 16-byte chunks per output row
   constexpr int RPPO = NT / CPRO;                  // rows per pass
   static_assert(NT % CPRO == 0 && SROWS % RPPO == 0, "output tile shape");
@@ -741,7 +725,7 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   g.plane_runs = sh.n_runs;
   g.jump2 = (long long)(sh.plane_rows - sh.n_runs * sh.run_rows) * Cp;   // ... and one grid plane further
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
-  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0; g.pair = 0; g.sM2 = 0;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
   g.n_run = sh.n_run; g.total_runs = sh.n_planes * sh.n_runs;
   g.run_rows = sh.run_rows; g.plane_extra = sh.plane_rows - sh.n_runs * sh.run_rows;
   g.sV = (long long)(P + sh.tail) * Cp; g.sU = (long long)K * g.Cp; g.sM = (long long)P * ldm;
@@ -757,17 +741,17 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
 }
 
 // ---- 3-D F(2,3)^3 plans with the width axis taken directly inside the product ----------------------------------------
-// Along the width nothing is transformed: V' = (B^T d B over depth and height) of every input pixel column, 4 x 4 x 2
-// elements per tile of two columns (the tile F(2,1): identity transforms), half the size of V; the filter Uw
-// (16, K, 3 Cp) holds, per (depth, height) element g, the three width taps side by side, each transformed along depth
-// and height only.  Output column j of a tile is then ONE product over a three times longer reduction,
-//   M'[g][j] = sum over the taps kx of V'[g][(j + kx) mod 2] at tile row p + (j + kx) / 2, times Uw[g][kx],
-// gemm_kernel<SHIFT> in pairs (GemmArgs.pair): the members j = 0, 1 of a group g are neighbouring workgroups reading the
-// same two element planes.  M' holds 32 elements per tile instead of 64, the output transform has nothing left to do
-// along the width (kinds F(2,3), F(2,3), F(2,1)), and V' is read and written at half the size: 12 multiplications per
-// output where F(2,3)^3 has 8, in a pipeline that waits for memory in every stage.  Uw comes from the ordinary U
-// (64, K, Cp): with G of F(2,3) = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1] its width elements are g0, (g0 + g1 + g2) / 2,
-// (g0 - g1 + g2) / 2, g2, so tap 0 is element 0, tap 2 element 3, and tap 1 element 1 minus element 2.
+// Along the width nothing is transformed: V' = (B^T d B over depth and height) of every input pixel column, 16 elements
+// per tile of 2 x 2 x 1 outputs, one row of V' per pixel column of the padded image; the filter Uw (16, K, 3 Cp) holds,
+// per (depth, height) element g, the three width taps side by side, each transformed along depth and height only.
+// Output column x is then
+//   M'[g][x] = sum over the taps kx of V'[g][x + kx] times Uw[g][kx]:
+// the product of a plan whose pieces share one transformed input, with one run of three pieces (batched_gemm_shifted).
+// M' has 16 elements per 2 x 2 x 1 outputs where F(2,3)^3 has 64 per 2 x 2 x 2, the output transform has nothing left
+// to do along the width, and V' is read and written at half the size: 12 multiplications per output where F(2,3)^3 has
+// 8, in a pipeline that waits for memory in every stage.  Uw comes from the ordinary U (64, K, Cp): with G of F(2,3) =
+// [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1] its width elements are g0, (g0 + g1 + g2) / 2, (g0 - g1 + g2) / 2, g2, so tap 0
+// is element 0, tap 2 element 3, and tap 1 element 1 minus element 2.
 __global__ __launch_bounds__(256) void fold_filter_kernel(const uint16_t* __restrict__ U, uint16_t* __restrict__ Uw, int K, int Cp,
                                                           int is_bf16, long long total) {
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -808,40 +792,6 @@ int fold_filter_w(const void* U, void* Uw, int K, int Cp, int dtype, void* strea
   hipLaunchKernelGGL(fold_filter_kernel, dim3((unsigned)ceil_div_ll(total, 256)), dim3(256), 0, as_stream(stream),
                      static_cast<const uint16_t*>(U), static_cast<uint16_t*>(Uw), K, Cp, dtype == WC_BF16, total);
   WC_CHECK_LAUNCH("fold_filter_kernel");
-  return WC_OK;
-}
-
-// V': (32, P, Cp) with one more row readable behind its end; Uw (16, K, 3 Cp); M' (32, P, ldm), element 2 g + j
-int batched_gemm_fold_w(const void* V, const void* Uw, void* Mf, int P, int Cp, int K, int ldm, int dtype, void* stream) {
-  WC_CHECK_ARG(V && Uw && Mf, "batched_gemm_fold_w: null pointer");
-  WC_CHECK_ARG(P > 0 && K > 0 && Cp > 0 && Cp % 32 == 0 && ldm >= K && ldm % 8 == 0, "batched_gemm_fold_w: P %d, K %d, Cp %d, ldm %d", P, K, Cp, ldm);
-  if (dtype != WC_F16 && dtype != WC_BF16) return fail(WC_ERR_UNSUPPORTED, "batched_gemm_fold_w: 16-bit types only");
-  const GemmConfig c = dtype == WC_F16 ? choose_shifted<half_t>(32, P, K) : choose_shifted<bf16_t>(32, P, K);
-  const long long plane = (long long)P * Cp;
-  GemmArgs g;
-  g.V = V; g.U = Uw; g.M = Mf;
-  g.P = P; g.K = K; g.ldm = ldm;
-  g.Cp = 3 * Cp;                                         // reduction length = row length of Uw
-  g.ldv = Cp;
-  g.run_blocks = Cp / c.bk;                              // blocks of one tap
-  g.jump = 0; g.plane_runs = 1 << 30; g.jump2 = 0;
-  g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
-  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
-  g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
-  g.pair = 1;
-  g.sV = 2 * plane; g.sU = (long long)K * g.Cp; g.sM = 2ll * P * ldm; g.sM2 = (long long)P * ldm;
-  for (int j = 0; j < 2; ++j)
-    for (int i = 0; i < 3; ++i)          // (minus i Cp: the reduction index has moved on by the channels of i taps)
-      g.vtab[j][i] = (long long)((j + i) & 1) * plane + (long long)((j + i) >> 1) * Cp - (long long)i * Cp;
-  g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 32;
-  const long long blocks = (long long)g.tiles_p * g.tiles_k * 32;
-  WC_CHECK_ARG(blocks < (1ll << 30), "batched_gemm_fold_w: problem too large");
-  g.n_blocks = (int)blocks;
-  g.per_xcd = ceil_div((int)blocks, kXcds);
-  g.per_xcd += g.per_xcd & 1;                            // the two members of a pair on one XCD
-  if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(c.fn), c.lds)) return rc;
-  hipLaunchKernelGGL(c.fn, dim3((unsigned)(g.per_xcd * kXcds)), dim3(c.threads), c.lds, as_stream(stream), g);
-  WC_CHECK_LAUNCH("gemm_kernel (three taps along the reduction, in pairs)");
   return WC_OK;
 }
 
@@ -915,7 +865,7 @@ int gemm_direct_conv(const void* x, const void* U, const void* bias, void* y, in
   g.H = H; g.W = W; g.oH = oH; g.oW = oW; g.conv_stride = stride; g.pad_h = pad_h; g.pad_w = pad_w;
   g.kw = kw; g.cblocks = C / c.bk;
   g.o_step = o_step; g.o_y0 = o_y0; g.o_x0 = o_x0; g.o_H = o_H; g.o_W = o_W;
-  g.sV = 0; g.sU = 0; g.sM = 0; g.pair = 0; g.sM2 = 0;
+  g.sV = 0; g.sU = 0; g.sM = 0;
   g.tiles_p = ceil_div((int)P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = 1;
   const long long blocks = (long long)g.tiles_p * g.tiles_k;
   g.n_blocks = (int)blocks;
@@ -957,7 +907,7 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   g.ldv = Cp; g.run_blocks = 0; g.jump = 0; g.plane_runs = 0; g.jump2 = 0;
   g.n_run = 0; g.total_runs = 0; g.run_rows = 0; g.plane_extra = 0;
   g.H = g.W = g.oH = g.oW = g.conv_stride = g.pad_h = g.pad_w = g.kw = g.cblocks = 0; g.bias = nullptr;
-  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0; g.pair = 0; g.sM2 = 0;
+  g.o_step = g.o_y0 = g.o_x0 = g.o_H = g.o_W = 0;
   g.tiles_p = ceil_div(P, c.bm); g.tiles_k = ceil_div(K, c.bn); g.T = T_;
   const long long blocks = (long long)g.tiles_p * g.tiles_k * T_;
   WC_CHECK_ARG(blocks < (1ll << 30), "wc_batched_gemm: problem too large");

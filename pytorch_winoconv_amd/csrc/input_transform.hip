@@ -195,6 +195,42 @@ extern "C" int wc_input_transform(const wc_conv_desc* d, const wc_plan* plan, co
 
 namespace wc {
 
+int columns_width(const wc_conv_desc* d) { return d->in[2] + 2 * d->pad[2]; }
+
+int input_transform_columns(const wc_conv_desc* d, const void* x, int n_images, void* V, void* stream) {
+  WC_CHECK_ARG(d && x && V && n_images > 0, "input_transform_columns: null pointer or no images");
+  WC_CHECK_ARG(d->ndim == 3 && d->stride == 1 && d->x_layout == 0 && d->kernel[0] == 3 && d->kernel[1] == 3 && d->kernel[2] == 3 &&
+               d->dtype != WC_F32, "input_transform_columns: 3x3x3 kernels at stride 1 on channel-last 16-bit tensors");
+  int out[3], grid[3];
+  wc_conv_desc t = *d;
+  t.m = 2;
+  int rc = wc_conv_out_dims(&t, out, grid);
+  if (rc) return rc;
+  const int Cp = wc_padded_channels(d->C);
+  const int Wx = columns_width(d);
+  const long long P = (long long)n_images * grid[0] * grid[1] * Wx;
+  int vec = 1;
+  for (int v = 4; v > 1; v /= 2)
+    if (d->C % v == 0) { vec = v; break; }
+  InArgs a;
+  a.x = x; a.V = V;
+  a.D = d->in[0]; a.H = d->in[1]; a.W = d->in[2]; a.C = d->C; a.Cp = Cp;
+  a.nD = grid[0]; a.nH = grid[1]; a.nW = Wx;
+  a.base0 = -d->pad[0]; a.base1 = -d->pad[1]; a.base2 = -d->pad[2];
+  a.step = 1;
+  a.t_stride = (P + 2) * Cp;
+  a.t_offset = 0;
+  a.n_cvec = Cp / vec;
+  a.total = P * a.n_cvec;
+  a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);
+  a.x_bytes = 0;
+  a.nq1 = a.nq2 = 1; a.q_cols = 0;
+  WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "input_transform_columns: problem too large");
+  hipLaunchKernelGGL(pick_in_columns(d->dtype, vec), dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, as_stream(stream), a);
+  WC_CHECK_LAUNCH("input_transform_kernel (pixel columns)");
+  return WC_OK;
+}
+
 int input_filter_transform(const wc_conv_desc* d, const wc_plan* plan, const void* x, int n_images, void* V,
                            const void* w, const int64_t w_strides[5], void* U, void* stream) {
   WC_CHECK_ARG(w && w_strides && U, "input_filter_transform: null pointer");

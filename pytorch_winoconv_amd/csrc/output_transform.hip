@@ -323,9 +323,6 @@ static OutKernel pick_single(int k0, int k1, int k2, int vec) {
   if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_23)
     return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 2>
                     : &output_transform_kernel<T, KIND_23, KIND_23, KIND_23, 1>;
-  if (k0 == KIND_23 && k1 == KIND_23 && k2 == KIND_21)        // F(2,3)^3 with the width half done by the product
-    return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_21, 2>
-                    : &output_transform_kernel<T, KIND_23, KIND_23, KIND_21, 1>;
   if (k0 == KIND_23 && k1 == KIND_43 && k2 == KIND_43)
     return vec == 4 ? &output_transform_3d_m4_kernel<T, 2> : &output_transform_3d_m4_kernel<T, 1>;
   // whole-kernel tiles F(2,r) x F(2,r), r = 4..7
@@ -349,23 +346,8 @@ static OutMultiKernel pick_multi(bool flat, int m, int vec) {
 
 using namespace wc;
 
-namespace wc {
-int output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, const void* M, const void* bias, int n_images,
-                          void* y, int grid_w, void* stream);
-int output_transform_wide(const wc_conv_desc* d, const wc_plan* plan, const void* M, const void* bias, int n_images, void* y,
-                          int grid_w, void* stream) {
-  return output_transform_impl(d, plan, M, bias, n_images, y, grid_w, stream);
-}
-}  // namespace wc
-
 extern "C" int wc_output_transform(const wc_conv_desc* d, const wc_plan* plan_in, const void* M,
                                    const void* bias, int n_images, void* y, void* stream) {
-  return wc::output_transform_impl(d, plan_in, M, bias, n_images, y, 0, stream);
-}
-
-// grid_w: 0, or the width of the tile grid M was computed on (at least what the output needs)
-int wc::output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, const void* M, const void* bias,
-                              int n_images, void* y, int grid_w, void* stream) {
   WC_CHECK_ARG(d && plan_in && M && y, "wc_output_transform: null pointer");
   // a stacked plan has one set of products (the batched GEMM has added the pieces): the output
   // transform of a single piece with the shared tile
@@ -382,10 +364,6 @@ int wc::output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, con
   int out[3], grid[3];
   int rc = wc_conv_out_dims(d, out, grid);
   if (rc) return rc;
-  if (grid_w) {
-    WC_CHECK_ARG(grid_w >= grid[2], "wc_output_transform: a tile grid %d wide for %d tiles", grid_w, grid[2]);
-    grid[2] = grid_w;
-  }
   WC_CHECK_ARG(plan->n_pieces > 0 && plan->n_pieces <= WC_MAX_PIECES, "wc_output_transform: bad plan");
   const int ldm = wc_padded_channels8(d->K);
   const long long P = (long long)n_images * grid[0] * grid[1] * grid[2];
@@ -449,5 +427,38 @@ int wc::output_transform_impl(const wc_conv_desc* d, const wc_plan* plan_in, con
   OutMultiKernel fn = dispatch_dtype(d->dtype, [&](auto t) { return pick_multi<decltype(t)>(flat, plan->m[1], vec); });
   hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, s, g);
   WC_CHECK_LAUNCH("output_multi_kernel");
+  return WC_OK;
+}
+
+// M (16, P, ldm) over pixel columns: P = n_images x tiles in depth x tiles in height x grid_w columns, of which the
+// first oW hold outputs (input_transform_columns, the product with the width taps along its reduction: gemm.hip)
+int wc::output_transform_columns(const wc_conv_desc* d, const void* M, const void* bias, int n_images, void* y, void* stream) {
+  WC_CHECK_ARG(d && M && y && n_images > 0, "output_transform_columns: null pointer or no images");
+  WC_CHECK_ARG(d->ndim == 3 && d->stride == 1 && d->y_layout == 0 && d->kernel[0] == 3 && d->kernel[1] == 3 && d->kernel[2] == 3 &&
+               d->dtype != WC_F32, "output_transform_columns: 3x3x3 kernels at stride 1 on channel-last 16-bit tensors");
+  int out[3], grid[3];
+  wc_conv_desc t = *d;
+  t.m = 2;
+  int rc = wc_conv_out_dims(&t, out, grid);
+  if (rc) return rc;
+  const int Wx = columns_width(d);
+  const long long P = (long long)n_images * grid[0] * grid[1] * Wx;
+  const int vec = d->K % 4 == 0 ? 4 : 1;
+  OutArgs a;
+  a.M = M; a.bias = bias; a.y = y;
+  a.oD = out[0]; a.oH = out[1]; a.oW = out[2]; a.K = d->K; a.ldm = wc_padded_channels8(d->K);
+  a.nD = grid[0]; a.nH = grid[1]; a.nW = Wx;
+  a.t_stride = P * a.ldm;
+  a.t_offset = 0;
+  a.n_kvec = d->K / vec;
+  a.total = P * a.n_kvec;
+  a.per_xcd = (int)ceil_div_ll(ceil_div_ll(a.total, 256), kXcds);
+  WC_CHECK_ARG((long long)a.per_xcd * kXcds < (1ll << 31), "output_transform_columns: problem too large");
+  OutKernel fn = dispatch_dtype(d->dtype, [&](auto t_) -> OutKernel {
+    using T = decltype(t_);
+    return vec == 4 ? &output_transform_kernel<T, KIND_23, KIND_23, KIND_11, 4> : &output_transform_kernel<T, KIND_23, KIND_23, KIND_11, 1>;
+  });
+  hipLaunchKernelGGL(fn, dim3((unsigned)(a.per_xcd * kXcds)), dim3(256), 0, as_stream(stream), a);
+  WC_CHECK_LAUNCH("output_transform_kernel (pixel columns)");
   return WC_OK;
 }

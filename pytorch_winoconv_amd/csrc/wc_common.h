@@ -119,13 +119,13 @@ inline SharedShift shared_shift(const wc_conv_desc* d, const int grid[3]) {
 int batched_gemm_shifted(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm,
                          int dtype, void* stream);
 
-// 3-D F(2,3)^3 plans with the width axis inside the product (gemm.hip): U (64, K, Cp) -> Uw (16, K, 3 Cp), and the
-// product on V' (32, P, Cp: depth and height transformed only, one more row readable behind its end) -> M' (32, P, ldm)
+// 3-D F(2,3)^3 plans with the width axis inside the product: transforms along depth and height only, over the pixel
+// columns of the padded image (columns_width per tile row); V (16, P + 2, Cp), U (64, K, Cp) -> Uw (16, K, 3 Cp)
+// (gemm.hip), the product by batched_gemm_shifted with one run of three pieces, M (16, P, ldm)
+int columns_width(const wc_conv_desc* d);
+int input_transform_columns(const wc_conv_desc* d, const void* x, int n_images, void* V, void* stream);
 int fold_filter_w(const void* U, void* Uw, int K, int Cp, int dtype, void* stream);
-int batched_gemm_fold_w(const void* V, const void* Uw, void* Mf, int P, int Cp, int K, int ldm, int dtype, void* stream);
-// wc_output_transform on a tile grid that is grid_w tiles wide (wider than the output needs: tiles beyond it write nothing)
-int output_transform_wide(const wc_conv_desc* d, const wc_plan* plan, const void* M, const void* bias, int n_images, void* y,
-                          int grid_w, void* stream);
+int output_transform_columns(const wc_conv_desc* d, const void* M, const void* bias, int n_images, void* y, void* stream);
 // wc_batched_gemm on persistent 256 x 256 tiles fed by LDS-DMA (gemm_persistent.hip): 16-bit types, K a multiple of 256
 bool gemm_persistent_fits(int T, int P, int Cp, int K, int dtype);
 int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, void* stream);

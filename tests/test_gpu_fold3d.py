@@ -1,9 +1,10 @@
-"""3-D F(2,3)^3 plans in 16-bit types with the width axis taken inside the product (`batched_gemm_fold_w`,
-csrc/gemm.hip).  The input is transformed along depth and height only (V: 32 elements per tile of two columns, on a grid
-one tile wider than the output's), the three width taps lie side by side along the reduction, and the two output columns
-of a tile are two products on the same two element planes: M too holds 32 elements per tile instead of 64.  The library
-takes the path by size; forced here (wc_test_gemm_override(12, .)) so that small shapes reach it.  Nothing the reference
-does (its 3-D path is F(2,3)^3 through three kernels: src/base_conv_launchers.cu); the convolution itself pins it."""
+"""3-D F(2,3)^3 plans in 16-bit types with the width axis taken inside the product (csrc/conv.hip, `fold`).  The input
+is transformed along depth and height only, over the pixel columns of the padded image (V: 16 elements per column of a
+tile row), the three width taps lie side by side along the reduction of the shifted batched GEMM (one run of three
+pieces, each one row of V further), and M too holds 16 elements per column: half of what F(2,3)^3 reads and writes.
+The library takes the path by size; forced here (wc_test_gemm_override(12, .)) so that small shapes reach it, with each
+of the three kernels of the shifted product (rows_mode 0, 2, 3).  Nothing the reference does (its 3-D path is F(2,3)^3
+through three kernels: src/base_conv_launchers.cu); the convolution itself pins it."""
 import pytest
 import torch
 import torch.nn.functional as F
@@ -26,9 +27,10 @@ def _rel(a, r):
     return float((a.double().cpu() - r).abs().max() / r.abs().max().clamp_min(1e-30))
 
 
+@pytest.mark.parametrize("rows_mode", [0, 2, 3])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", CASES)
-def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case, gemm_override, host_layer):
+def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case, rows_mode, gemm_override, host_layer):
     xs, K, pad = case
     g = torch.Generator().manual_seed(31)
     x = torch.randn(*xs, generator=g).to(dtype)
@@ -37,7 +39,7 @@ def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case,
     ref = F.conv3d(x.double(), w.double(), b.double(), padding=pad)
     gemm_override(config=11)
     y0 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2)
-    gemm_override(config=12)
+    gemm_override(config=12, rows_mode=rows_mode)
     y1 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, 2)
     tol = 2e-3 if dtype == torch.float16 else 1.6e-2
     assert tuple(y1.shape) == tuple(ref.shape)
@@ -50,8 +52,9 @@ def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case,
     assert ycf.is_contiguous() and torch.equal(ycf, y1)
 
 
+@pytest.mark.parametrize("rows_mode", [0, 2, 3])
 @pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
-def test_folded_product_is_exact_on_small_integers(dev, case, gemm_override):
+def test_folded_product_is_exact_on_small_integers(dev, case, rows_mode, gemm_override):
     """x in -3..3, taps multiples of 8 (G of F(2,3) halves per axis): every U, V and product is an integer and the sums
     stay below 2048 in fp16, whichever way they are grouped."""
     xs, K, pad = case
@@ -64,7 +67,7 @@ def test_folded_product_is_exact_on_small_integers(dev, case, gemm_override):
     ref = F.conv3d(x, w, b, padding=pad)
     if float(ref.abs().max()) >= 2048:
         pytest.skip("sums beyond the exact range of fp16")
-    gemm_override(config=12)
+    gemm_override(config=12, rows_mode=rows_mode)
     y = engine.conv_forward(x.half().to(dev), w.half().to(dev), b.half().to(dev), 1, pad, 2)
     assert torch.equal(y.cpu(), ref.half())
 
