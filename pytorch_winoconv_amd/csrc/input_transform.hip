@@ -209,8 +209,10 @@ int input_transform_columns(const wc_conv_desc* d, const void* x, int n_images, 
   const int Cp = wc_padded_channels(d->C);
   const int Wx = columns_width(d);
   const long long P = (long long)n_images * grid[0] * grid[1] * Wx;
+  // 16 window elements per thread: 16-byte accesses fit (measured at N=8, 128 channels, 16x56x56 fp16: 8 channels per
+  // thread 118 us, 4 125, 2 133)
   int vec = 1;
-  for (int v = 4; v > 1; v /= 2)
+  for (int v = 8; v > 1; v /= 2)
     if (d->C % v == 0) { vec = v; break; }
   InArgs a;
   a.x = x; a.V = V;

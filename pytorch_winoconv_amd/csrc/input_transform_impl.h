@@ -145,7 +145,7 @@ InKernel pick_in_2d_whole(int dtype, int k1, int k2, int vec);    // ... whole-k
 InKernel pick_in_3d_21(int dtype, int k1, int k2, int vec);       // depth kind KIND_21, vec 2 or 1
 InKernel pick_in_3d_22(int dtype, int k1, int k2, int vec);
 InKernel pick_in_3d_23(int dtype, int k1, int k2, int vec);
-InKernel pick_in_columns(int dtype, int vec);                      // kinds F(2,3), F(2,3), F(1,1); vec 4, 2 or 1
+InKernel pick_in_columns(int dtype, int vec);                      // kinds F(2,3), F(2,3), F(1,1); vec 8, 4, 2 or 1
 struct FilterFastArgs;
 // channels per thread of the filter part of that launch
 constexpr int in_filter_vec(int elem_bytes, int k1) { return elem_bytes == 4 && k1 == KIND_43 ? 1 : 8 / elem_bytes; }

@@ -443,7 +443,7 @@ int wc::output_transform_columns(const wc_conv_desc* d, const void* M, const voi
   if (rc) return rc;
   const int Wx = columns_width(d);
   const long long P = (long long)n_images * grid[0] * grid[1] * Wx;
-  const int vec = d->K % 4 == 0 ? 4 : 1;
+  const int vec = d->K % 4 == 0 ? 4 : 1;           // (2 and 8 channels per thread measured the same)
   OutArgs a;
   a.M = M; a.bias = bias; a.y = y;
   a.oD = out[0]; a.oH = out[1]; a.oW = out[2]; a.K = d->K; a.ldm = wc_padded_channels8(d->K);
