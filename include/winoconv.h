@@ -140,8 +140,9 @@ const char* wc_last_error(void);
  * library's list of shapes; -1 = choose by problem size) on wc_batched_gemm, and for plans that
  * share one transformed input the kernel with one operand tile per piece (rows_mode 0), the
  * choice by size (1, the default), one tile per run of pieces wherever the plan has runs (2), or
- * the persistent kernel with one tile per run fed by LDS-DMA wherever it runs (3: runs of 2 to 5
- * pieces, else as 1).
+ * the persistent kernel with one tile per run fed by LDS-DMA wherever it runs (runs of 2 to 5
+ * pieces, else as 1): 3 with every tile written out when it is done, 4 with the write-out riding on
+ * the workgroup's next tile wherever the tiles have the steps for that (what the choice by size takes).
  * config 10: wc_batched_gemm on persistent 256 x 256 tiles wherever that kernel runs (16-bit types, K a
  * multiple of 256, reductions of 96 and more).
  * config 11 / 12: 3-D F(2,3)^3 plans in 16-bit types never / always take the width axis inside the product

@@ -705,11 +705,13 @@ int batched_gemm_shifted(const void* V, const void* U, void* M, int T_, int P, i
   const int rows_mode = test_gemm_rows();
   // Runs of two to five pieces on at least two rounds of 512 x 128 tiles whose last block of 128 channels is at least
   // three quarters full: the persistent kernel fed by LDS-DMA (3-13 % ahead of gemm_rows_kernel there, behind it on
-  // fewer tiles and on 64 channels).  wc_test_gemm_override(., 3) takes it wherever it runs.
+  // fewer tiles and on 64 channels), with a tile's results written out during the next tile's first steps wherever a
+  // tile has the steps for that (2-6 % again).  wc_test_gemm_override(., 3) takes the kernel wherever it runs with the
+  // write-out at the end of each tile, (., 4) with the write-out riding on the next tile wherever that fits.
   if (gemm_rows_dma_fits(sh, P, Cp, K, dtype) &&
-      (rows_mode == 3 || (rows_mode == 1 && (K % 128 == 0 || K % 128 >= 96) &&
+      (rows_mode >= 3 || (rows_mode == 1 && (K % 128 == 0 || K % 128 >= 96) &&
                           (long long)ceil_div(P, 512) * ceil_div(K, 128) * T_ >= 2 * kCus)))
-    return gemm_rows_dma(V, U, M, T_, P, Cp, sh, K, ldm, dtype, stream);
+    return gemm_rows_dma(V, U, M, T_, P, Cp, sh, K, ldm, dtype, rows_mode != 3 && gemm_rows_dma_deferred_fits(sh, P, Cp, ldm), stream);
   bool rows = sh.n_run >= 2 && sh.n_run <= kRunExtra + 1 && rows_mode != 0 && (K > 32 || rows_mode == 2);
   if (rows) {
     GemmConfig r = dtype == WC_F16 ? choose_rows<half_t>(T_, P, K, rows_mode == 2) : choose_rows<bf16_t>(T_, P, K, rows_mode == 2);

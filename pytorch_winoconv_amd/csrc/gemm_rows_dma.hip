@@ -18,6 +18,12 @@
 // bytes with their 16-byte chunks swizzled by the row, as in gemm_kernel; the swizzle of a fragment read depends on the
 // piece (rows l + b), so fragment addresses are held per (piece, sub-step).  Same order of additions as
 // gemm_rows_kernel: bit-identical results.
+//
+// With one workgroup per CU nobody multiplies while a tile is written out.  Where a tile has enough steps (DG > 0
+// below) its results are therefore only packed to 16 bits when it is done (128 registers), and go out during the first
+// eight steps of the workgroup's next tile, two 32 x 32 blocks per step, each staged before a sub-step and stored
+// behind it; the last tile's follow the loop.  Those stores are counted with the loads (memory operations of both
+// kinds retire in order on this part), so the waits of the steps that carry them stay exact.
 #include "wc_common.h"
 
 namespace wc {
@@ -97,9 +103,54 @@ constexpr int prologue_in_flight(int KW) {
   return n;
 }
 
-template <typename T, int KW>
+// ---- deferred write-out (DG > 0).  A tile's results are packed into 128 registers when its last step is done, and go
+// out during the first kNS steps of the workgroup's NEXT tile, two 32 x 32 blocks per step (each through the wavefront's
+// staging area: staged before a sub-step, read back and stored behind it), so that the matrix cores do not wait for the
+// write-out.  The stores are buffer stores - lanes beyond the tensor are dropped by the bounds check of the descriptor, an
+// empty descriptor drops all of them before the first tile - so each of them is issued by every wavefront at every such
+// step and the counts below hold.  The first DG groups of a tile are unrolled (their steps know which blocks they
+// carry); the unrolled part ends late enough behind the last store that the steps of the rolled part, and the first steps
+// of the next tile, see no store in the window they count (dg_steps_ok).
+constexpr int kNS = 8;
+constexpr int imod(int a, int n) { return ((a % n) + n) % n; }
+constexpr int stores_at(int DG, int r) {      // r: step of a tile (group * KW + piece); negative: a step of the tile before
+  return DG > 0 && r >= 0 && r < kNS ? 4 : 0;
+}
+constexpr int ops_at(int KW, int DG, int r) { return v_share(KW, imod(r, KW)) + 2 + stores_at(DG, r); }
+// in_flight() with the stores counted: the order inside a step is V loads, filter loads, stores
+constexpr int in_flight_at(int KW, int DG, int s) {
+  int a = stores_at(DG, s - (kUAhead - 1));
+  for (int d = 1; d <= kUAhead - 2; ++d) a += ops_at(KW, DG, s - d);
+  if (imod(s, KW) == KW - 1) {
+    int jl = KW - 1;
+    while (v_share(KW, jl) == 0) --jl;
+    const int sp = s - 2 * KW + 1 + jl;          // the step of the previous group that queued the last load of the next V tile
+    int b = 2 + stores_at(DG, sp);
+    for (int x = sp + 1; x <= s - 1; ++x) b += ops_at(KW, DG, x);
+    if (b < a) a = b;
+  }
+  return a;
+}
+constexpr bool counts_agree(int KW) {
+  for (int kx = 0; kx < KW; ++kx)
+    if (in_flight_at(KW, 0, kx) != in_flight(KW, kx) || in_flight_at(KW, 0, kx + 3 * KW) != in_flight(KW, kx)) return false;
+  return true;
+}
+static_assert(counts_agree(2) && counts_agree(3) && counts_agree(4) && counts_agree(5), "the two ways of counting agree without stores");
+// how many steps back the count of a step reaches
+constexpr int count_reach(int KW) {
+  int jl = KW - 1;
+  while (v_share(KW, jl) == 0) --jl;
+  const int b = 2 * KW - 1 - jl;
+  return b > kUAhead - 1 ? b : kUAhead - 1;
+}
+constexpr bool dg_steps_ok(int KW, int DG) { return DG * KW - count_reach(KW) >= kNS; }
+constexpr int deferred_groups(int KW) { return (kNS + count_reach(KW) + KW - 1) / KW; }     // the fewest unrolled groups
+
+template <typename T, int KW, int DG = 0>
 __global__ __launch_bounds__(256, 1) void gemm_rows_dma_kernel(RowsDmaArgs g) {
   static_assert(KW >= 2 && KW <= 9 && sizeof(T) == 2, "runs of 2 to 9 pieces, 16-bit types");
+  static_assert(DG == 0 || dg_steps_ok(KW, DG), "unrolled groups cover the stores and their wake");
   using MF = MfmaR<T>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
@@ -245,37 +296,116 @@ __global__ __launch_bounds__(256, 1) void gemm_rows_dma_kernel(RowsDmaArgs g) {
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  // ---- deferred write-out: the previous tile's results (packed), where they go, and the two halves of a block's trip
+  // through the staging area.  Accumulator (i, j), register 4 q + e holds output channel 32 j + 8 q + 4 lhi + e of tile row
+  // 32 i + l32; held[i][j][2 q], [2 q + 1] are its registers 4 q .. 4 q + 3 as 16-bit pairs.
+  uint32_t held[DG > 0 ? WM : 1][DG > 0 ? WN : 1][8];
+  __amdgpu_buffer_rsrc_t hdesc = __builtin_amdgcn_make_buffer_rsrc(g.M, 0, 0, 0x00020000);   // no tile yet: every store is dropped
+  unsigned held_off = 0;           // byte offset in the batch of M of what this lane stores first
+  int held_kleft = 0;              // this lane stores channel blocks j with 32 j below this
+  int stg_w = 0, stg_r = 0;        // this lane's staging addresses: writes (q = 0), reads (h = 0)
+  int stg_z = 0;
+  if constexpr (DG > 0) {
+    stg_z = (l32 >> 2) & 3;
+    stg_w = kStaging + wave * 2048 + l32 * 64 + lhi * 8;
+    stg_r = kStaging + wave * 2048 + (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+  }
+  auto stage_block = [&](auto blkc) {
+    constexpr int blk = decltype(blkc)::value, i = blk / WN, j = blk % WN;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      *reinterpret_cast<u32x2*>(lds + stg_w + ((q ^ stg_z) * 16)) = u32x2{held[i][j][2 * q], held[i][j][2 * q + 1]};
+    }
+  };
+  auto store_block = [&](auto blkc) {
+    constexpr int blk = decltype(blkc)::value, i = blk / WN, j = blk % WN;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const u32x4 val = *reinterpret_cast<const u32x4*>(lds + stg_r + h * 1024);
+      unsigned off = held_off + (unsigned)(((i * 32 + h * 16) * g.ldm + j * 32) * 2);
+      if (j * 32 >= held_kleft) off = 0xFFFFFFF0u;                 // beyond the row: out of bounds, dropped
+      __builtin_amdgcn_raw_buffer_store_b128(val, hdesc, off, 0, 0);
+    }
+  };
+
+  auto run_group = [&](auto dgc) {
+    constexpr int dg = decltype(dgc)::value;          // the group's index in its tile where that is unrolled, else -1
+    static_for<0, KW>([&](auto bc) {
+      constexpr int b = decltype(bc)::value;
+      constexpr int s = dg * KW + b;
+      constexpr bool carries = dg >= 0 && s < kNS;    // this step writes blocks 2 s and 2 s + 1 of the previous tile
+      // the filter block of the next step has landed everywhere (at the last piece the next V tile too), and nobody
+      // reads the filter stage of the previous step or the V stage of the previous group any more
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(dg >= 0 ? in_flight_at(KW, DG, s) : in_flight(KW, b)) : "memory");
+      if constexpr (v_share(KW, b) > 0) issue_v(2, vs2, v_begin(KW, b), v_begin(KW, b + 1));
+      int uis = ust + kUAhead;
+      if (uis >= kUStages) uis -= kUStages;
+      issue_u((b + kUAhead) / KW, (b + kUAhead) % KW, uis);
+      __builtin_amdgcn_sched_barrier(0);
+      int usn = ust + 1;
+      if (usn == kUStages) usn = 0;
+      if constexpr (carries) { stage_block(ic<2 * (carries ? s : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
+      substep(0, vs0, ic<b>{}, ust, 1);                       // sub-step 0 multiplies; reads sub-step 1 of this step
+      if constexpr (carries) {
+        __builtin_amdgcn_sched_barrier(0);
+        store_block(ic<2 * (carries ? s : 0)>{});
+        stage_block(ic<2 * (carries ? s : 0) + 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (b + 1 < KW) substep(1, vs0, ic<b + 1>{}, usn, 0);   // sub-step 1; reads sub-step 0 of the next step
+      else substep(1, vs1, ic<0>{}, usn, 0);
+      if constexpr (carries) { __builtin_amdgcn_sched_barrier(0); store_block(ic<2 * (carries ? s : 0) + 1>{}); }
+      __builtin_amdgcn_sched_barrier(0);
+      ust = usn;
+    });
+    advance();
+    const int f = vs0; vs0 = vs1; vs1 = vs2; vs2 = f;
+  };
+
 #pragma unroll 1
   for (int local = local_first; local < local_end; local += g.wgs_per_xcd) {
+    if constexpr (DG > 0) {
+      static_for<0, DG>([&](auto dgc) { run_group(dgc); });
 #pragma unroll 1
-    for (int gi = 0; gi < G; ++gi) {
-      static_for<0, KW>([&](auto bc) {
-        constexpr int b = decltype(bc)::value;
-        // the filter block of the next step has landed everywhere (at the last piece the next V tile too), and nobody
-        // reads the filter stage of the previous step or the V stage of the previous group any more
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(in_flight(KW, b)) : "memory");
-        if constexpr (v_share(KW, b) > 0) issue_v(2, vs2, v_begin(KW, b), v_begin(KW, b + 1));
-        int uis = ust + kUAhead;
-        if (uis >= kUStages) uis -= kUStages;
-        issue_u((b + kUAhead) / KW, (b + kUAhead) % KW, uis);
-        __builtin_amdgcn_sched_barrier(0);
-        int usn = ust + 1;
-        if (usn == kUStages) usn = 0;
-        substep(0, vs0, ic<b>{}, ust, 1);                       // sub-step 0 multiplies; reads sub-step 1 of this step
-        if constexpr (b + 1 < KW) substep(1, vs0, ic<b + 1>{}, usn, 0);   // sub-step 1; reads sub-step 0 of the next step
-        else substep(1, vs1, ic<0>{}, usn, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        ust = usn;
-      });
-      advance();
-      const int f = vs0; vs0 = vs1; vs1 = vs2; vs2 = f;
+      for (int gi = DG; gi < G; ++gi) run_group(ic<-1>{});
+    } else {
+#pragma unroll 1
+      for (int gi = 0; gi < G; ++gi) run_group(ic<-1>{});
     }
 
+    const int tile = tile0 + local;
+    const int kt = tile % g.tiles_k, pt = (tile / g.tiles_k) % g.tiles_p, t = tile / (g.tiles_k * g.tiles_p);
+    if constexpr (DG > 0) {
+      // ---- the tile's results into `held` (the write-out rides on the next tile's first steps, or follows the loop)
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      const int row_first = pt * BM + wave * 128, k_first = kt * BN;
+      hdesc = __builtin_amdgcn_make_buffer_rsrc(static_cast<T*>(g.M) + (long long)t * g.sM, 0, (int)((unsigned)g.P * (unsigned)g.ldm * 2u), 0x00020000);
+      held_off = (unsigned)(((row_first + (lane_e >> 2)) * g.ldm + k_first + (lane_e & 3) * 8) * 2);
+      held_kleft = g.ldm - k_first - (lane_e & 3) * 8;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          asm volatile("" : "+a"(acc[i][j]));      // read here, block by block
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            Pack<T, 4> o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            const u32x2 w = __builtin_bit_cast(u32x2, o);
+            held[i][j][2 * q] = w[0]; held[i][j][2 * q + 1] = w[1];
+          }
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;          // for the next tile
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
     // ---- the tile's results: every wavefront stages one 32 x 32 block at a time (64-byte rows, chunks swizzled by the
     // row) and writes 64-byte row segments.  Accumulator (i, j), register 4 q + e holds output channel 32 j + 8 q + 4 lhi + e
     // of tile row 32 i + l32.  The loads of the next tile's first groups are in flight meanwhile.
-    const int tile = tile0 + local;
-    const int kt = tile % g.tiles_k, pt = (tile / g.tiles_k) % g.tiles_p, t = tile / (g.tiles_k * g.tiles_p);
     // scalar base of the tile + one lane offset: no per-store 64-bit lane addresses (which the compiler would compute
     // before the loop over the tiles and keep in registers that the loop needs)
     // lane-derived values of this part are computed here, tile by tile (behind an opaque copy of the lane id), so that
@@ -312,13 +442,29 @@ __global__ __launch_bounds__(256, 1) void gemm_rows_dma_kernel(RowsDmaArgs g) {
         }
         __builtin_amdgcn_sched_barrier(0);     // block by block: not all 256 accumulators read and converted up front
       }
+      }
+  }
+  if constexpr (DG > 0) {
+    // the last tile's results: the same trips through the staging area, with nothing to ride on
+    static_for<0, WM * WN>([&](auto blkc) {
+      stage_block(blkc);
+      store_block(blkc);
+    });
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the queue's last loads write LDS: not after this workgroup has gone
 }
 
 using RowsDmaKernel = void (*)(RowsDmaArgs);
 template <typename T>
-RowsDmaKernel pick_rows_dma(int n_run) {
+RowsDmaKernel pick_rows_dma(int n_run, bool deferred) {
+  if (deferred)
+    switch (n_run) {
+      case 2: return &gemm_rows_dma_kernel<T, 2, deferred_groups(2)>;
+      case 3: return &gemm_rows_dma_kernel<T, 3, deferred_groups(3)>;
+      case 4: return &gemm_rows_dma_kernel<T, 4, deferred_groups(4)>;
+      case 5: return &gemm_rows_dma_kernel<T, 5, deferred_groups(5)>;
+      default: return nullptr;
+    }
   switch (n_run) {
     case 2: return &gemm_rows_dma_kernel<T, 2>;
     case 3: return &gemm_rows_dma_kernel<T, 3>;
@@ -337,10 +483,26 @@ bool gemm_rows_dma_fits(SharedShift sh, int P, int Cp, int K, int dtype) {
          (long long)(P + tail) * Cp * 2 < (1ll << 31) && (long long)K * n_pieces * Cp * 2 < (1ll << 31) && K <= (1 << 17);
 }
 
+// The deferred write-out needs a tile of at least deferred_groups groups and a batch of M below 2 GB (32-bit offsets
+// into a buffer descriptor)
+bool gemm_rows_dma_deferred_fits(SharedShift sh, int P, int Cp, int ldm) {
+  const int groups = sh.n_planes * sh.n_runs * (Cp / 32);
+  int need = 1 << 30;
+  switch (sh.n_run) {
+    case 2: need = deferred_groups(2); break;
+    case 3: need = deferred_groups(3); break;
+    case 4: need = deferred_groups(4); break;
+    case 5: need = deferred_groups(5); break;
+    default: break;
+  }
+  return groups >= need && (long long)P * ldm * 2 < (1ll << 31);
+}
+
 int gemm_rows_dma(const void* V, const void* U, void* M, int T_, int P, int Cp, SharedShift sh, int K, int ldm, int dtype,
-                  void* stream) {
+                  bool deferred, void* stream) {
   const int n_pieces = sh.n_planes * sh.n_runs * sh.n_run;
   WC_CHECK_ARG(gemm_rows_dma_fits(sh, P, Cp, K, dtype), "gemm_rows_dma: runs of %d pieces, rows of %d", sh.n_run, Cp);
+  WC_CHECK_ARG(!deferred || gemm_rows_dma_deferred_fits(sh, P, Cp, ldm), "gemm_rows_dma: too few steps per tile for the deferred write-out");
   RowsDmaArgs g;
   g.V = V; g.U = U; g.M = M;
   g.P = P; g.K = K; g.ldv = Cp; g.Cu = n_pieces * Cp; g.ldm = ldm;
@@ -354,7 +516,8 @@ int gemm_rows_dma(const void* V, const void* U, void* M, int T_, int P, int Cp, 
   g.n_tiles = (int)tiles;
   g.per_xcd = ceil_div(g.n_tiles, kXcds);
   g.wgs_per_xcd = g.per_xcd < kCus / kXcds ? g.per_xcd : kCus / kXcds;
-  RowsDmaKernel fn = dtype == WC_F16 ? pick_rows_dma<half_t>(sh.n_run) : pick_rows_dma<bf16_t>(sh.n_run);
+
+  RowsDmaKernel fn = dtype == WC_F16 ? pick_rows_dma<half_t>(sh.n_run, deferred) : pick_rows_dma<bf16_t>(sh.n_run, deferred);
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), kLdsBytes)) return rc;
   hipLaunchKernelGGL(fn, dim3((unsigned)(g.wgs_per_xcd * kXcds)), dim3(256), kLdsBytes, as_stream(stream), g);
   WC_CHECK_LAUNCH("gemm_rows_dma_kernel");

@@ -108,7 +108,7 @@ using namespace wc;
 extern "C" {
 
 int wc_test_gemm_override(int config, int rows_mode) {
-  WC_CHECK_ARG(config >= -1 && config < 16 && rows_mode >= 0 && rows_mode <= 3,
+  WC_CHECK_ARG(config >= -1 && config < 16 && rows_mode >= 0 && rows_mode <= 4,
                "wc_test_gemm_override: config %d, rows_mode %d", config, rows_mode);
   if (!test_hooks_enabled())
     return fail(WC_ERR_UNSUPPORTED, "wc_test_gemm_override: test hooks are off (set WINOCONV_TEST_HOOKS=1 before the first call)");

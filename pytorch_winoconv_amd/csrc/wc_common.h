@@ -131,8 +131,10 @@ bool gemm_persistent_fits(int T, int P, int Cp, int K, int dtype);
 int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, void* stream);
 // The same product on tiles of 512 x 128 fed by LDS-DMA (gemm_rows_dma.hip): runs of 2 to 5 pieces
 bool gemm_rows_dma_fits(SharedShift sh, int P, int Cp, int K, int dtype);
+// ... with a tile's results written out during the first steps of the workgroup's next tile: tiles of enough steps
+bool gemm_rows_dma_deferred_fits(SharedShift sh, int P, int Cp, int ldm);
 int gemm_rows_dma(const void* V, const void* U, void* M, int T, int P, int Cp, SharedShift sh, int K, int ldm, int dtype,
-                  void* stream);
+                  bool deferred, void* stream);
 
 // Input transform of single-piece 2-D plans at stride 1 that reads channel-first x (input_transform_2d_nchw.hip):
 // whether the plan is in its range, and the launch.

@@ -3,7 +3,7 @@ is transformed along depth and height only, over the pixel columns of the padded
 tile row), the three width taps lie side by side along the reduction of the shifted batched GEMM (one run of three
 pieces, each one row of V further), and M too holds 16 elements per column: half of what F(2,3)^3 reads and writes.
 The library takes the path by size; forced here (wc_test_gemm_override(12, .)) so that small shapes reach it, with each
-of the three kernels of the shifted product (rows_mode 0, 2, 3).  Nothing the reference does (its 3-D path is F(2,3)^3
+of the kernels of the shifted product (rows_mode 0, 2, 3, 4).  Nothing the reference does (its 3-D path is F(2,3)^3
 through three kernels: src/base_conv_launchers.cu); the convolution itself pins it."""
 import pytest
 import torch
@@ -18,6 +18,7 @@ CASES = [
     # x shape, K, pad
     ((2, 32, 6, 10, 12), 8, 1), ((1, 5, 4, 7, 9), 6, 1), ((2, 64, 5, 9, 8), 40, (0, 1, 1)), ((1, 128, 8, 12, 12), 128, 1),
     ((3, 16, 3, 3, 3), 8, 1), ((1, 40, 7, 11, 6), 33, (1, 0, 1)), ((2, 8, 9, 14, 15), 16, 0), ((1, 136, 4, 6, 6), 24, 1),
+    ((2, 128, 8, 40, 40), 136, 1),       # more 512-row tiles than workgroups
 ]
 DISC = {torch.float16: "fp16", torch.bfloat16: "bf16"}
 
@@ -27,7 +28,7 @@ def _rel(a, r):
     return float((a.double().cpu() - r).abs().max() / r.abs().max().clamp_min(1e-30))
 
 
-@pytest.mark.parametrize("rows_mode", [0, 2, 3])
+@pytest.mark.parametrize("rows_mode", [0, 2, 3, 4])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", CASES)
 def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case, rows_mode, gemm_override, host_layer):
@@ -52,7 +53,7 @@ def test_folded_product_against_fp64_and_the_three_kernel_path(dev, dtype, case,
     assert ycf.is_contiguous() and torch.equal(ycf, y1)
 
 
-@pytest.mark.parametrize("rows_mode", [0, 2, 3])
+@pytest.mark.parametrize("rows_mode", [0, 2, 3, 4])
 @pytest.mark.parametrize("case", [c for c in CASES if c[0][1] <= 64])
 def test_folded_product_is_exact_on_small_integers(dev, case, rows_mode, gemm_override):
     """x in -3..3, taps multiples of 8 (G of F(2,3) halves per axis): every U, V and product is an integer and the sums

@@ -140,6 +140,10 @@ DMA_CASES = [
     ((1, 64, 45, 45), (256, 64, 3, 3), 1, 2),
     # more tiles than workgroups: a workgroup walks over two or three tiles of its XCD's range
     ((2, 32, 160, 160), (136, 32, 5, 5), 2, 3), ((1, 32, 200, 190), (128, 32, 7, 7), 3, 2),
+    # tiles of enough steps for the write-out that rides on the next tile (runs of 2, 3 and 4 pieces), on more tiles
+    # than workgroups
+    ((1, 96, 80, 80), (64, 96, 5, 5), 2, 3), ((2, 96, 160, 160), (136, 96, 5, 5), 2, 3), ((2, 64, 200, 190), (128, 64, 7, 7), 3, 3),
+    ((2, 64, 150, 150), (128, 64, 7, 7), 3, 2),
 ]
 
 
@@ -162,6 +166,9 @@ def test_dma_fed_tile_per_run_equals_the_register_staged_one(dev, dtype, case, g
     gemm_override(rows_mode=3)
     y3 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, m, stacked=2)
     assert torch.equal(y2, y3)
+    gemm_override(rows_mode=4)          # ... with the write-out of a tile riding on the next one, where the tiles have the steps
+    y4 = engine.conv_forward(x.to(dev), w.to(dev), b.to(dev), 1, pad, m, stacked=2)
+    assert torch.equal(y2, y4)
     tol = {2: (3e-3, 2e-2), 3: (1e-2, 5e-2)}[m]             # F(3,3) evaluates at 2 as well: 3.1e-3 in fp16, 2.6e-2 in bf16
     assert _rel(y3, ref) <= tol[dtype == torch.bfloat16]
 
