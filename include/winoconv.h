@@ -144,7 +144,9 @@ const char* wc_last_error(void);
  * pieces, else as 1): 3 with every tile written out when it is done, 4 with the write-out riding on
  * the workgroup's next tile wherever the tiles have the steps for that (what the choice by size takes).
  * config 10: wc_batched_gemm on persistent 256 x 256 tiles wherever that kernel runs (16-bit types, K a
- * multiple of 256, reductions of 96 and more).
+ * multiple of 256, reductions of 96 and more), every tile written out when it is done; config 13: the
+ * same with most of a tile's write-out riding on the workgroup's next tile (reductions of 160 and more;
+ * what the choice by size takes).
  * config 11 / 12: 3-D F(2,3)^3 plans in 16-bit types never / always take the width axis inside the product
  * (transforms along depth and height only, the three width taps along the reduction; by size otherwise).
  * config 8 / 9: the one-kernel F(2x2,3x3) path with workgroups of 64 / 32 output channels whatever

@@ -890,16 +890,22 @@ extern "C" int wc_batched_gemm(const void* V, const void* U, void* M, int T_, in
   WC_CHECK_ARG(ldm >= K && ldm % 8 == 0, "wc_batched_gemm: row stride %d (needs >= K, multiple of 8)", ldm);
   WC_CHECK_ARG(dtype == WC_F16 || dtype == WC_F32 || dtype == WC_BF16, "wc_batched_gemm: dtype %d", dtype);
   // Persistent 256 x 256 tiles (gemm_persistent.hip) where whole layers measured faster with them than with every
-  // tile below (fp16, N = 64: 512 -> 512 channels at 28 x 28 0.148 ms against 0.154, 512 -> 256 at 56 x 56 0.349 against
-  // 0.375): reductions of 512 and more channels over at least three and a half rounds of tiles, the last round mostly
-  // full.  At 256 channels the product alone is 10 % faster on operands that come from HBM, but not behind an input
-  // transform that has just written them (0.234 ms either way at the 256-channel 56 x 56 layer), and smaller problems
-  // lose.  wc_test_gemm_override(10, .) takes the kernel wherever it runs.
+  // tile below.  With most of a tile's write-out riding on the workgroup's next tile (reductions of 160 channels and
+  // more): from one and a half rounds of tiles on, the last round mostly full - fp16 N = 64, ms per layer against the
+  // tiles below: 256 -> 256 channels at 56 x 56 0.218 | 0.233 (F(2,3): 0.369 | 0.396), at 28 x 28 0.065 | 0.067, 256 -> 512 at
+  // 28 x 28 0.100 | 0.107, 512 -> 512 at 28 x 28 0.143 | 0.147, 512 -> 256 at 56 x 56 0.338 | 0.346, N = 32 192 -> 256 at 56 x 56
+  // 0.104 | 0.108; equal at 252 tiles (N = 32 at 28 x 28, N = 8 at 56 x 56), behind below that (N = 64 at 14 x 14
+  // 0.034 | 0.033).  Without that (batches of 2 GB and more): reductions of 512 and more channels over at least three
+  // and a half rounds.  wc_test_gemm_override(10, .) takes the kernel wherever it runs with every tile written out when
+  // it is done, (13, .) with the write-out riding on the next tile wherever that fits.
   if (gemm_persistent_fits(T_, P, Cp, K, dtype)) {
     const int force = test_gemm_config();
     const long long tiles = (long long)ceil_div(P, 256) * (K / 256) * T_, rounds = ceil_div_ll(tiles, kCus);
-    const bool by_size = Cp >= 512 && tiles >= 896 && tiles * 100 >= rounds * kCus * 85;
-    if (force == 10 || (force < 0 && by_size)) return gemm_persistent(V, U, M, T_, P, Cp, K, ldm, dtype, stream);
+    const bool last_round_full = tiles * 100 >= rounds * kCus * 85;
+    const bool rides = gemm_persistent_deferred_fits(P, Cp, K, ldm);
+    const bool by_size = last_round_full && (rides ? tiles >= 384 : (Cp >= 512 && tiles >= 896));
+    if (force == 10 || force == 13 || (force < 0 && by_size))
+      return gemm_persistent(V, U, M, T_, P, Cp, K, ldm, dtype, force != 10 && rides, stream);
   }
   GemmConfig c = dispatch_dtype(dtype, [&](auto t) { return choose<decltype(t)>(T_, P, K, Cp); });
   GemmArgs g;

@@ -13,6 +13,9 @@
 // Measured against gemm_kernel's choice (fp16, three rotating operand sets): T = 36, P = 12544, C = K = 256 125 us
 // against 140; P = 3136, C = K = 512 94 against 111.
 #include "wc_common.h"
+#ifndef WC_HELD_ROWS
+#define WC_HELD_ROWS 3
+#endif
 
 namespace wc {
 
@@ -227,6 +230,228 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_kernel(PersistentArgs 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+
+// ---- the same kernel with a tile's results written out during the first four steps of the workgroup's next tile.
+// With one workgroup per CU nobody multiplies, and nothing is requested, while a tile is written out; here a finished
+// tile is only packed to 16 bits (128 registers) and each of the next tile's first four steps stages one 32-row block of
+// it before its first sub-step and stores it (eight instructions per wavefront) between its sub-steps.  The stores are
+// buffer stores: rows beyond the problem are dropped by the bounds check of the tile's descriptor, and before the first
+// tile an empty descriptor drops everything, so every wavefront issues every one of them and they are counted with the
+// loads: behind a step that carried stores, eight more operations may be in flight.  To make room for the 128 registers
+// the operand addresses are a scalar base and a lane offset computed when a load is queued (batches of V, U and M below
+// 2 GB).  A tile needs at least five steps.  Same order of additions: bit-identical results.
+__device__ __forceinline__ void dma16s(const void* base, unsigned offset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(offset), "s"(base), "s"(lds_addr) : "memory");
+}
+
+template <typename T, int HR>
+__global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(PersistentArgs g) {
+  static_assert(HR >= 1 && HR <= WM, "row blocks of a tile that ride on the next one");
+  using MF = MfmaP<T>;
+  using Frag = typename MF::Frag;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+
+  const int xcd = blockIdx.x % kXcds, in_xcd = blockIdx.x / kXcds, per_xcd_wg = g.n_wg / kXcds;
+  const int t_begin = (int)((long long)g.n_tiles * xcd / kXcds), t_end = (int)((long long)g.n_tiles * (xcd + 1) / kXcds);
+  const int first = t_begin + in_xcd;
+  if (first >= t_end) return;
+  const int my_tiles = (t_end - first + per_xcd_wg - 1) / per_xcd_wg;
+  const int NK = g.Cp / 32;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wp = wave >> 1, wk = wave & 1;
+  const int l32 = lane & 31, lhi = lane >> 5;
+
+  // ---- issue side: the tile being multiplied (0) and the one after it (1) as scalars
+  const T* tV[2]; const T* tU[2];
+  int tp0[2], tk0[2];
+  auto set_tile = [&](int w, int tile) {
+    const int kt_ = tile % g.tiles_k, pt = (tile / g.tiles_k) % g.tiles_p, t = tile / (g.tiles_k * g.tiles_p);
+    tV[w] = static_cast<const T*>(g.V) + (long long)t * g.sV;
+    tU[w] = static_cast<const T*>(g.U) + (long long)t * g.sU;
+    tp0[w] = pt * BM; tk0[w] = kt_ * BN;
+  };
+  const unsigned chunk16 = ((lane & 3) ^ swizzle(lane >> 2)) * 16;       // (rows 16 n + r share r's swizzle)
+  const unsigned row_bytes = (unsigned)g.Cp * 2;
+  // the loads of reduction step `ks` of tile set `next` into the ring stage of global step `gstep`; share q of 8
+  auto issue_part = [&](bool next, int ks, int gstep, int q) {
+    const unsigned dst = lds_base + (gstep & (S - 1)) * STAGE + wave * 1024 + q * 4096;
+    int rl = lane >> 2;
+    asm volatile("" : "+v"(rl));          // computed here, load by load: eight offsets per tile would otherwise be kept in registers
+    const int row = (wave + 4 * q) * 16 + rl;
+    const int w = next ? 1 : 0;
+    if (q < VG) dma16s(tV[w], (unsigned)min(tp0[w] + row, g.P - 1) * row_bytes + chunk16 + (unsigned)ks * 64, dst);
+    else dma16s(tU[w], (unsigned)min(tk0[w] + row - BM, g.K - 1) * row_bytes + chunk16 + (unsigned)ks * 64, dst);
+  };
+
+  int voff[2], uoff[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    const int phys = ((kk * 2 + lhi) ^ swizzle(l32)) * 16;
+    voff[kk] = (wp * WM * 32 + l32) * 64 + phys;
+    uoff[kk] = (BM + wk * WN * 32 + l32) * 64 + phys;
+  }
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  Frag vf[2][WM], uf[2][WN];
+
+  auto substep = [&](int b, int rstage, int rkk, bool which, int iks, int gstep, int half) {
+    const unsigned char* st = lds + rstage * STAGE;
+#pragma unroll
+    for (int q = 0; q < WM; ++q) {
+      vf[b ^ 1][q] = *reinterpret_cast<const Frag*>(st + voff[rkk] + q * 2048);
+      uf[b ^ 1][q] = *reinterpret_cast<const Frag*>(st + uoff[rkk] + q * 2048);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) acc[q][j] = MF::run(uf[b][j], vf[b][q], acc[q][j]);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, WN - 2, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_part(which, iks, gstep, half * WM + q);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- the previous tile's results (packed) and where they go.  Accumulator (i, j), register 4 q + e holds output
+  // channel 32 j + 8 q + 4 lhi + e of tile row 32 i + l32; held[i][j][2 q], [2 q + 1] are its registers 4 q .. 4 q + 3 as
+  // 16-bit pairs.  A 32-row block (i, 0 .. 3) is staged as rows of 256 bytes, chunks swizzled by the row.
+  constexpr int CPR = WN * 4, RPI = 64 / CPR;
+  uint32_t held[HR][WN][8];
+  __amdgpu_buffer_rsrc_t hdesc = __builtin_amdgcn_make_buffer_rsrc(g.M, 0, 0, 0x00020000);   // no tile yet: every store is dropped
+  unsigned held_off = 0;
+  // (staging addresses are computed where they are used, behind an opaque copy of the lane id: sixteen write and eight
+  // read addresses per lane would otherwise be kept in registers across the reduction loops)
+  auto stage_rows = [&](auto ic_) {
+    constexpr int i = decltype(ic_)::value;
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    int le = lane;
+    asm volatile("" : "+v"(le));
+    const int z = le & (CPR - 1);
+    unsigned char* row = lds + S * STAGE + wave * (32 * WN * 64) + (le & 31) * (CPR * 16) + (le >> 5) * 8;
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<u32x2*>(row + (((4 * j + q) ^ z) * 16)) = u32x2{held[i][j][2 * q], held[i][j][2 * q + 1]};
+  };
+  auto store_rows = [&](auto ic_) {
+    constexpr int i = decltype(ic_)::value;
+    int le = lane;
+    asm volatile("" : "+v"(le));
+    const int c = le % CPR, r = le / CPR;
+    const unsigned char* blk = lds + S * STAGE + wave * (32 * WN * 64);
+#pragma unroll
+    for (int r0 = 0; r0 < 32; r0 += RPI) {
+      const int row = r0 + r;
+      const u32x4 val = *reinterpret_cast<const u32x4*>(blk + row * (CPR * 16) + ((c ^ (row & (CPR - 1))) * 16));
+      __builtin_amdgcn_raw_buffer_store_b128(val, hdesc, held_off + (unsigned)((i * 32 + r0) * g.ldm * 2), 0, 0);
+      if ((r0 / RPI) % 2 == 1) __builtin_amdgcn_sched_barrier(0);       // two at a time: few registers live
+    }
+  };
+
+  // ---- steps 0 .. 2 of the first tile in flight
+  set_tile(0, first);
+  set_tile(1, my_tiles > 1 ? first + per_xcd_wg : first);
+  int gstep = 0;
+#pragma unroll
+  for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+    for (int q = 0; q < GPW; ++q) issue_part(false, s3, s3, q);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(2 * GPW) : "memory");
+  {
+    const unsigned char* st = lds;
+#pragma unroll
+    for (int q = 0; q < WM; ++q) {
+      vf[0][q] = *reinterpret_cast<const Frag*>(st + voff[0] + q * 2048);
+      uf[0][q] = *reinterpret_cast<const Frag*>(st + uoff[0] + q * 2048);
+    }
+  }
+
+  constexpr int IM = (WM - HR) * 2 * WM;      // stores per wavefront that follow a tile at once (row blocks HR .. 3)
+  constexpr int SU = HR + 1 > 2 ? HR + 1 : 2; // steps whose counts differ from the plain one
+#pragma unroll 1
+  for (int ti = 0; ti < my_tiles; ++ti) {
+    // steps 0 .. HR - 1 carry the previous tile's row blocks 0 .. HR - 1 (eight stores each, between the sub-steps).
+    // Stage gstep + 1 has landed everywhere and nobody reads stage gstep - 1 any more when all that is in flight is what
+    // was queued behind the last load of step gstep - 2: the loads of step gstep - 1, the stores it carried, and behind
+    // the first two steps of a tile the stores that followed the tile before at once.
+    static_for<0, SU>([&](auto kc) {
+      constexpr int ks = decltype(kc)::value;
+      constexpr int carried = ks >= 1 && ks - 1 < HR ? 2 * WM : 0;
+      if (ti > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(GPW + carried + (ks < 2 ? IM : 0)) : "memory");
+      else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(GPW + carried) : "memory");
+      const bool which = ks + 3 >= NK;
+      const int iks = ks + 3 < NK ? ks + 3 : ks + 3 - NK;
+      const int cs = gstep & (S - 1), ns = (gstep + 1) & (S - 1);
+      if constexpr (ks < HR) { stage_rows(ic<(ks < HR ? ks : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
+      substep(0, cs, 1, which, iks, gstep + 3, 0);
+      if constexpr (ks < HR) { store_rows(ic<(ks < HR ? ks : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
+      substep(1, ns, 0, which, iks, gstep + 3, 1);
+      ++gstep;
+    });
+#pragma unroll 1
+    for (int ks = SU; ks < NK; ++ks) {
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(GPW) : "memory");
+      const bool which = ks + 3 >= NK;
+      const int iks = ks + 3 < NK ? ks + 3 : ks + 3 - NK;
+      const int cs = gstep & (S - 1), ns = (gstep + 1) & (S - 1);
+      substep(0, cs, 1, which, iks, gstep + 3, 0);
+      substep(1, ns, 0, which, iks, gstep + 3, 1);
+      ++gstep;
+    }
+    // ---- the tile's results: row blocks 0 .. HR - 1 into `held`, the others out at once
+    {
+      const int tile = first + ti * per_xcd_wg;
+      const int kt_ = tile % g.tiles_k, pt = (tile / g.tiles_k) % g.tiles_p, t = tile / (g.tiles_k * g.tiles_p);
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      hdesc = __builtin_amdgcn_make_buffer_rsrc(static_cast<T*>(g.M) + (long long)t * g.sM, 0, (int)((unsigned)g.P * (unsigned)g.ldm * 2u), 0x00020000);
+      held_off = (unsigned)(((pt * BM + wp * WM * 32 + lane_e / CPR) * g.ldm + kt_ * BN + wk * WN * 32 + (lane_e % CPR) * 8) * 2);
+      static_for<0, WM>([&](auto ic_) {
+        constexpr int i = decltype(ic_)::value;
+        unsigned char* row = lds + S * STAGE + wave * (32 * WN * 64) + (lane_e & 31) * (CPR * 16) + (lane_e >> 5) * 8;
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          asm volatile("" : "+a"(acc[i][j]));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            Pack<T, 4> o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * q + e]);
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            const u32x2 w2 = __builtin_bit_cast(u32x2, o);
+            if constexpr (i < HR) { held[i < HR ? i : 0][j][2 * q] = w2[0]; held[i < HR ? i : 0][j][2 * q + 1] = w2[1]; }
+            else *reinterpret_cast<u32x2*>(row + (((4 * j + q) ^ (lane_e & (CPR - 1))) * 16)) = w2;
+          }
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (i >= HR) store_rows(ic_);
+      });
+    }
+    // the tile after the next one
+    tV[0] = tV[1]; tU[0] = tU[1]; tp0[0] = tp0[1]; tk0[0] = tk0[1];
+    set_tile(1, ti + 2 < my_tiles ? first + (ti + 2) * per_xcd_wg : first + (my_tiles - 1) * per_xcd_wg);
+  }
+  // the last tile's results: nothing to ride on
+  static_for<0, HR>([&](auto kc) {
+    stage_rows(kc);
+    store_rows(kc);
+  });
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 }  // namespace
 
 // 16-bit types, output channels in whole tiles, at least three reduction steps, and enough tiles for two rounds
@@ -235,8 +460,15 @@ bool gemm_persistent_fits(int T_, int P, int Cp, int K, int dtype) {
          (long long)ceil_div(P, BM) * (K / BN) * T_ < (1ll << 30);
 }
 
-int gemm_persistent(const void* V, const void* U, void* M, int T_, int P, int Cp, int K, int ldm, int dtype, void* stream) {
+constexpr int kHeldRows = WC_HELD_ROWS;
+// ... with the write-out riding on the next tile: at least five steps per tile, batches below 2 GB
+bool gemm_persistent_deferred_fits(int P, int Cp, int K, int ldm) {
+  return Cp >= 160 && (long long)P * Cp * 2 < (1ll << 31) && (long long)K * Cp * 2 < (1ll << 31) && (long long)P * ldm * 2 < (1ll << 31);
+}
+
+int gemm_persistent(const void* V, const void* U, void* M, int T_, int P, int Cp, int K, int ldm, int dtype, bool deferred, void* stream) {
   WC_CHECK_ARG(gemm_persistent_fits(T_, P, Cp, K, dtype), "gemm_persistent: P %d, K %d, reduction %d", P, K, Cp);
+  WC_CHECK_ARG(!deferred || gemm_persistent_deferred_fits(P, Cp, K, ldm), "gemm_persistent: reduction %d too short for the deferred write-out", Cp);
   PersistentArgs a;
   a.V = V; a.U = U; a.M = M;
   a.P = P; a.K = K; a.Cp = Cp; a.ldm = ldm;
@@ -244,7 +476,8 @@ int gemm_persistent(const void* V, const void* U, void* M, int T_, int P, int Cp
   a.tiles_p = ceil_div(P, BM); a.tiles_k = K / BN;
   a.n_tiles = a.tiles_p * a.tiles_k * T_;
   a.n_wg = kCus;
-  auto fn = dtype == WC_F16 ? &gemm_persistent_kernel<half_t> : &gemm_persistent_kernel<bf16_t>;
+  auto fn = deferred ? (dtype == WC_F16 ? &gemm_persistent_deferred_kernel<half_t, kHeldRows> : &gemm_persistent_deferred_kernel<bf16_t, kHeldRows>)
+                     : (dtype == WC_F16 ? &gemm_persistent_kernel<half_t> : &gemm_persistent_kernel<bf16_t>);
   if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), kPersistentLds)) return rc;
   hipLaunchKernelGGL(fn, dim3((unsigned)a.n_wg), dim3(256), kPersistentLds, as_stream(stream), a);
   WC_CHECK_LAUNCH("gemm_persistent_kernel");

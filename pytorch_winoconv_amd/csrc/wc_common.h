@@ -128,7 +128,8 @@ int fold_filter_w(const void* U, void* Uw, int K, int Cp, int dtype, void* strea
 int output_transform_columns(const wc_conv_desc* d, const void* M, const void* bias, int n_images, void* y, void* stream);
 // wc_batched_gemm on persistent 256 x 256 tiles fed by LDS-DMA (gemm_persistent.hip): 16-bit types, K a multiple of 256
 bool gemm_persistent_fits(int T, int P, int Cp, int K, int dtype);
-int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, void* stream);
+bool gemm_persistent_deferred_fits(int P, int Cp, int K, int ldm);      // ... with a tile written out during the next tile's first steps
+int gemm_persistent(const void* V, const void* U, void* M, int T, int P, int Cp, int K, int ldm, int dtype, bool deferred, void* stream);
 // The same product on tiles of 512 x 128 fed by LDS-DMA (gemm_rows_dma.hip): runs of 2 to 5 pieces
 bool gemm_rows_dma_fits(SharedShift sh, int P, int Cp, int K, int dtype);
 // ... with a tile's results written out during the first steps of the workgroup's next tile: tiles of enough steps

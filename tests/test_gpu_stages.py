@@ -210,16 +210,21 @@ def test_batched_gemm_long_reduction_tile(dev, dtype, gemm_override):
     (1, 31, 512, 256),         # fewer tiles than workgroups: most return at once
     (60, 1300, 96, 256),       # 360 tiles: some workgroups walk over two
     (41, 1100, 128, 512),      # 410 tiles, ranges of 51 and 52 tiles per XCD
+    (60, 1300, 256, 256),      # reductions long enough for the write-out that rides on the next tile: 360 tiles
+    (36, 3000, 160, 512),      # ... five steps (the fewest for it), 864 tiles
+    (9, 2100, 512, 256),
 ])
-def test_batched_gemm_persistent_tiles(dev, dtype, T, P, C, K, gemm_override):
+@pytest.mark.parametrize("form", [10, 13])
+def test_batched_gemm_persistent_tiles(dev, dtype, T, P, C, K, form, gemm_override):
     """The persistent 256 x 256 kernel (chosen by size for long reductions over many tiles; forced here through
     wc_test_gemm_override so that small shapes reach it): against an fp64 product, and bit for bit against the
     256 x 128 tile of gemm_kernel, which adds the same products in the same order.  Rows of M beyond K are not
-    written by either."""
+    written by either.  Form 13: most of a tile's results ride on the workgroup's next tile (reductions of 160
+    channels and more; as 10 below that)."""
     g = torch.Generator().manual_seed(6)
     V = torch.randn(T, P, C, generator=g).to(dtype).to(dev)
     U = (torch.randn(T, K, C, generator=g) / C ** 0.5).to(dtype).to(dev)
-    gemm_override(config=10)
+    gemm_override(config=form)
     M = engine.batched_gemm(V, U)
     want = torch.bmm(V.double(), U.double().transpose(1, 2))
     assert _rel(M[:, :, :K], want) <= (2e-3 if dtype == torch.float16 else 8e-3)
