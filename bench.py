@@ -33,10 +33,10 @@ sys.path.insert(0, ROOT)
 N, C, K, H, W, R, PAD, M_TILE = 64, 256, 256, 56, 56, 3, 1, 4
 MFMA_FP16_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 matrix peak
 HBM_PEAK_GB_S = 8000.0              # MI355X published HBM3E bandwidth
-# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (116806 KiB, x2.00 by the copy
+# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (127139 KiB, x2.00 by the copy
 # probe) + WRITE_SIZE (225792 KiB, x1.00); runs and scale factors are recorded in
-# profiles/mfma_utilisation_shipped_gemms.md.
-GEMM_HBM_TRAFFIC_BYTES = int((116806 * 2.0 + 225792 * 1.0) * 1024)
+# profiles/conv3x3_f16_n64_c256_56x56_all_kernels.md.
+GEMM_HBM_TRAFFIC_BYTES = int((127139 * 2.0 + 225792 * 1.0) * 1024)
 
 
 def synthetic(n):
@@ -650,7 +650,7 @@ def main():
                                "transform included in every step"},
         "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": MFMA_FP16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP16_PEAK_TFLOPS,
-                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "wc::gemm_kernel (batched_gemm)",
+                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "wc::gemm_persistent_deferred_kernel (wc_batched_gemm)",
                      "flops_per_launch": gemm_flops, "avg_us": stage_us["batched_gemm"],
                      "hbm_view": {"bytes_per_launch": gemm_bytes, "achieved": gemm_gb_s, "peak": HBM_PEAK_GB_S,
                                   "unit": "GB/s", "frac": gemm_gb_s / HBM_PEAK_GB_S}},
