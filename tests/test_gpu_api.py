@@ -226,6 +226,7 @@ def test_winoconv3d_module(dev):
     ((48, 32, 3, 3), 2, 0, None),        # thin 16-bit 3x3 layer: filter transform + the one fused kernel
     ((48, 32, 5, 5), 2, 2, (-1, 3)),     # ... the shifted product on its persistent LDS-DMA kernel
     ((256, 96, 3, 3), 4, 0, (10, 1)),    # the batched GEMM on its persistent LDS-DMA kernel
+    ((256, 160, 3, 3), 4, 0, (13, 1)),   # ... with a tile's write-out riding on the next tile (buffer stores)
 ])
 def test_forward_is_capturable_in_a_hip_graph(dev, ws, m, stacked, force, gemm_override):
     """The library allocates nothing, never synchronises and takes its stream from the caller, so a
