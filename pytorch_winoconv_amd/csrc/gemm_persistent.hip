@@ -233,13 +233,15 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_kernel(PersistentArgs 
 
 // ---- the same kernel with a tile's results written out during the first four steps of the workgroup's next tile.
 // With one workgroup per CU nobody multiplies, and nothing is requested, while a tile is written out; here a finished
-// tile is only packed to 16 bits (128 registers) and each of the next tile's first four steps stages one 32-row block of
-// it before its first sub-step and stores it (eight instructions per wavefront) between its sub-steps.  The stores are
+// tile is only packed to 16 bits - three of its four 32-row blocks into 96 registers, the fourth into the wavefront's
+// staging area - and each of the next tile's first four steps stores one block (eight instructions per wavefront)
+// between its sub-steps: first the one that waits in the staging area, then the others, each staged before the first
+// sub-step of its step.  The stores are
 // buffer stores: rows beyond the problem are dropped by the bounds check of the tile's descriptor, and before the first
 // tile an empty descriptor drops everything, so every wavefront issues every one of them and they are counted with the
-// loads: behind a step that carried stores, eight more operations may be in flight.  To make room for the 128 registers
+// loads: behind a step that carried stores, eight more operations may be in flight.  To make room for the registers
 // the operand addresses are a scalar base and a lane offset computed when a load is queued (batches of V, U and M below
-// 2 GB).  A tile needs at least five steps.  Same order of additions: bit-identical results.
+// 2 GB; all four blocks in registers spill).  A tile needs at least five steps.  Same order of additions: bit-identical results.
 __device__ __forceinline__ void dma16s(const void* base, unsigned offset, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(offset), "s"(base), "s"(lds_addr) : "memory");
 }
@@ -377,25 +379,26 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(Persis
     }
   }
 
-  constexpr int IM = (WM - HR) * 2 * WM;      // stores per wavefront that follow a tile at once (row blocks HR .. 3)
-  constexpr int SU = HR + 1 > 2 ? HR + 1 : 2; // steps whose counts differ from the plain one
+  constexpr int IM = (WM - HR - 1) * 2 * WM;  // stores per wavefront that follow a tile at once (row blocks HR + 1 .. 3)
+  constexpr int SU = HR + 2;                  // steps whose counts differ from the plain one
 #pragma unroll 1
   for (int ti = 0; ti < my_tiles; ++ti) {
-    // steps 0 .. HR - 1 carry the previous tile's row blocks 0 .. HR - 1 (eight stores each, between the sub-steps).
-    // Stage gstep + 1 has landed everywhere and nobody reads stage gstep - 1 any more when all that is in flight is what
-    // was queued behind the last load of step gstep - 2: the loads of step gstep - 1, the stores it carried, and behind
-    // the first two steps of a tile the stores that followed the tile before at once.
+    // Step 0 carries the previous tile's row block HR, which has waited in the staging area; steps 1 .. HR carry its row
+    // blocks 0 .. HR - 1 from the registers (eight stores each, between the sub-steps).  Stage gstep + 1 has landed
+    // everywhere and nobody reads stage gstep - 1 any more when all that is in flight is what was queued behind the last
+    // load of step gstep - 2: the loads of step gstep - 1, the stores it carried, and behind the first two steps of a
+    // tile the stores that followed the tile before at once.
     static_for<0, SU>([&](auto kc) {
       constexpr int ks = decltype(kc)::value;
-      constexpr int carried = ks >= 1 && ks - 1 < HR ? 2 * WM : 0;
+      constexpr int carried = ks >= 1 && ks - 1 <= HR ? 2 * WM : 0;
       if (ti > 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(GPW + carried + (ks < 2 ? IM : 0)) : "memory");
       else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(GPW + carried) : "memory");
       const bool which = ks + 3 >= NK;
       const int iks = ks + 3 < NK ? ks + 3 : ks + 3 - NK;
       const int cs = gstep & (S - 1), ns = (gstep + 1) & (S - 1);
-      if constexpr (ks < HR) { stage_rows(ic<(ks < HR ? ks : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
+      if constexpr (ks >= 1 && ks <= HR) { stage_rows(ic<(ks >= 1 && ks <= HR ? ks - 1 : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
       substep(0, cs, 1, which, iks, gstep + 3, 0);
-      if constexpr (ks < HR) { store_rows(ic<(ks < HR ? ks : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
+      if constexpr (ks <= HR) { store_rows(ic<(ks == 0 ? HR : ks <= HR ? ks - 1 : 0)>{}); __builtin_amdgcn_sched_barrier(0); }
       substep(1, ns, 0, which, iks, gstep + 3, 1);
       ++gstep;
     });
@@ -409,7 +412,8 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(Persis
       substep(1, ns, 0, which, iks, gstep + 3, 1);
       ++gstep;
     }
-    // ---- the tile's results: row blocks 0 .. HR - 1 into `held`, the others out at once
+    // ---- the tile's results: row blocks 0 .. HR - 1 into `held`, the others through the staging area - the last ones
+    // out at once, row block HR left there for step 0 of the next tile
     {
       const int tile = first + ti * per_xcd_wg;
       const int kt_ = tile % g.tiles_k, pt = (tile / g.tiles_k) % g.tiles_p, t = tile / (g.tiles_k * g.tiles_p);
@@ -417,8 +421,9 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(Persis
       asm volatile("" : "+v"(lane_e));
       hdesc = __builtin_amdgcn_make_buffer_rsrc(static_cast<T*>(g.M) + (long long)t * g.sM, 0, (int)((unsigned)g.P * (unsigned)g.ldm * 2u), 0x00020000);
       held_off = (unsigned)(((pt * BM + wp * WM * 32 + lane_e / CPR) * g.ldm + kt_ * BN + wk * WN * 32 + (lane_e % CPR) * 8) * 2);
-      static_for<0, WM>([&](auto ic_) {
-        constexpr int i = decltype(ic_)::value;
+      // (descending: the block that stays in the staging area is written there last)
+      static_for<0, WM>([&](auto rc) {
+        constexpr int i = WM - 1 - decltype(rc)::value;
         unsigned char* row = lds + S * STAGE + wave * (32 * WN * 64) + (lane_e & 31) * (CPR * 16) + (lane_e >> 5) * 8;
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
@@ -437,7 +442,7 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(Persis
           for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
           __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (i >= HR) store_rows(ic_);
+        if constexpr (i > HR) store_rows(ic<i>{});
       });
     }
     // the tile after the next one
@@ -445,6 +450,7 @@ __global__ __launch_bounds__(256, 1) void gemm_persistent_deferred_kernel(Persis
     set_tile(1, ti + 2 < my_tiles ? first + (ti + 2) * per_xcd_wg : first + (my_tiles - 1) * per_xcd_wg);
   }
   // the last tile's results: nothing to ride on
+  if constexpr (HR < WM) store_rows(ic<(HR < WM ? HR : 0)>{});
   static_for<0, HR>([&](auto kc) {
     stage_rows(kc);
     store_rows(kc);
