@@ -13,9 +13,6 @@
 // Measured against gemm_kernel's choice (fp16, three rotating operand sets): T = 36, P = 12544, C = K = 256 125 us
 // against 140; P = 3136, C = K = 512 94 against 111.
 #include "wc_common.h"
-#ifndef WC_HELD_ROWS
-#define WC_HELD_ROWS 3
-#endif
 
 namespace wc {
 
@@ -466,7 +463,7 @@ bool gemm_persistent_fits(int T_, int P, int Cp, int K, int dtype) {
          (long long)ceil_div(P, BM) * (K / BN) * T_ < (1ll << 30);
 }
 
-constexpr int kHeldRows = WC_HELD_ROWS;
+constexpr int kHeldRows = 3;      // row blocks of a tile kept in registers (four spill)
 // ... with the write-out riding on the next tile: at least five steps per tile, batches below 2 GB
 bool gemm_persistent_deferred_fits(int P, int Cp, int K, int ldm) {
   return Cp >= 160 && (long long)P * Cp * 2 < (1ll << 31) && (long long)K * Cp * 2 < (1ll << 31) && (long long)P * ldm * 2 < (1ll << 31);
