@@ -634,16 +634,24 @@ static GemmConfig choose(int T_, int P, int K, int Cp) {
   }
   if (sizeof(T) == 4 || Cp <= 64) return Configs<T>::get(n_auto - 1);
   // Long reductions over many output channels: the 128 x 256 tile of eight wavefronts reads V
-  // once per 256 channels (measured 3-13 % faster than any four-wavefront tile for Cp >= 512).
+  // once per 256 channels (measured 3-13 % faster than any four-wavefront tile for Cp >= 512 from four rounds of
+  // tiles on; at 576 tiles - N = 64, 512 -> 512 channels at 14 x 14 - the 128 x 128 tile is 6 % ahead, 0.055 against
+  // 0.059 ms per layer).
   if constexpr (sizeof(T) == 2) {
-    if (Cp >= 512 && K >= 256 && (long long)ceil_div(P, 128) * ceil_div(K, 256) * T_ >= 512) return Configs<T>::get(5);
+    if (Cp >= 512 && K >= 256 && (long long)ceil_div(P, 128) * ceil_div(K, 256) * T_ >= 1024) return Configs<T>::get(5);
   }
   GemmConfig best = Configs<T>::get(n_auto - 1);
   for (int i = 0; i < n_auto; ++i) {
     GemmConfig c = Configs<T>::get(i);
     if (c.bn > 64 && c.bn / 2 >= K) continue;                 // half of the tile would be padding
     const long long blocks = (long long)ceil_div(P, c.bm) * ceil_div(K, c.bn) * T_;
-    if (blocks >= 512 || i == n_auto - 1) { best = c; break; }
+    // The 256 x 128 tile runs two workgroups per CU: 512 are resident at once.  It is the best tile when it fills
+    // that once (fp16 N = 64, F(4,3): 384 -> 384 channels at 14 x 14, 432 tiles, 0.040 ms per layer against 0.044 for the
+    // next best; 128 -> 128 and 256 -> 128 at 28 x 28, 468 tiles, 0.036 | 0.038 and 0.046 | 0.048) and the worst when a few
+    // tiles are left for a second round (512 -> 512 at 14 x 14, 576 tiles: 0.062 against 0.055 on 128 x 128; N = 32
+    // 256 -> 384 at 28 x 28, 756 tiles: 0.052 | 0.050); from two full rounds on the tail no longer decides.
+    const bool ok = i == 0 ? (blocks >= 1024 || (blocks >= 400 && blocks <= 512)) : blocks >= 512;
+    if (ok || i == n_auto - 1) { best = c; break; }
   }
   return best;
 }
