@@ -103,3 +103,20 @@ def test_the_library_folds_by_size(dev, gemm_override):
     ref = F.conv3d(x[:1].double(), w.double(), None, padding=1)
     assert _rel(y[:1], ref) <= 2e-3
     assert _rel(y[:1, :, :2], ow.dwm_conv(x[:1, :, :3], w, None, 1, 1, 2, "fp16")[:, :, :2]) <= 2e-3
+
+
+@pytest.mark.parametrize("chunk", [1, 2])
+def test_folded_path_in_chunks_of_images(dev, chunk, gemm_override):
+    """Batches cut into passes of `chunk` images (the last one partial) give what one pass gives, bit for bit: V and M of
+    a pass are laid out by the images it holds."""
+    g = torch.Generator().manual_seed(35)
+    xs, K = (5, 64, 6, 12, 20), 72
+    x = torch.randn(*xs, generator=g).half().to(dev)
+    w = (torch.randn(K, xs[1], 3, 3, 3, generator=g) * (2.0 / (27 * xs[1])) ** 0.5).half().to(dev)
+    b = torch.randn(K, generator=g).half().to(dev)
+    gemm_override(config=12)
+    whole = engine.conv_forward(x, w, b, 1, 1, 2)
+    parts = engine.conv_forward(x, w, b, 1, 1, 2, chunk_images=chunk)
+    assert torch.equal(whole, parts)
+    ref = F.conv3d(x.double().cpu(), w.double().cpu(), b.double().cpu(), padding=1)
+    assert _rel(parts, ref) <= 2e-3
